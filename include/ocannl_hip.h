@@ -1,0 +1,138 @@
+/* ocannl_hip.h -- C ABI of the MI355X (gfx950) arrayjit backend for OCANNL.
+ *
+ * This is the surface an OCaml `Hip_backend : Backend_impl.Lowered_backend` binds through ctypes;
+ * it replaces what the CUDA backend gets from the external `cudajit` package plus the CUDA
+ * backend's own compile/link/launch code.  Every entry point cites the reference interface it
+ * stands behind (paths relative to the OCANNL tree).
+ *
+ * Conventions
+ *   - every function returns 0 on success or a negative OCANNL_HIP_E_* code; the message for the
+ *     calling thread's last failure is ocannl_hip_last_error().  The OCaml stub maps
+ *     E_USER -> Utils.User_error, E_INVALID -> Invalid_argument, the rest -> Failure
+ *     (arrayjit/lib/cuda_backend.ml:1017-1035 uses exactly this split).
+ *   - one FIFO stream per device (arrayjit/lib/backend_intf.ml:262-265); every call makes its
+ *     device current first (cuda_backend.ml:56 `set_ctx`).
+ *   - buffers are named by (pool_id, byte offset): Backend_intf.buffer_loc
+ *     (arrayjit/lib/backend_intf.ml:7-16); the pool_id -> base table is private to the library
+ *     (cuda_backend.ml:60-94).
+ *   - host memory passed to from_host/to_host is caller-owned and must stay valid until the
+ *     caller's next ocannl_hip_await on that device (arrayjit/lib/context.ml:338-343,389).
+ *   - all calls come from one host thread at a time.
+ */
+#ifndef OCANNL_HIP_H
+#define OCANNL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OCANNL_HIP_OK 0
+#define OCANNL_HIP_E_USER (-1)     /* Utils.User_error: bad static index, unsupported precision ... */
+#define OCANNL_HIP_E_INVALID (-2)  /* Invalid_argument: misuse of the interface, malformed IR      */
+#define OCANNL_HIP_E_RUNTIME (-3)  /* Failure: HIP / hiprtc error                                  */
+
+typedef struct ocannl_hip_device ocannl_hip_device;    /* (dev, runner) of one ordinal            */
+typedef struct ocannl_hip_event ocannl_hip_event;      /* Lowered_backend.event                   */
+typedef struct ocannl_hip_code ocannl_hip_code;        /* Lowered_backend.code / code_batch       */
+typedef struct ocannl_hip_routine ocannl_hip_routine;  /* the linked launch closure (Task.t work) */
+
+/* Backend_intf.buffer_loc for one tensor node (backend_intf.ml:7-18: ctx_buffers entries). */
+typedef struct {
+  int32_t node_id;
+  int32_t pool_id;
+  uint64_t offset;   /* bytes */
+} ocannl_hip_node_loc;
+
+/* Kparam description (Backend_intf.kparam_source, backend_intf.ml:41-57). */
+typedef struct {
+  int32_t kind;        /* 0 = Kparam_ptr, 1 = Static_idx, 2 = Merge_buffer */
+  int32_t id;          /* node id or static symbol                       */
+  int64_t size_bytes;  /* Kparam_ptr: padded node size; Static_idx: range or -1 */
+} ocannl_hip_kparam;
+
+/* One device kernel of a compiled routine, for measurement and debugging. */
+typedef struct {
+  int32_t kind;            /* 0 = generated pointwise/reduction kernel, 1 = fill, 2 = MFMA contraction */
+  int32_t coop_lanes;      /* lanes cooperating on one output (generated reduction kernels)          */
+  double flops;            /* algorithmic: 2 * product of all loop extents for a contraction         */
+  double bytes;            /* algorithmic: distinct elements read once + written once, in bytes      */
+  int64_t m, n, k, batch;  /* contraction shape after symbol classification (0 otherwise)            */
+  char name[96];
+} ocannl_hip_kernel_info;
+
+const char* ocannl_hip_last_error(void);
+
+/* ---- devices: Backend_device_common (backend_intf.ml:206-266) ------------------------------- */
+/* Cu.init + lazy per-device set-up (cuda_backend.ml:113-118,215-238). Idempotent. */
+int ocannl_hip_init(void);
+int ocannl_hip_num_devices(int* count);                                  /* num_devices, :258    */
+int ocannl_hip_get_device(int ordinal, ocannl_hip_device** dev);         /* get_device, :257     */
+int ocannl_hip_get_name(ocannl_hip_device* dev, char* buf, size_t cap);  /* Device.get_name, :204 */
+int ocannl_hip_static_properties(char* buf, size_t cap);   /* static_properties sexp, :231; cuda_backend.ml:1092-1112 */
+int ocannl_hip_get_used_memory(ocannl_hip_device* dev, uint64_t* bytes); /* get_used_memory, :239 */
+int ocannl_hip_get_debug_info(ocannl_hip_device* dev, char* buf, size_t cap); /* get_debug_info, :244 */
+int ocannl_hip_await(ocannl_hip_device* dev);                            /* await, :247          */
+int ocannl_hip_is_idle(ocannl_hip_device* dev, int* idle);               /* is_idle, :254        */
+
+/* ---- events (backend_intf.ml:221-251; cuda_backend.ml:108-111) ------------------------------- */
+int ocannl_hip_all_work(ocannl_hip_device* dev, ocannl_hip_event** ev);  /* all_work             */
+int ocannl_hip_sync(ocannl_hip_event* ev);                               /* sync                 */
+int ocannl_hip_is_done(ocannl_hip_event* ev, int* done);                 /* is_done              */
+int ocannl_hip_will_wait_for(ocannl_hip_device* dev, ocannl_hip_event* ev); /* will_wait_for     */
+void ocannl_hip_event_free(ocannl_hip_event* ev);
+
+/* ---- Slab_alloc (backend_intf.ml:22-37; cuda_backend.ml:60-94) ------------------------------- */
+/* Allocating an existing pool_id frees the old slab first (merge-buffer regrowth, :71-76). */
+int ocannl_hip_alloc_pool(ocannl_hip_device* dev, int pool_id, uint64_t size_in_bytes, uint64_t alignment);
+int ocannl_hip_free_pool(ocannl_hip_device* dev, int pool_id);
+int ocannl_hip_memset_zero(ocannl_hip_device* dev, int pool_id, uint64_t offset, uint64_t size_in_bytes);
+
+/* ---- copies: No_buffer_retrieval_or_syncing (arrayjit/lib/backend_impl.ml:292-314) ----------- */
+/* Asynchronous on the device stream (cuda_backend.ml:267-287). */
+int ocannl_hip_from_host(ocannl_hip_device* dst, int pool_id, uint64_t offset, const void* src, uint64_t bytes);
+int ocannl_hip_to_host(ocannl_hip_device* src, int pool_id, uint64_t offset, void* dst, uint64_t bytes);
+/* Same-device or peer copy (cuda_backend.ml:289-314); dst_pool_id < 0 means "into the merge buffer of dst",
+   which is (re)grown to `bytes` as pool 0 (cuda_backend.ml:130-134). */
+int ocannl_hip_device_to_device(ocannl_hip_device* dst, int dst_pool_id, uint64_t dst_offset,
+                                ocannl_hip_device* src, int src_pool_id, uint64_t src_offset, uint64_t bytes);
+
+/* ---- compile / link / run (backend_impl.ml:347-367) ------------------------------------------ */
+/* Lowered_backend.compile / compile_batch: `llir` is the serialised Low_level.optimized of one or
+   more routines (name, static indices, node table, statement tree).  Splits each routine into
+   kernels, maps large `+*` contractions to the MFMA kernels, generates HIP for the rest and
+   compiles it with hiprtc for gfx950.  Needs no GPU. */
+int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** code);
+/* Same, with "key=value;..." options: mfma=0|1, coop=0|1, min_mfma_flops=<n>. */
+int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, ocannl_hip_code** code);
+void ocannl_hip_code_free(ocannl_hip_code* code);
+int ocannl_hip_code_num_routines(ocannl_hip_code* code, int* n);
+int ocannl_hip_code_routine_name(ocannl_hip_code* code, int index, char* buf, size_t cap);
+/* The kparam list of routine `index` (c_syntax.ml:1046-1084): pass params=NULL to query the count. */
+int ocannl_hip_code_kparams(ocannl_hip_code* code, int index, ocannl_hip_kparam* params, int cap, int* count);
+/* Generated HIP source (the `.hip` dump under output_debug_files_in_build_directory). */
+int ocannl_hip_code_source(ocannl_hip_code* code, char* buf, size_t cap, size_t* needed);
+int ocannl_hip_code_num_kernels(ocannl_hip_code* code, int index, int* n);
+int ocannl_hip_code_kernel_info(ocannl_hip_code* code, int index, int kernel, ocannl_hip_kernel_info* info);
+
+/* Lowered_backend.link (backend_impl.ml:355; cuda_backend.ml:983-1066): loads the module on `dev`,
+   resolves every Kparam_ptr through `locs` (the resulting context's ctx_buffers), allocates the
+   routine-private scratch for `Local` nodes.  Missing nodes raise E_USER (cc_backend.ml:411-415). */
+int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, const ocannl_hip_node_loc* locs,
+                    int n_locs, ocannl_hip_routine** routine);
+void ocannl_hip_routine_free(ocannl_hip_routine* routine);
+/* lowered_bindings: the `int ref` behind a Static_idx (arrayjit/lib/indexing.ml:60-93). */
+int ocannl_hip_routine_set_static(ocannl_hip_routine* routine, int symbol, int64_t value);
+/* Task.run of the launch closure (cuda_backend.ml:991-1044): range-checks static indices
+   (E_USER on failure, :1015-1030), then enqueues the routine's kernels on the device stream. */
+int ocannl_hip_routine_run(ocannl_hip_routine* routine);
+/* Same, bracketing every kernel with HIP events on the device stream; synchronises and writes the
+   per-kernel milliseconds (cap >= number of kernels).  For measurement only. */
+int ocannl_hip_routine_run_timed(ocannl_hip_routine* routine, float* kernel_ms, int cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OCANNL_HIP_H */

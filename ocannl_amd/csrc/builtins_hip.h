@@ -1,0 +1,184 @@
+// Device-side scalar builtins prepended to every generated HIP module.
+//
+// Same names and results as the C builtins OCANNL's generated code calls
+// (arrayjit/lib/builtins.c:11-743; call sites are produced from arrayjit/lib/ops.ml:579-876), so
+// that a routine computes on gfx950 what the `cc` backend computes on the host:
+//   bf16 <-> float  builtins.c:611-627      fp8 (E5M2) <-> float  builtins.c:646-743
+//   half            native _Float16 (builtins.c:12-21 "HAS_NATIVE_FLOAT16" arm)
+//   threefry4x32    builtins.c:156-329      uint4x32 -> uniform   builtins.c:345-528
+//   X -> uint4x32   builtins.c:531-606
+// This text is compiled by hiprtc (which predeclares the fixed-width integer types and the math
+// library) and, for a syntax check, by hipcc via builtins_check.hip.
+#pragma once
+
+#ifdef __HIPCC_RTC__
+typedef unsigned int uint32_t;
+typedef int int32_t;
+typedef unsigned long long uint64_t;
+typedef long long int64_t;
+#endif
+
+#define OCN_DEV __device__ __forceinline__
+#ifndef INFINITY
+#define INFINITY __builtin_huge_valf()
+#endif
+#ifndef NAN
+#define NAN __builtin_nanf("")
+#endif
+
+#define HALF_T _Float16
+#define HALF_TO_FP(x) (x)
+#define FP_TO_HALF(x) (x)
+#define HALF_TO_FLOAT(x) ((float)(x))
+#define FLOAT_TO_HALF(x) ((_Float16)(x))
+
+struct uint4x32_t { uint32_t v[4]; };
+struct float4_t { float v[4]; };
+struct double2_t { double v[2]; };
+struct int32x4_t { int32_t v[4]; };
+struct uint32x4_t { uint32_t v[4]; };
+struct int64x2_t { long long v[2]; };
+struct uint64x2_t { uint64_t v[2]; };
+struct int8x16_t { signed char v[16]; };
+struct uint16x8_t { unsigned short v[8]; };
+struct uint8x16_t { unsigned char v[16]; };
+struct half8_t { _Float16 v[8]; };
+
+// ---- bf16 / fp8 ---------------------------------------------------------------------------------
+OCN_DEV float bfloat16_to_single(unsigned short b) { return __uint_as_float(((uint32_t)b) << 16); }
+// Round to nearest even through an integer add; NaN inputs are not special-cased, exactly as on the
+// host (builtins.c:620-627).
+OCN_DEV unsigned short single_to_bfloat16(float f) {
+  const uint32_t w = __float_as_uint(f);
+  return (unsigned short)((w + 0x7FFFu + ((w >> 16) & 1u)) >> 16);
+}
+OCN_DEV float fp8_to_single(unsigned char v) {
+  if (v == 0) return 0.0f;
+  const uint32_t sgn = v >> 7, e = (v >> 2) & 31u, m = v & 3u;
+  float r;
+  if (e == 31u) { if (m) return NAN; r = INFINITY; }
+  else if (e == 0u) r = ldexpf((float)m * 0.25f, -14);
+  else r = (1.0f + (float)m * 0.25f) * ldexpf(1.0f, (int)e - 15);
+  return sgn ? -r : r;
+}
+OCN_DEV unsigned char single_to_fp8(float f) {
+  if (f == 0.0f) return 0;
+  const uint32_t sgn = f < 0 ? 1u : 0u;
+  f = fabsf(f);
+  if (isinf(f)) return (unsigned char)((sgn << 7) | 0x7Cu);
+  if (isnan(f)) return (unsigned char)((sgn << 7) | 0x7Fu);
+  int ev;
+  const float mf = frexpf(f, &ev);
+  const int e = ev + 14;
+  if (e < 0) return (unsigned char)(sgn << 7);
+  if (e > 30) return (unsigned char)((sgn << 7) | 0x7Cu);
+  uint32_t mb;
+  if (e == 0) {
+    mb = (uint32_t)(f * 16384.0f * 4.0f + 0.5f);
+    if (mb > 3u) mb = 3u;
+    return (unsigned char)((sgn << 7) | mb);
+  }
+  mb = (uint32_t)((mf - 0.5f) * 4.0f + 0.5f);
+  if (mb > 3u) mb = 3u;
+  return (unsigned char)((sgn << 7) | (((uint32_t)e & 31u) << 2) | mb);
+}
+
+// ---- threefry4x32 -------------------------------------------------------------------------------
+OCN_DEV uint32_t ocn_rotl32(uint32_t x, uint32_t n) { return (x << n) | (x >> (32u - n)); }
+#define OCN_TF_MIX(x, ra, rb)                                   \
+  x.v[0] += x.v[1]; x.v[1] = ocn_rotl32(x.v[1], ra) ^ x.v[0];   \
+  x.v[2] += x.v[3]; x.v[3] = ocn_rotl32(x.v[3], rb) ^ x.v[2];   \
+  { const uint32_t t_ = x.v[1]; x.v[1] = x.v[3]; x.v[3] = t_; }
+// The reference's "round" = two mix+swap layers; rotation sets alternate (builtins.c:163-196).
+#define OCN_TF_EVEN(x) OCN_TF_MIX(x, 13u, 15u) OCN_TF_MIX(x, 26u, 6u)
+#define OCN_TF_ODD(x) OCN_TF_MIX(x, 17u, 29u) OCN_TF_MIX(x, 16u, 24u)
+OCN_DEV uint4x32_t arrayjit_threefry4x32_light(uint4x32_t key, uint4x32_t ctr) {
+  const uint32_t k4 = key.v[0] ^ key.v[1] ^ key.v[2] ^ key.v[3] ^ 0x1BD11BDAu;
+  uint4x32_t x;
+  for (int i = 0; i < 4; ++i) x.v[i] = ctr.v[i] + key.v[i];
+  OCN_TF_EVEN(x) OCN_TF_ODD(x)
+  x.v[0] += key.v[1]; x.v[1] += key.v[2]; x.v[2] += key.v[3]; x.v[3] += k4 + 1u;
+  return x;
+}
+OCN_DEV uint4x32_t arrayjit_threefry4x32_crypto(uint4x32_t key, uint4x32_t ctr) {
+  uint32_t ks[5];
+  ks[4] = 0x1BD11BDAu;
+  uint4x32_t x;
+  for (int i = 0; i < 4; ++i) { ks[i] = key.v[i]; ks[4] ^= key.v[i]; x.v[i] = ctr.v[i] + key.v[i]; }
+#pragma unroll
+  for (uint32_t g = 1; g <= 5; ++g) {   // 20 "rounds", key injection after every 4 (builtins.c:199-281)
+    OCN_TF_EVEN(x) OCN_TF_ODD(x) OCN_TF_EVEN(x) OCN_TF_ODD(x)
+    for (uint32_t i = 0; i < 4; ++i) x.v[i] += ks[(g + i) % 5u];
+    x.v[3] += g;
+  }
+  return x;
+}
+OCN_DEV uint4x32_t arrayjit_threefry4x32(uint4x32_t key, uint4x32_t ctr) {
+  return arrayjit_threefry4x32_light(key, ctr);
+}
+
+// ---- uint4x32 -> uniform ------------------------------------------------------------------------
+OCN_DEV float uint32_to_single_uniform(uint32_t x) { return (float)(x >> 8) * 5.9604644775390625e-08f; }
+OCN_DEV double uint32_to_double_uniform(uint32_t x) { return (double)x * 2.3283064365386963e-10; }
+OCN_DEV uint64_t ocn_lo64(uint4x32_t x) { return ((uint64_t)x.v[1] << 32) | x.v[0]; }
+OCN_DEV uint64_t ocn_hi64(uint4x32_t x) { return ((uint64_t)x.v[3] << 32) | x.v[2]; }
+OCN_DEV unsigned short ocn_bf16_guard_round(float f) {   // builtins.c:397-406
+  const uint32_t b = __float_as_uint(f);
+  unsigned short r = (unsigned short)(b >> 16);
+  if ((b & 0x8000u) && ((b & 0x7FFFu) || (r & 1u))) r++;
+  return r;
+}
+OCN_DEV float ocn_u16_unit(uint32_t w, int hi) { return (float)((w >> (hi ? 16 : 0)) & 0xFFFFu) * 1.52587890625e-05f; }
+OCN_DEV float uint4x32_to_single_uniform(uint4x32_t x) { return uint32_to_single_uniform(x.v[0]); }
+OCN_DEV double uint4x32_to_double_uniform(uint4x32_t x) { return (double)ocn_lo64(x) * 5.421010862427522e-20; }
+OCN_DEV int uint4x32_to_int32_uniform(uint4x32_t x) { return (int)x.v[0]; }
+OCN_DEV long long uint4x32_to_int64_uniform(uint4x32_t x) { return (long long)ocn_lo64(x); }
+OCN_DEV uint32_t uint4x32_to_uint32_uniform(uint4x32_t x) { return x.v[0]; }
+OCN_DEV uint64_t uint4x32_to_uint64_uniform(uint4x32_t x) { return ocn_lo64(x); }
+OCN_DEV signed char uint4x32_to_byte_uniform(uint4x32_t x) { return (signed char)(x.v[0] & 0xFFu); }
+OCN_DEV unsigned short uint4x32_to_uint16_uniform(uint4x32_t x) { return (unsigned short)(x.v[0] & 0xFFFFu); }
+OCN_DEV unsigned short uint4x32_to_bfloat16_uniform(uint4x32_t x) { return ocn_bf16_guard_round(uint32_to_single_uniform(x.v[0])); }
+OCN_DEV _Float16 uint4x32_to_half_uniform(uint4x32_t x) { return (_Float16)ocn_u16_unit(x.v[0], 0); }
+OCN_DEV unsigned char uint4x32_to_fp8_uniform(uint4x32_t x) { return (unsigned char)(x.v[0] & 0xFFu); }
+
+OCN_DEV float4_t uint4x32_to_single_uniform_vec(uint4x32_t x) {
+  float4_t r; for (int i = 0; i < 4; ++i) r.v[i] = uint32_to_single_uniform(x.v[i]); return r; }
+OCN_DEV double2_t uint4x32_to_double_uniform_vec(uint4x32_t x) {
+  double2_t r; r.v[0] = (double)ocn_lo64(x) * 5.421010862427522e-20; r.v[1] = (double)ocn_hi64(x) * 5.421010862427522e-20; return r; }
+OCN_DEV int32x4_t uint4x32_to_int32_uniform_vec(uint4x32_t x) {
+  int32x4_t r; for (int i = 0; i < 4; ++i) r.v[i] = (int32_t)x.v[i]; return r; }
+OCN_DEV uint32x4_t uint4x32_to_uint32_uniform_vec(uint4x32_t x) {
+  uint32x4_t r; for (int i = 0; i < 4; ++i) r.v[i] = x.v[i]; return r; }
+OCN_DEV int64x2_t uint4x32_to_int64_uniform_vec(uint4x32_t x) {
+  int64x2_t r; r.v[0] = (long long)ocn_lo64(x); r.v[1] = (long long)ocn_hi64(x); return r; }
+OCN_DEV uint64x2_t uint4x32_to_uint64_uniform_vec(uint4x32_t x) {
+  uint64x2_t r; r.v[0] = ocn_lo64(x); r.v[1] = ocn_hi64(x); return r; }
+OCN_DEV int8x16_t uint4x32_to_byte_uniform_vec(uint4x32_t x) {
+  int8x16_t r; for (int i = 0; i < 16; ++i) r.v[i] = (signed char)((x.v[i >> 2] >> (8 * (i & 3))) & 0xFFu); return r; }
+OCN_DEV uint16x8_t uint4x32_to_uint16_uniform_vec(uint4x32_t x) {
+  uint16x8_t r; for (int i = 0; i < 8; ++i) r.v[i] = (unsigned short)((x.v[i >> 1] >> (16 * (i & 1))) & 0xFFFFu); return r; }
+OCN_DEV uint16x8_t uint4x32_to_bfloat16_uniform_vec(uint4x32_t x) {
+  uint16x8_t r; for (int i = 0; i < 8; ++i) r.v[i] = ocn_bf16_guard_round(ocn_u16_unit(x.v[i >> 1], i & 1)); return r; }
+OCN_DEV half8_t uint4x32_to_half_uniform_vec(uint4x32_t x) {
+  half8_t r; for (int i = 0; i < 8; ++i) r.v[i] = (_Float16)ocn_u16_unit(x.v[i >> 1], i & 1); return r; }
+OCN_DEV uint8x16_t uint4x32_to_fp8_uniform_vec(uint4x32_t x) {
+  uint8x16_t r; for (int i = 0; i < 16; ++i) r.v[i] = (unsigned char)((x.v[i >> 2] >> (8 * (i & 3))) & 0xFFu); return r; }
+
+// ---- X -> uint4x32 ------------------------------------------------------------------------------
+OCN_DEV uint4x32_t ocn_u4(uint32_t a, uint32_t b, uint32_t c, uint32_t d) { uint4x32_t r; r.v[0] = a; r.v[1] = b; r.v[2] = c; r.v[3] = d; return r; }
+// 32-bit counters are spread over all four words (builtins.c:545-576)
+OCN_DEV uint4x32_t uint32_to_uint4x32(uint32_t x) { return ocn_u4(x, x ^ 0x9E3779B9u, x ^ 0x6C078965u, x ^ ocn_rotl32(x, 16u)); }
+OCN_DEV uint4x32_t int32_to_uint4x32(int x) { return uint32_to_uint4x32((uint32_t)x); }
+OCN_DEV uint4x32_t uint64_to_uint4x32(uint64_t x) { return ocn_u4((uint32_t)x, (uint32_t)(x >> 32), 0u, 0u); }
+OCN_DEV uint4x32_t int64_to_uint4x32(long long x) { return uint64_to_uint4x32((uint64_t)x); }
+OCN_DEV uint4x32_t single_to_uint4x32(float x) { return ocn_u4(__float_as_uint(x), 0u, 0u, 0u); }
+OCN_DEV uint4x32_t double_to_uint4x32(double x) { return uint64_to_uint4x32((uint64_t)__double_as_longlong(x)); }
+OCN_DEV uint4x32_t byte_to_uint4x32(unsigned char x) { return ocn_u4(x, 0u, 0u, 0u); }
+OCN_DEV uint4x32_t uint16_to_uint4x32(unsigned short x) { return ocn_u4(x, 0u, 0u, 0u); }
+OCN_DEV uint4x32_t bfloat16_to_uint4x32(unsigned short x) { return ocn_u4(x, 0u, 0u, 0u); }
+OCN_DEV uint4x32_t half_to_uint4x32(unsigned short x) { return ocn_u4(x, 0u, 0u, 0u); }
+OCN_DEV uint4x32_t fp8_to_uint4x32(unsigned char x) { return ocn_u4(x, 0u, 0u, 0u); }
+
+// ---- lane-group combine used by cooperative reductions ------------------------------------------
+OCN_DEV float ocn_xshfl(float v, int m) { return __shfl_xor(v, m, 64); }
+OCN_DEV double ocn_xshfl(double v, int m) { return __shfl_xor(v, m, 64); }

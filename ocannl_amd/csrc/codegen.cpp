@@ -1,0 +1,674 @@
+#include "codegen.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <functional>
+#include <set>
+#include <sstream>
+
+namespace ocannl {
+namespace {
+
+// ------------------------------------------------------------------------------------------------
+// syntax tables (arrayjit/lib/ops.ml)
+// ------------------------------------------------------------------------------------------------
+
+const char* c_typ(Prec p) {   // Ops.c_typ_of_prec, ops.ml:324-337 (HALF_T = _Float16 on device)
+  switch (p) {
+    case Prec::Byte: return "unsigned char";
+    case Prec::Uint16: return "unsigned short";
+    case Prec::Int32: return "int";
+    case Prec::Uint32: return "uint32_t";
+    case Prec::Int64: return "long long";
+    case Prec::Uint64: return "uint64_t";
+    case Prec::Uint4x32: return "uint4x32_t";
+    case Prec::Half: return "HALF_T";
+    case Prec::Bfloat16: return "unsigned short";
+    case Prec::Fp8: return "unsigned char";
+    case Prec::Single: return "float";
+    case Prec::Double: return "double";
+    case Prec::Void: return "void";
+  }
+  return "void";
+}
+
+std::string c_vec_typ(int length, Prec p) {   // Ops.c_vec_typ_of_prec, ops.ml:339-351
+  if (p == Prec::Single && length == 4) return "float4_t";
+  if (p == Prec::Double && length == 2) return "double2_t";
+  if (p == Prec::Int32 && length == 4) return "int32x4_t";
+  if (p == Prec::Uint32 && length == 4) return "uint32x4_t";
+  if (p == Prec::Int64 && length == 2) return "int64x2_t";
+  if (p == Prec::Uint64 && length == 2) return "uint64x2_t";
+  if ((p == Prec::Byte || p == Prec::Fp8) && length == 16) return "int8x16_t";
+  if ((p == Prec::Uint16 || p == Prec::Bfloat16) && length == 8) return "uint16x8_t";
+  if (p == Prec::Half && length == 8) return "half8_t";
+  if (length == 1) return c_typ(p);
+  throw InvalidArgument("vector type: invalid (precision, length) combination");
+}
+
+bool plain_int(Prec p) {
+  return p == Prec::Byte || p == Prec::Uint16 || p == Prec::Int32 || p == Prec::Uint32 ||
+         p == Prec::Int64 || p == Prec::Uint64;
+}
+bool dbl_or_intish(Prec p) { return p == Prec::Double || prec_is_intish(p); }
+
+using Pair = std::pair<std::string, std::string>;
+
+Pair convert_precision(Prec f, Prec t) {   // Ops.c_convert_precision, ops.ml:808-876
+  if (f == t) return {"", ""};
+  using P = Prec;
+  if (f == P::Bfloat16 && t == P::Single) return {"bfloat16_to_single(", ")"};
+  if (f == P::Single && t == P::Bfloat16) return {"single_to_bfloat16(", ")"};
+  if (f == P::Bfloat16 && t == P::Double) return {"(double)bfloat16_to_single(", ")"};
+  if (f == P::Double && t == P::Bfloat16) return {"single_to_bfloat16((float)", ")"};
+  if (f == P::Fp8 && t == P::Single) return {"fp8_to_single(", ")"};
+  if (f == P::Single && t == P::Fp8) return {"single_to_fp8(", ")"};
+  if (f == P::Fp8 && t == P::Double) return {"(double)fp8_to_single(", ")"};
+  if (f == P::Double && t == P::Fp8) return {"single_to_fp8((float)", ")"};
+  if (f == P::Bfloat16 && t == P::Half) return {"FLOAT_TO_HALF(bfloat16_to_single(", "))"};
+  if (f == P::Half && t == P::Bfloat16) return {"single_to_bfloat16(HALF_TO_FLOAT(", "))"};
+  if (f == P::Bfloat16 && plain_int(t)) return {std::string("(") + c_typ(t) + ")bfloat16_to_single(", ")"};
+  if (plain_int(f) && t == P::Bfloat16) return {"single_to_bfloat16((float)", ")"};
+  if (f == P::Fp8 && t == P::Half) return {"FLOAT_TO_HALF(fp8_to_single(", "))"};
+  if (f == P::Half && t == P::Fp8) return {"single_to_fp8(HALF_TO_FLOAT(", "))"};
+  if (f == P::Fp8 && plain_int(t)) return {std::string("(") + c_typ(t) + ")fp8_to_single(", ")"};
+  if (plain_int(f) && t == P::Fp8) return {"single_to_fp8((float)", ")"};
+  if (f == P::Bfloat16 && t == P::Fp8) return {"single_to_fp8(bfloat16_to_single(", "))"};
+  if (f == P::Fp8 && t == P::Bfloat16) return {"single_to_bfloat16(fp8_to_single(", "))"};
+  if (f == P::Half && t == P::Single) return {"HALF_TO_FLOAT(", ")"};
+  if (f == P::Single && t == P::Half) return {"FLOAT_TO_HALF(", ")"};
+  if (f == P::Half && t == P::Double) return {"(double)HALF_TO_FLOAT(", ")"};
+  if (f == P::Double && t == P::Half) return {"FLOAT_TO_HALF((float)", ")"};
+  if (f == P::Half && plain_int(t)) return {std::string("(") + c_typ(t) + ")HALF_TO_FLOAT(", ")"};
+  if (plain_int(f) && t == P::Half) return {"FLOAT_TO_HALF((float)", ")"};
+  if (f == P::Uint4x32) return {std::string("uint4x32_to_") + prec_string(t) + "(", ")"};
+  if (t == P::Uint4x32) return {std::string(prec_string(f)) + "_to_uint4x32(", ")"};
+  return {std::string("(") + c_typ(t) + ")(", ")"};
+}
+
+struct Syn3 { std::string p, i, s; };
+struct Syn4 { std::string p, i1, i2, s; };
+
+Syn3 binop_syntax(Prec prec, Binop op) {   // Ops.binop_c_syntax, ops.ml:579-630
+  const bool ii = prec_is_intish(prec);
+  switch (op) {
+    case Binop::Add: return {"(", " +", ")"};
+    case Binop::Sub: return {"(", " -", ")"};
+    case Binop::Mul: return {"(", " *", ")"};
+    case Binop::Div: return {"(", " /", ")"};
+    case Binop::Pow:
+      if (prec == Prec::Double) return {"pow(", ",", ")"};
+      if (ii) throw InvalidArgument("ToPowOf not supported for integer precisions");
+      return {"powf(", ",", ")"};
+    case Binop::ReluGate: return ii ? Syn3{"(", " > 0 ?", " : 0)"} : Syn3{"(", " > 0.0 ?", " : 0.0)"};
+    case Binop::Sat01Gate:
+      if (ii) return {"(abs(", " ) > 0 ? 0 : (", "))"};
+      if (prec == Prec::Single) return {"(fabsf(floorf(", ")) > 0.0 ? 0.0 : (", "))"};
+      return {"(fabs(floor(", ")) > 0.0 ? 0.0 : (", "))"};
+    case Binop::Max: return dbl_or_intish(prec) ? Syn3{"fmax(", ",", ")"} : Syn3{"fmaxf(", ",", ")"};
+    case Binop::Min: return dbl_or_intish(prec) ? Syn3{"fmin(", ",", ")"} : Syn3{"fminf(", ",", ")"};
+    case Binop::Mod: return {"(", " %", ")"};
+    case Binop::Lt: return {"(", " <", ")"};
+    case Binop::Eq: return {"(", " ==", ")"};
+    case Binop::Ne: return {"(", " !=", ")"};
+    case Binop::Or: return {"(", " ||", ")"};
+    case Binop::And: return {"(", " &&", ")"};
+    case Binop::ThreefryCrypto: return {"arrayjit_threefry4x32_crypto(", ",", ")"};
+    case Binop::ThreefryLight: return {"arrayjit_threefry4x32_light(", ",", ")"};
+    default: throw InvalidArgument("binop syntax: Arg1/Arg2 are not operators");
+  }
+}
+
+Pair unop_syntax(Prec prec, Unop op) {   // Ops.unop_c_syntax, ops.ml:688-782
+  const bool wide = dbl_or_intish(prec), ii = prec_is_intish(prec);
+  const std::string fmax = wide ? "fmax" : "fmaxf", fmin = wide ? "fmin" : "fminf";
+  auto libm = [&](const char* n) -> Pair { return {std::string(n) + (wide ? "(" : "f("), ")"}; };
+  switch (op) {
+    case Unop::Id: return {"", ""};
+    case Unop::Relu: return ii ? Pair{"fmax(0, ", ")"} : Pair{fmax + "(0.0, ", ")"};
+    case Unop::Sat01: return ii ? Pair{"fmax(0, fmin(1, ", "))"} : Pair{fmax + "(0.0, " + fmin + "(1.0, ", "))"};
+    case Unop::Exp: return libm("exp");
+    case Unop::Log: return libm("log");
+    case Unop::Exp2: return libm("exp2");
+    case Unop::Log2: return libm("log2");
+    case Unop::Sin: return libm("sin");
+    case Unop::Cos: return libm("cos");
+    case Unop::Sqrt: return libm("sqrt");
+    case Unop::Recip:
+      if (ii) throw InvalidArgument("Recip not supported for integer precisions");
+      return {"(1.0 / (", "))"};
+    case Unop::RecipSqrt:
+      if (ii) throw InvalidArgument("Recip_sqrt not supported for integer precisions");
+      return prec == Prec::Double ? Pair{"(1.0 / sqrt(", "))"} : Pair{"(1.0 / sqrtf(", "))"};
+    case Unop::Neg: return {"(-(", "))"};
+    case Unop::Trunc: return prec == Prec::Double ? Pair{"trunc(", ")"} : Pair{"truncf(", ")"};
+    case Unop::Tanh:
+      if (ii) throw InvalidArgument("Tanh_approx not supported for integer precisions");
+      return {"tanhf(", ")"};
+    case Unop::Not: return {"(", " == 0.0 ? 1.0 : 0.0)"};
+    case Unop::Uniform1:
+      if (prec == Prec::Uint4x32) throw InvalidArgument("Uint4x32_to_prec_uniform1 not supported for Uint4x32");
+      return {std::string("uint4x32_to_") + prec_string(prec) + "_uniform(", ")"};
+  }
+  return {"", ""};
+}
+
+Syn4 ternop_syntax(Prec prec, Ternop op) {   // Ops.ternop_c_syntax, ops.ml:793-806
+  switch (op) {
+    case Ternop::Where:
+      return prec_is_intish(prec) ? Syn4{"((", ") != 0 ? (", ") : (", "))"} : Syn4{"((", ") != 0.0 ? (", ") : (", "))"};
+    case Ternop::Fma: return dbl_or_intish(prec) ? Syn4{"fma(", ",", ",", ")"} : Syn4{"fmaf(", ",", ",", ")"};
+    case Ternop::Mul3: return {"((", ") * (", ") * (", "))"};
+  }
+  return {};
+}
+
+// cc_backend.ml:169-323: reduced precisions compute in float
+bool via_float(Prec p, std::string* to_f, std::string* from_f) {
+  if (p == Prec::Bfloat16) { *to_f = "bfloat16_to_single("; *from_f = "single_to_bfloat16("; return true; }
+  if (p == Prec::Half) { *to_f = "HALF_TO_FP("; *from_f = "FP_TO_HALF("; return true; }
+  if (p == Prec::Fp8) { *to_f = "fp8_to_single("; *from_f = "single_to_fp8("; return true; }
+  return false;
+}
+
+std::string emit_ternop(Prec prec, Ternop op, const std::string& a, const std::string& b, const std::string& c) {
+  std::string tf, ff;
+  if (via_float(prec, &tf, &ff)) {
+    Syn4 s = ternop_syntax(Prec::Single, op);
+    return ff + s.p + tf + a + ")" + s.i1 + " " + tf + b + ")" + s.i2 + " " + tf + c + ")" + s.s + ")";
+  }
+  Syn4 s = ternop_syntax(prec, op);
+  return s.p + a + s.i1 + " " + b + s.i2 + " " + c + s.s;
+}
+
+std::string emit_binop(Prec prec, Binop op, const std::string& a, const std::string& b) {
+  if (op == Binop::ThreefryCrypto || op == Binop::ThreefryLight) {
+    if (prec != Prec::Uint4x32) throw UserError("threefry4x32 on non-uint4x32 precision");
+    return std::string(op == Binop::ThreefryCrypto ? "arrayjit_threefry4x32_crypto(" : "arrayjit_threefry4x32_light(") +
+           a + ", " + b + ")";
+  }
+  std::string tf, ff;
+  if (via_float(prec, &tf, &ff)) {
+    Syn3 s = binop_syntax(Prec::Single, op);
+    return ff + s.p + tf + a + ")" + s.i + " " + tf + b + ")" + s.s + ")";
+  }
+  Syn3 s = binop_syntax(prec, op);
+  return s.p + a + s.i + " " + b + s.s;
+}
+
+std::string emit_unop(Prec prec, Unop op, const std::string& a) {
+  std::string tf, ff;
+  if (via_float(prec, &tf, &ff)) {
+    Pair s = unop_syntax(Prec::Single, op);
+    return ff + s.first + tf + a + ")" + s.second + ")";
+  }
+  Pair s = unop_syntax(prec, op);
+  return s.first + a + s.second;
+}
+
+std::string axis_str(const AxisIndex& a) {   // Doc_helpers.pp_axis_index, indexing.ml:454-476
+  if (a.kind == AxisIndex::Iter) return sym_ident(a.sym);
+  if (a.kind == AxisIndex::Fixed) return std::to_string(a.fixed);
+  std::string out;
+  for (auto& t : a.terms) {
+    if (!out.empty()) out += "+";
+    out += t.first == 1 ? sym_ident(t.second) : std::to_string(t.first) + "*" + sym_ident(t.second);
+  }
+  if (a.offset > 0) out += (out.empty() ? "" : "+") + std::to_string(a.offset);
+  else if (a.offset < 0) out += (out.empty() ? "" : "+") + ("-" + std::to_string(-a.offset));
+  return out.empty() ? "0" : out;
+}
+
+std::string offset_str(const Indices& idcs, const std::vector<int64_t>& dims, int dyn_axis = -1,
+                       const std::string& dyn = "") {   // pp_array_offset, c_syntax.ml:367-397
+  if (idcs.empty()) return "0";
+  auto part = [&](size_t i) { return (int)i == dyn_axis ? dyn : axis_str(idcs[i]); };
+  std::string doc = part(0);
+  for (size_t i = 1; i < idcs.size(); ++i) doc = "(" + doc + ") * " + std::to_string(dims[i]) + " + " + part(i);
+  return doc;
+}
+
+std::string const_str(double c) {
+  if (std::isinf(c)) return c > 0 ? "INFINITY" : "(-INFINITY)";
+  if (std::isnan(c)) return "NAN";
+  char buf[64];
+  std::snprintf(buf, sizeof buf, "%.16g", c);
+  return buf;
+}
+
+// low_level.ml:1998-2037
+bool reads_scope_before_set(const ScopeId& target, const Block& body) {
+  std::function<bool(const Scalar&)> sc_reads;
+  std::function<bool(const Block&)> blk_reads = [&](const Block& b) {
+    for (auto& s : b) {
+      if (s->kind == Stmt::For && blk_reads(s->body)) return true;
+      if ((s->kind == Stmt::Set || s->kind == Stmt::SetVec || s->kind == Stmt::SetLocal) && sc_reads(*s->value)) return true;
+    }
+    return false;
+  };
+  sc_reads = [&](const Scalar& s) -> bool {
+    switch (s.kind) {
+      case Scalar::GetLocal: return s.scope == target;
+      case Scalar::LocalScope: return blk_reads(s.body);
+      case Scalar::GetDyn: case Scalar::Un: return sc_reads(*s.a);
+      case Scalar::Bin: return sc_reads(*s.a) || sc_reads(*s.b);
+      case Scalar::Tern: return sc_reads(*s.a) || sc_reads(*s.b) || sc_reads(*s.c);
+      default: return false;
+    }
+  };
+  enum R { Read, Written, Neither };
+  std::function<R(const Block&)> scan = [&](const Block& b) -> R {
+    for (auto& s : b) {
+      R r = Neither;
+      switch (s->kind) {
+        case Stmt::Set: case Stmt::SetVec: r = sc_reads(*s->value) ? Read : Neither; break;
+        case Stmt::SetLocal: r = sc_reads(*s->value) ? Read : (s->scope == target ? Written : Neither); break;
+        case Stmt::For: { R in = scan(s->body); r = in == Written ? (s->from <= s->to ? Written : Neither) : in; break; }
+        default: break;
+      }
+      if (r != Neither) return r;
+    }
+    return Neither;
+  };
+  return scan(body) != Written;
+}
+
+// ------------------------------------------------------------------------------------------------
+// statement / scalar printer
+// ------------------------------------------------------------------------------------------------
+
+struct Printer {
+  const Routine& r;
+  std::set<int> used_nodes;
+  std::set<int> used_statics;
+  // when set, a read of exactly this (node, indices) prints as `self_name`
+  const Stmt* self_set = nullptr;
+  std::string self_name;
+  int fresh = 0;
+
+  explicit Printer(const Routine& rr) : r(rr) {}
+
+  std::string scope_name(const ScopeId& s) { return "v" + std::to_string(s.scope) + "_" + r.node(s.node).ident; }
+  void note_idx(const AxisIndex& a) {
+    if (a.kind == AxisIndex::Iter && r.is_static(a.sym)) used_statics.insert(a.sym);
+    if (a.kind == AxisIndex::Affine) for (auto& t : a.terms) if (r.is_static(t.second)) used_statics.insert(t.second);
+  }
+  void note(int node, const Indices& idcs) {
+    if (r.node(node).mode == Mode::Virtual)
+      throw InvalidArgument("hip backend: access to virtual node " + r.node(node).ident + " survived optimisation");
+    used_nodes.insert(node);
+    for (auto& a : idcs) note_idx(a);
+  }
+  std::string init_zero(Prec p) { Pair c = convert_precision(Prec::Int32, p); return " = " + c.first + "0" + c.second; }
+
+  struct Def { int scope; std::vector<std::string> lines; };
+
+  std::string scalar(Prec prec, const Scalar& s, const std::string& ind, std::vector<Def>& defs) {
+    switch (s.kind) {
+      case Scalar::LocalScope: {
+        const Prec sp = r.node(s.scope.node).prec;
+        Def d; d.scope = s.scope.scope;
+        d.lines.push_back(ind + c_typ(sp) + " " + scope_name(s.scope) +
+                          (reads_scope_before_set(s.scope, s.body) ? init_zero(sp) : "") + ";");
+        block(s.body, ind, d.lines);
+        defs.push_back(std::move(d));
+        Pair c = convert_precision(sp, prec);
+        return c.first + scope_name(s.scope) + c.second;
+      }
+      case Scalar::GetLocal: {
+        Pair c = convert_precision(r.node(s.scope.node).prec, prec);
+        return c.first + scope_name(s.scope) + c.second;
+      }
+      case Scalar::GetMerge: {
+        const Node& n = r.node(s.node);
+        for (auto& a : s.idcs) note_idx(a);
+        Pair c = convert_precision(n.prec, prec);
+        return c.first + "merge_buffer[" + offset_str(s.idcs, n.dims) + "]" + c.second;
+      }
+      case Scalar::Get: {
+        const Node& n = r.node(s.node);
+        Pair c = convert_precision(n.prec, prec);
+        if (self_set && s.node == self_set->node && s.idcs == self_set->idcs) return c.first + self_name + c.second;
+        note(s.node, s.idcs);
+        return c.first + n.ident + "[" + offset_str(s.idcs, n.dims) + "]" + c.second;
+      }
+      case Scalar::GetDyn: {
+        const Node& n = r.node(s.node);
+        note(s.node, s.idcs);
+        Pair c = convert_precision(n.prec, prec);
+        std::string dyn = std::string("((") + c_typ(Prec::Uint32) + ")(" + scalar(s.arg_prec, *s.a, ind, defs) + "))";
+        return c.first + n.ident + "[" + offset_str(s.idcs, n.dims, s.dyn_axis, dyn) + "]" + c.second;
+      }
+      case Scalar::Const: {
+        Pair c = convert_precision(Prec::Double, prec);
+        const std::string cs = const_str(s.cst);
+        if (c.first.empty() && s.cst < 0.0 && !std::isinf(s.cst)) return "(" + cs + ")" + c.second;
+        return c.first + cs + c.second;
+      }
+      case Scalar::Bits: {
+        Pair c = convert_precision(Prec::Int64, prec);
+        return c.first + std::to_string((long long)s.bits) + "LL" + c.second;
+      }
+      case Scalar::Index: {
+        note_idx(s.index);
+        Pair c = convert_precision(Prec::Uint32, prec);
+        return c.first + axis_str(s.index) + c.second;
+      }
+      case Scalar::Tern: {
+        // Where is heterogeneous: its condition keeps its own precision (c_syntax.ml:798-829)
+        std::string a = scalar(s.tern == Ternop::Where ? s.arg_prec : prec, *s.a, ind, defs);
+        std::string b = scalar(prec, *s.b, ind, defs);
+        std::string c = scalar(prec, *s.c, ind, defs);
+        return emit_ternop(prec, s.tern, a, b, c);
+      }
+      case Scalar::Bin: {
+        if (s.bin == Binop::Arg1) return scalar(prec, *s.a, ind, defs);
+        if (s.bin == Binop::Arg2) return scalar(prec, *s.b, ind, defs);
+        std::string a = scalar(prec, *s.a, ind, defs);
+        std::string b = scalar(prec, *s.b, ind, defs);
+        return emit_binop(prec, s.bin, a, b);
+      }
+      case Scalar::Un: {
+        std::string a = scalar(s.un == Unop::Uniform1 ? s.arg_prec : prec, *s.a, ind, defs);
+        return emit_unop(prec, s.un, a);
+      }
+    }
+    return "";
+  }
+
+  void with_defs(std::vector<Def>& defs, const std::vector<std::string>& lines, const std::string& ind,
+                 std::vector<std::string>& out) {
+    if (defs.empty()) { for (auto& l : lines) out.push_back(ind + l); return; }
+    std::stable_sort(defs.begin(), defs.end(), [](const Def& a, const Def& b) { return a.scope < b.scope; });
+    out.push_back(ind + "{");
+    int last = -1; bool first = true;
+    for (auto& d : defs) {
+      if (!first && d.scope == last) continue;   // c_syntax.ml:406-409 dedup by scope id
+      first = false; last = d.scope;
+      for (auto& l : d.lines) out.push_back(l);
+    }
+    for (auto& l : lines) out.push_back(ind + "  " + l);
+    out.push_back(ind + "}");
+  }
+
+  void stmt(const Stmt& c, const std::string& ind, std::vector<std::string>& out) {
+    switch (c.kind) {
+      case Stmt::Comment: out.push_back(ind + "/* " + c.text + " */"); break;
+      case Stmt::For: {
+        const std::string s = sym_ident(c.sym);
+        out.push_back(ind + "for (uint32_t " + s + " = " + std::to_string(c.from) + "; " + s + " <= " +
+                      std::to_string(c.to) + "; ++" + s + ") {");
+        block(c.body, ind + "  ", out);
+        out.push_back(ind + "}");
+        break;
+      }
+      case Stmt::ZeroOut: {
+        // a re-zero reached inside a kernel: plain serial loop over the node (c_syntax.ml:476-479)
+        const Node& n = r.node(c.node);
+        used_nodes.insert(c.node);
+        const std::string v = "z" + std::to_string(fresh++);
+        Pair cv = convert_precision(Prec::Double, n.prec);
+        out.push_back(ind + "for (uint32_t " + v + " = 0; " + v + " < " + std::to_string(n.num_elems()) + "; ++" + v +
+                      ") " + n.ident + "[" + v + "] = " + cv.first + "0" + cv.second + ";");
+        break;
+      }
+      case Stmt::Set: {
+        const Node& n = r.node(c.node);
+        note(c.node, c.idcs);
+        std::vector<Def> defs;
+        std::string v = scalar(n.prec, *c.value, ind + "  ", defs);
+        with_defs(defs, {n.ident + "[" + offset_str(c.idcs, n.dims) + "] = " + v + ";"}, ind, out);
+        break;
+      }
+      case Stmt::SetVec: {
+        const Node& n = r.node(c.node);
+        note(c.node, c.idcs);
+        std::vector<Def> defs;
+        std::string a = scalar(c.arg_prec, *c.value, ind + "  ", defs);
+        if (n.prec == Prec::Uint4x32) throw InvalidArgument("Uint4x32_to_prec_uniform not supported for Uint4x32");
+        std::vector<std::string> lines;
+        lines.push_back(c_vec_typ(c.length, n.prec) + " vec_result = uint4x32_to_" + prec_string(n.prec) +
+                        "_uniform_vec(" + a + ");");
+        for (int i = 0; i < c.length; ++i) {
+          std::string off;
+          const AxisIndex& last = c.idcs.back();
+          if (last.kind == AxisIndex::Fixed) {
+            Indices el = c.idcs; el.back().fixed += i;
+            off = offset_str(el, n.dims);
+          } else off = offset_str(c.idcs, n.dims) + " + " + std::to_string(i);
+          lines.push_back(n.ident + "[" + off + "] = " +
+                          (c.length == 1 ? std::string("vec_result") : "vec_result.v[" + std::to_string(i) + "]") + ";");
+        }
+        // always a block here: several statements of one kernel may declare vec_result
+        out.push_back(ind + "{");
+        std::vector<std::string> inner;
+        with_defs(defs, lines, ind + "  ", inner);
+        for (auto& l : inner) out.push_back(l);
+        out.push_back(ind + "}");
+        break;
+      }
+      case Stmt::SetLocal: {
+        std::vector<Def> defs;
+        std::string v = scalar(r.node(c.scope.node).prec, *c.value, ind + "  ", defs);
+        with_defs(defs, {scope_name(c.scope) + " = " + v + ";"}, ind, out);
+        break;
+      }
+      case Stmt::DeclareLocal: {
+        const Prec p = r.node(c.scope.node).prec;
+        out.push_back(ind + c_typ(p) + " " + scope_name(c.scope) + (c.needs_init ? init_zero(p) : "") + ";");
+        break;
+      }
+    }
+  }
+
+  void block(const Block& b, const std::string& ind, std::vector<std::string>& out) {
+    for (auto& s : b) stmt(*s, ind, out);
+  }
+};
+
+std::string neutral_literal(Binop accum, bool dbl) {
+  switch (accum) {
+    case Binop::Max: return dbl ? "(-__builtin_huge_val())" : "(-INFINITY)";
+    case Binop::Min: return dbl ? "__builtin_huge_val()" : "INFINITY";
+    default: return dbl ? "0.0" : "0.0f";
+  }
+}
+
+std::string combine_expr(Binop accum, bool dbl, const std::string& a, const std::string& b) {
+  switch (accum) {
+    case Binop::Max: return std::string(dbl ? "fmax(" : "fmaxf(") + a + ", " + b + ")";
+    case Binop::Min: return std::string(dbl ? "fmin(" : "fminf(") + a + ", " + b + ")";
+    default: return "(" + a + " + " + b + ")";
+  }
+}
+
+}  // namespace
+
+GeneratedModule generate_module(const Routine& r, const Plan& plan) {
+  GeneratedModule mod;
+  std::ostringstream src;
+  src << builtins_hip_source() << "\n";
+  int kidx = 0;
+  for (size_t pi = 0; pi < plan.phases.size(); ++pi) {
+    const Phase& ph = plan.phases[pi];
+    if (ph.kind != Phase::Generic) continue;
+    Printer pr(r);
+    std::vector<std::string> body;
+    const std::string ind = "  ";
+
+    // --- thread -> point decode: the symbol with the smallest stride in the first written array
+    //     varies fastest across adjacent threads (coalesced stores)
+    std::vector<size_t> order(ph.par_syms.size());
+    for (size_t i = 0; i < order.size(); ++i) order[i] = i;
+    const Stmt* first_set = nullptr;
+    std::function<void(const Block&)> find_set = [&](const Block& b) {
+      for (auto& s : b) {
+        if (first_set) return;
+        if (s->kind == Stmt::Set || s->kind == Stmt::SetVec) first_set = s.get();
+        else if (s->kind == Stmt::For) find_set(s->body);
+      }
+    };
+    find_set(ph.inner);
+    auto lhs_stride = [&](int sym) -> int64_t {
+      if (!first_set) return 0;
+      const Node& n = r.node(first_set->node);
+      int64_t st = 0, rs = 1;
+      for (int p = (int)first_set->idcs.size() - 1; p >= 0; --p) {
+        const AxisIndex& a = first_set->idcs[p];
+        if (a.kind == AxisIndex::Iter && a.sym == sym) st += rs;
+        if (a.kind == AxisIndex::Affine) for (auto& t : a.terms) if (t.second == sym) st += t.first * rs;
+        rs *= n.dims[p];
+      }
+      return st;
+    };
+    std::stable_sort(order.begin(), order.end(), [&](size_t x, size_t y) {
+      return lhs_stride(ph.par_syms[x]) > lhs_stride(ph.par_syms[y]); });   // slowest first
+
+    uint64_t P = 1;
+    for (auto e : ph.par_ext) P *= (uint64_t)e;
+    const int G = ph.coop_lanes;
+    body.push_back(ind + "const uint64_t gtid_ = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;");
+    if (G > 1) {
+      body.push_back(ind + "const uint32_t lane_ = (uint32_t)(gtid_ % " + std::to_string(G) + "u);");
+      body.push_back(ind + "uint64_t pt_ = gtid_ / " + std::to_string(G) + "u;");
+    } else {
+      body.push_back(ind + "uint64_t pt_ = gtid_;");
+    }
+    body.push_back(ind + "if (pt_ >= " + std::to_string(P) + "ull) return;");
+    for (int k = (int)order.size() - 1; k >= 0; --k) {
+      const size_t i = order[k];
+      const std::string s = sym_ident(ph.par_syms[i]);
+      const std::string ext = std::to_string(ph.par_ext[i]) + "ull";
+      std::string line = ind + "const uint32_t " + s + " = (uint32_t)(" + std::to_string(ph.par_from[i]) + " + ";
+      if (k == 0) line += "pt_);";
+      else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
+      body.push_back(line);
+    }
+
+    Binop accum = Binop::Add;
+    bool is_reduction = false;
+    const Stmt* set = nullptr;
+    if (!ph.seq_syms.empty() && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set) {
+      set = ph.inner[0].get();
+      const Scalar& v = *set->value;
+      auto is_self = [&](const Scalar& s) { return s.kind == Scalar::Get && s.node == set->node && s.idcs == set->idcs; };
+      if (v.kind == Scalar::Tern && v.tern == Ternop::Fma && is_self(*v.c)) { is_reduction = true; accum = Binop::Add; }
+      else if (v.kind == Scalar::Bin && (v.bin == Binop::Add || v.bin == Binop::Max || v.bin == Binop::Min) &&
+               (is_self(*v.a) || is_self(*v.b))) { is_reduction = true; accum = v.bin; }
+      // the lhs indices must not depend on a sequential symbol (they cannot: it would be parallel)
+    }
+
+    auto open_seq_loops = [&](std::string& cur_ind, bool coop_last) {
+      for (size_t i = 0; i < ph.seq_syms.size(); ++i) {
+        const std::string s = sym_ident(ph.seq_syms[i]);
+        if (coop_last && i + 1 == ph.seq_syms.size())
+          body.push_back(cur_ind + "for (uint32_t " + s + " = " + std::to_string(ph.seq_from[i]) + " + lane_; " + s +
+                         " <= " + std::to_string(ph.seq_to[i]) + "; " + s + " += " + std::to_string(G) + ") {");
+        else
+          body.push_back(cur_ind + "for (uint32_t " + s + " = " + std::to_string(ph.seq_from[i]) + "; " + s + " <= " +
+                         std::to_string(ph.seq_to[i]) + "; ++" + s + ") {");
+        cur_ind += "  ";
+      }
+    };
+    auto close_seq_loops = [&](std::string& cur_ind) {
+      for (size_t i = 0; i < ph.seq_syms.size(); ++i) { cur_ind.resize(cur_ind.size() - 2); body.push_back(cur_ind + "}"); }
+    };
+
+    if (is_reduction && G > 1) {
+      // lanes of a group stride the innermost sequential loop; partials are combined by butterfly
+      // shuffles in a fixed order (deterministic), accumulating in float (double for double).
+      const Node& n = r.node(set->node);
+      pr.note(set->node, set->idcs);
+      const bool dbl = n.prec == Prec::Double;
+      const std::string accT = dbl ? "double" : "float";
+      const Prec accP = dbl ? Prec::Double : Prec::Single;
+      body.push_back(ind + accT + " part_ = " + neutral_literal(accum, dbl) + ";");
+      std::string ci = ind;
+      open_seq_loops(ci, true);
+      const Scalar& v = *set->value;
+      std::vector<Printer::Def> defs;
+      std::vector<std::string> lines;
+      auto widen = [&](const std::string& e) { Pair c = convert_precision(n.prec, accP); return c.first + e + c.second; };
+      if (v.kind == Scalar::Tern) {
+        std::string a = pr.scalar(n.prec, *v.a, ci + "  ", defs), b = pr.scalar(n.prec, *v.b, ci + "  ", defs);
+        lines.push_back(std::string("part_ = ") + (dbl ? "fma(" : "fmaf(") + widen(a) + ", " + widen(b) + ", part_);");
+      } else {
+        auto is_self = [&](const Scalar& s) { return s.kind == Scalar::Get && s.node == set->node && s.idcs == set->idcs; };
+        const Scalar& e = is_self(*v.a) ? *v.b : *v.a;
+        std::string es = pr.scalar(n.prec, e, ci + "  ", defs);
+        lines.push_back("part_ = " + combine_expr(accum, dbl, "part_", widen(es)) + ";");
+      }
+      pr.with_defs(defs, lines, ci, body);
+      close_seq_loops(ci);
+      for (int o = G / 2; o > 0; o >>= 1)
+        body.push_back(ind + "part_ = " + combine_expr(accum, dbl, "part_", "ocn_xshfl(part_, " + std::to_string(o) + ")") + ";");
+      const std::string lhs = n.ident + "[" + offset_str(set->idcs, n.dims) + "]";
+      Pair narrow = convert_precision(accP, n.prec);
+      Pair wide = convert_precision(n.prec, accP);
+      if (ph.fused_zero_init)
+        body.push_back(ind + "if (lane_ == 0) " + lhs + " = " + narrow.first + "part_" + narrow.second + ";");
+      else
+        body.push_back(ind + "if (lane_ == 0) " + lhs + " = " + narrow.first +
+                       combine_expr(accum, dbl, wide.first + lhs + wide.second, "part_") + narrow.second + ";");
+    } else if (is_reduction) {
+      // one thread per output element, sequential loops in the reference's order: for fp32 this is
+      // the same operation sequence as the `cc` backend's serial loop.
+      const Node& n = r.node(set->node);
+      pr.note(set->node, set->idcs);
+      const std::string lhs = n.ident + "[" + offset_str(set->idcs, n.dims) + "]";
+      Pair zero = convert_precision(Prec::Double, n.prec);
+      body.push_back(ind + c_typ(n.prec) + " acc_ = " + (ph.fused_zero_init ? zero.first + "0" + zero.second : lhs) + ";");
+      std::string ci = ind;
+      open_seq_loops(ci, false);
+      pr.self_set = set; pr.self_name = "acc_";
+      std::vector<Printer::Def> defs;
+      std::string v = pr.scalar(n.prec, *set->value, ci + "  ", defs);
+      pr.with_defs(defs, {"acc_ = " + v + ";"}, ci, body);
+      pr.self_set = nullptr;
+      close_seq_loops(ci);
+      body.push_back(ind + lhs + " = acc_;");
+    } else {
+      if (ph.fused_zero_init) throw InvalidArgument("planner: fused zero-init on a non-reduction phase");
+      std::string ci = ind;
+      open_seq_loops(ci, false);
+      pr.block(ph.inner, ci, body);
+      close_seq_loops(ci);
+    }
+
+    GeneratedKernel gk;
+    gk.name = r.name + "_k" + std::to_string(kidx++);
+    gk.phase_index = (int)pi;
+    gk.threads = P * (uint64_t)G;
+    gk.block = 256;
+    std::vector<std::string> decls;
+    for (int id : r.node_order) {
+      if (!pr.used_nodes.count(id)) continue;
+      const Node& n = r.node(id);
+      decls.push_back(std::string(c_typ(n.prec)) + " * __restrict__ " + n.ident);
+      gk.params.push_back({KernelParam::NodePtr, id});
+    }
+    for (int id : pr.used_nodes) {   // planner-made scratch nodes are not in node_order
+      if (std::find(r.node_order.begin(), r.node_order.end(), id) != r.node_order.end()) continue;
+      const Node& n = r.node(id);
+      decls.push_back(std::string(c_typ(n.prec)) + " * __restrict__ " + n.ident);
+      gk.params.push_back({KernelParam::NodePtr, id});
+    }
+    for (auto& s : r.statics) {
+      if (!pr.used_statics.count(s.sym)) continue;
+      decls.push_back("const uint32_t " + sym_ident(s.sym));
+      gk.params.push_back({KernelParam::StaticIdx, s.sym});
+    }
+    src << "/* phase " << pi << ": " << ph.label << " */\n";
+    src << "extern \"C\" __global__ void __launch_bounds__(256) " << gk.name << "(";
+    for (size_t i = 0; i < decls.size(); ++i) src << (i ? ", " : "") << decls[i];
+    src << ") {\n";
+    for (auto& l : body) src << l << "\n";
+    src << "}\n\n";
+    mod.kernels.push_back(std::move(gk));
+  }
+  mod.source = src.str();
+  return mod;
+}
+
+}  // namespace ocannl

@@ -1,0 +1,40 @@
+// HIP source generation for the generic (non-MFMA) phases of a routine.
+//
+// The scalar expression printer follows the reference's C printer rule for rule -- evaluate every
+// operation in the precision of the enclosing destination, convert on load, compute reduced
+// precisions in float with a conversion around each single operation
+// (arrayjit/lib/c_syntax.ml:706-855, arrayjit/lib/cc_backend.ml:169-323, tables
+// arrayjit/lib/ops.ml:579-876) -- while the statement printer differs by design: instead of one
+// serial function (c_syntax.ml:1021-1210) each phase becomes a __global__ kernel whose threads own
+// the points of the phase's parallel index space.
+#pragma once
+#include <string>
+#include <vector>
+
+#include "plan.hpp"
+
+namespace ocannl {
+
+struct KernelParam {
+  enum Kind { NodePtr, StaticIdx } kind;
+  int id;   // node id or static symbol
+};
+
+struct GeneratedKernel {
+  std::string name;
+  std::vector<KernelParam> params;
+  uint64_t threads = 0;      // total threads wanted (points x cooperating lanes)
+  int block = 256;
+  int phase_index = -1;
+};
+
+struct GeneratedModule {
+  std::string source;                      // builtins + all kernels
+  std::vector<GeneratedKernel> kernels;    // one per generic phase, in phase order
+};
+
+const char* builtins_hip_source();
+
+GeneratedModule generate_module(const Routine& r, const Plan& plan);
+
+}  // namespace ocannl

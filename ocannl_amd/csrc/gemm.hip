@@ -1,0 +1,492 @@
+// Hand-written CDNA4 (gfx950) MFMA kernels for OCANNL's `+*` contractions:
+//     C[batch, m, n] (+)= sum_k A[batch, m, k] * B[batch, n, k]
+// i.e. the loop nests `c[..] := fma(a[..], b[..], c[..])` that Assignments.to_low_level emits for
+// matmul / einsum and their gradients (arrayjit/lib/assignments.ml:311-488,
+// tensor/operation.ml:77-99), which the reference runs as a serial scalar loop.
+//
+// Layout freedom: each operand is unit-stride either along K or along its row dimension (M for A,
+// N for B) with an arbitrary leading stride, plus up to three batch strides -- this covers the
+// forward (both K-contiguous), dX (B row-contiguous) and dW (both row-contiguous) forms and the
+// attention contractions on [b, s, h, d] tensors without any transposition pass.
+//
+// Kernel structure (bf16 compute, fp32 accumulate):
+//   * 256 threads = 4 wavefronts in a 2x2 grid; block tile BM x BN, K step 64;
+//   * global -> registers (16-byte loads) -> LDS, double buffered, one barrier per K step;
+//     row-contiguous operands are transposed 8x8 in registers on the way so that LDS always holds
+//     [row][k] with k contiguous; rows are padded by 16 bytes so that ds_read_b128 of 16 rows hits
+//     distinct banks; fp32 sources are rounded to bf16 (RNE) on the way;
+//   * v_mfma_f32_32x32x16_bf16, each wavefront owns a (BM/2) x (BN/2) sub-tile;
+//   * workgroup ids are remapped so that each XCD (ids are dealt round-robin over 8 XCDs) works on
+//     a compact band of tiles and shares B/A panels through its own L2.
+// fp32 compute uses v_mfma_f32_32x32x2_f32 with the same staging.
+#include <hip/hip_runtime.h>
+
+#include "gemm.hpp"
+
+namespace ocannl {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kBK = 64;        // K elements per stage (bf16 compute)
+constexpr int kPad = 8;        // bf16 elements of row padding (16 bytes)
+constexpr int kBKf = 32;       // K elements per stage (fp32 compute)
+constexpr int kPadf = 4;       // floats of row padding (16 bytes)
+
+__device__ __forceinline__ unsigned f2bf(float f) {   // round to nearest even, as single_to_bfloat16
+  const unsigned w = __float_as_uint(f);
+  return (w + 0x7FFFu + ((w >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ unsigned pack2(float lo, float hi) { return f2bf(lo) | (f2bf(hi) << 16); }
+
+// 8 consecutive source elements -> 8 bf16 in a uint4
+template <typename T>
+__device__ __forceinline__ u32x4 load8(const T* p);
+template <>
+__device__ __forceinline__ u32x4 load8<unsigned short>(const unsigned short* p) {
+  return *reinterpret_cast<const u32x4*>(p);
+}
+template <>
+__device__ __forceinline__ u32x4 load8<float>(const float* p) {
+  const f32x4 x = *reinterpret_cast<const f32x4*>(p);
+  const f32x4 y = *reinterpret_cast<const f32x4*>(p + 4);
+  u32x4 r;
+  r.x = pack2(x.x, x.y); r.y = pack2(x.z, x.w); r.z = pack2(y.x, y.y); r.w = pack2(y.z, y.w);
+  return r;
+}
+
+__device__ __forceinline__ void decode_batch(const GemmArgs& g, long z, long& ao, long& bo, long& co) {
+  ao = bo = co = 0;
+  for (int i = g.nbatch - 1; i >= 0; --i) {
+    const long e = g.batch_ext[i];
+    const long q = z % e;
+    z /= e;
+    ao += q * g.a_batch[i]; bo += q * g.b_batch[i]; co += q * g.c_batch[i];
+  }
+}
+
+// XCD-aware tile order: consecutive hardware workgroup ids land on different XCDs; give XCD x the
+// x-th contiguous slice of the tile sequence, and walk tiles in column-bands of 8 row-tiles so that
+// a slice re-uses the same B panels.
+__device__ __forceinline__ void tile_of_block(long wg, long tiles_m, long tiles_n, long& tm, long& tn) {
+  const long total = tiles_m * tiles_n;
+  long t = wg;
+  if (total % 8 == 0) t = (wg % 8) * (total / 8) + wg / 8;
+  constexpr long kGroup = 8;
+  const long band = kGroup * tiles_n;
+  const long g = t / band;
+  const long first_m = g * kGroup;
+  const long gm = (tiles_m - first_m) < kGroup ? (tiles_m - first_m) : kGroup;
+  const long r = t % band;
+  tm = first_m + r % gm;
+  tn = r / gm;
+}
+
+// ---- staging one operand tile: global -> registers ---------------------------------------------
+// ROWS x kBK tile starting at (row0, k0).  K-contiguous: thread owns chunks of 8 k at one row.
+// Row-contiguous: thread owns 8(k) x 8(row) blocks, transposed in registers.
+template <int ROWS, typename T, bool KC>
+struct Stager {
+  static constexpr int kChunks = ROWS * (kBK / 8) / kThreads;   // 16-byte LDS chunks per thread
+  static constexpr int kBlocks = (ROWS + kThreads - 1) / kThreads;  // 8x8 blocks per thread (row-contiguous)
+  u32x4 regs[KC ? kChunks : kBlocks * 8];
+
+  __device__ __forceinline__ void load(const T* base, long ld, long row0, long k0, long rows, long K, int tid) {
+    if (KC) {
+#pragma unroll
+      for (int j = 0; j < kChunks; ++j) {
+        const int c = tid + kThreads * j;
+        const long row = row0 + c / (kBK / 8);
+        const long k = k0 + (c % (kBK / 8)) * 8;
+        u32x4 v = {0, 0, 0, 0};
+        if (row < rows && k < K) v = load8<T>(base + row * ld + k);
+        regs[j] = v;
+      }
+    } else {
+      // blocks: (kBK/8) k-groups x (ROWS/8) row-chunks; kChunks/8 blocks per thread
+#pragma unroll
+      for (int jb = 0; jb < kBlocks; ++jb) {
+        const int blk = tid + kThreads * jb;
+        const long row = row0 + (blk % (ROWS / 8)) * 8;
+        const long kg = k0 + (blk / (ROWS / 8)) * 8;
+        u32x4 in[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+          u32x4 v = {0, 0, 0, 0};
+          if (blk < ROWS && row < rows && kg + kk < K) v = load8<T>(base + (kg + kk) * ld + row);
+          in[kk] = v;
+        }
+        // transpose 8x8 of 16-bit: out[m] holds k = 0..7 for row m
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+          unsigned w[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const unsigned lo = in[2 * j][m / 2], hi = in[2 * j + 1][m / 2];
+            w[j] = (m & 1) ? ((lo >> 16) | (hi & 0xFFFF0000u)) : ((lo & 0xFFFFu) | (hi << 16));
+          }
+          u32x4 o = {w[0], w[1], w[2], w[3]};
+          regs[jb * 8 + m] = o;
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(unsigned short* lds, int tid) const {
+    constexpr int kStride = kBK + kPad;
+    if (KC) {
+#pragma unroll
+      for (int j = 0; j < kChunks; ++j) {
+        const int c = tid + kThreads * j;
+        *reinterpret_cast<u32x4*>(lds + (c / (kBK / 8)) * kStride + (c % (kBK / 8)) * 8) = regs[j];
+      }
+    } else {
+#pragma unroll
+      for (int jb = 0; jb < kBlocks; ++jb) {
+        const int blk = tid + kThreads * jb;
+        if (blk >= ROWS) break;
+        const int row = (blk % (ROWS / 8)) * 8, kg = (blk / (ROWS / 8)) * 8;
+#pragma unroll
+        for (int m = 0; m < 8; ++m)
+          *reinterpret_cast<u32x4*>(lds + (row + m) * kStride + kg) = regs[jb * 8 + m];
+      }
+    }
+  }
+};
+
+template <int BM, int BN, typename AT, typename BT, bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(kThreads) gemm_bf16_kernel(const GemmArgs g) {
+  constexpr int kStride = kBK + kPad;
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+  extern __shared__ __align__(16) unsigned short smem[];
+  unsigned short* const As0 = smem;
+  unsigned short* const Bs0 = smem + 2 * BM * kStride;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+  const long tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+  long tmi, tni;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, tmi, tni);
+  const long m0 = tmi * BM, n0 = tni * BN;
+  long ao, bo, co;
+  decode_batch(g, blockIdx.z, ao, bo, co);
+  const AT* A = static_cast<const AT*>(g.a) + ao;
+  const BT* B = static_cast<const BT*>(g.b) + bo;
+  const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  Stager<BM, AT, A_KC> sa;
+  Stager<BN, BT, B_KC> sb;
+  sa.load(A, lda, m0, 0, g.M, g.K, tid);
+  sb.load(B, ldb, n0, 0, g.N, g.K, tid);
+  sa.store(As0, tid);
+  sb.store(Bs0, tid);
+  __syncthreads();
+
+  const long ksteps = (g.K + kBK - 1) / kBK;
+  for (long ks = 0; ks < ksteps; ++ks) {
+    const int cur = ks & 1;
+    const bool more = ks + 1 < ksteps;
+    if (more) {
+      sa.load(A, lda, m0, (ks + 1) * kBK, g.M, g.K, tid);
+      sb.load(B, ldb, n0, (ks + 1) * kBK, g.N, g.K, tid);
+    }
+    const unsigned short* as = As0 + cur * BM * kStride + (wm0 + (lane & 31)) * kStride + (lane >> 5) * 8;
+    const unsigned short* bs = Bs0 + cur * BN * kStride + (wn0 + (lane & 31)) * kStride + (lane >> 5) * 8;
+#pragma unroll
+    for (int kk = 0; kk < kBK / 16; ++kk) {
+      bf16x8 af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(as + i * 32 * kStride + kk * 16);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(bs + j * 32 * kStride + kk * 16);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      sa.store(As0 + (cur ^ 1) * BM * kStride, tid);
+      sb.store(Bs0 + (cur ^ 1) * BN * kStride, tid);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane holds column (lane % 32); register e holds row 8*(e/4) + 4*(lane/32) + e%4
+  const long ldc = g.c_row;
+  const int col = lane & 31, rbase = (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const long n = n0 + wn0 + j * 32 + col;
+      if (n >= g.N) continue;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const long m = m0 + wm0 + i * 32 + (e >> 2) * 8 + rbase + (e & 3);
+        if (m >= g.M) continue;
+        const long off = co + m * ldc + n;
+        float v = acc[i][j][e];
+        if (g.c_is_bf16) {
+          unsigned short* C = static_cast<unsigned short*>(g.c);
+          if (g.accumulate) v += __uint_as_float(((unsigned)C[off]) << 16);
+          C[off] = (unsigned short)f2bf(v);
+        } else {
+          float* C = static_cast<float*>(g.c);
+          if (g.accumulate) v += C[off];
+          C[off] = v;
+        }
+      }
+    }
+  }
+}
+
+// ---- fp32 compute -------------------------------------------------------------------------------
+// LDS holds [row][k] floats, k contiguous; a lane reads 4 consecutive k of its row with one
+// ds_read_b128 and feeds four v_mfma_f32_32x32x2_f32: instruction q multiplies k = q (lanes 0-31)
+// and k = 4 + q (lanes 32-63) -- A and B use the same assignment, so the sum is complete.
+template <int ROWS, bool KC>
+struct StagerF {
+  static constexpr int kChunks = ROWS * (kBKf / 4) / kThreads;   // 16-byte chunks per thread
+  f32x4 regs[kChunks];
+
+  __device__ __forceinline__ void load(const float* base, long ld, long row0, long k0, long rows, long K, int tid) {
+    if (KC) {
+#pragma unroll
+      for (int j = 0; j < kChunks; ++j) {
+        const int c = tid + kThreads * j;
+        const long row = row0 + c / (kBKf / 4);
+        const long k = k0 + (c % (kBKf / 4)) * 4;
+        f32x4 v = {0, 0, 0, 0};
+        if (row < rows && k < K) v = *reinterpret_cast<const f32x4*>(base + row * ld + k);
+        regs[j] = v;
+      }
+    } else {
+      // 4(k) x 4(row) blocks: (kBKf/4) k-groups x (ROWS/4) row-chunks
+#pragma unroll
+      for (int jb = 0; jb < kChunks / 4; ++jb) {
+        const int blk = tid + kThreads * jb;
+        const long row = row0 + (blk % (ROWS / 4)) * 4;
+        const long kg = k0 + (blk / (ROWS / 4)) * 4;
+        f32x4 in[4];
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          f32x4 v = {0, 0, 0, 0};
+          if (row < rows && kg + kk < K) v = *reinterpret_cast<const f32x4*>(base + (kg + kk) * ld + row);
+          in[kk] = v;
+        }
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          f32x4 o = {in[0][m], in[1][m], in[2][m], in[3][m]};
+          regs[jb * 4 + m] = o;
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(float* lds, int tid) const {
+    constexpr int kStride = kBKf + kPadf;
+    if (KC) {
+#pragma unroll
+      for (int j = 0; j < kChunks; ++j) {
+        const int c = tid + kThreads * j;
+        *reinterpret_cast<f32x4*>(lds + (c / (kBKf / 4)) * kStride + (c % (kBKf / 4)) * 4) = regs[j];
+      }
+    } else {
+#pragma unroll
+      for (int jb = 0; jb < kChunks / 4; ++jb) {
+        const int blk = tid + kThreads * jb;
+        const int row = (blk % (ROWS / 4)) * 4, kg = (blk / (ROWS / 4)) * 4;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) *reinterpret_cast<f32x4*>(lds + (row + m) * kStride + kg) = regs[jb * 4 + m];
+      }
+    }
+  }
+};
+
+template <int BM, int BN, bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g) {
+  constexpr int kStride = kBKf + kPadf;
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+  extern __shared__ __align__(16) unsigned short smem[];
+  float* fsm = reinterpret_cast<float*>(smem);
+  float* const As0 = fsm;
+  float* const Bs0 = fsm + 2 * BM * kStride;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+  const long tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+  long tmi, tni;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, tmi, tni);
+  const long m0 = tmi * BM, n0 = tni * BN;
+  long ao, bo, co;
+  decode_batch(g, blockIdx.z, ao, bo, co);
+  const float* A = static_cast<const float*>(g.a) + ao;
+  const float* B = static_cast<const float*>(g.b) + bo;
+  const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  StagerF<BM, A_KC> sa;
+  StagerF<BN, B_KC> sb;
+  sa.load(A, lda, m0, 0, g.M, g.K, tid);
+  sb.load(B, ldb, n0, 0, g.N, g.K, tid);
+  sa.store(As0, tid);
+  sb.store(Bs0, tid);
+  __syncthreads();
+
+  const long ksteps = (g.K + kBKf - 1) / kBKf;
+  for (long ks = 0; ks < ksteps; ++ks) {
+    const int cur = ks & 1;
+    const bool more = ks + 1 < ksteps;
+    if (more) {
+      sa.load(A, lda, m0, (ks + 1) * kBKf, g.M, g.K, tid);
+      sb.load(B, ldb, n0, (ks + 1) * kBKf, g.N, g.K, tid);
+    }
+    const float* as = As0 + cur * BM * kStride + (wm0 + (lane & 31)) * kStride + (lane >> 5) * 4;
+    const float* bs = Bs0 + cur * BN * kStride + (wn0 + (lane & 31)) * kStride + (lane >> 5) * 4;
+#pragma unroll
+    for (int kk = 0; kk < kBKf / 8; ++kk) {
+      f32x4 af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const f32x4*>(as + i * 32 * kStride + kk * 8);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const f32x4*>(bs + j * 32 * kStride + kk * 8);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][q], bf[j][q], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      sa.store(As0 + (cur ^ 1) * BM * kStride, tid);
+      sb.store(Bs0 + (cur ^ 1) * BN * kStride, tid);
+    }
+    __syncthreads();
+  }
+
+  const long ldc = g.c_row;
+  const int col = lane & 31, rbase = (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const long n = n0 + wn0 + j * 32 + col;
+      if (n >= g.N) continue;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const long m = m0 + wm0 + i * 32 + (e >> 2) * 8 + rbase + (e & 3);
+        if (m >= g.M) continue;
+        const long off = co + m * ldc + n;
+        float v = acc[i][j][e];
+        if (g.c_is_bf16) {
+          unsigned short* C = static_cast<unsigned short*>(g.c);
+          if (g.accumulate) v += __uint_as_float(((unsigned)C[off]) << 16);
+          C[off] = (unsigned short)f2bf(v);
+        } else {
+          float* C = static_cast<float*>(g.c);
+          if (g.accumulate) v += C[off];
+          C[off] = v;
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN>
+constexpr size_t bf16_smem() { return 2ull * (BM + BN) * (kBK + kPad) * sizeof(unsigned short); }
+template <int BM, int BN>
+constexpr size_t f32_smem() { return 2ull * (BM + BN) * (kBKf + kPadf) * sizeof(float); }
+
+template <typename K>
+hipError_t launch(K kernel, size_t smem, int BM, int BN, const GemmArgs& a, hipStream_t s) {
+  static thread_local const void* configured[64];
+  static thread_local int n_configured = 0;
+  bool done = false;
+  for (int i = 0; i < n_configured; ++i) done |= configured[i] == (const void*)kernel;
+  if (!done) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return e;
+    if (n_configured < 64) configured[n_configured++] = (const void*)kernel;
+  }
+  const long tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  long nb = 1;
+  for (int i = 0; i < a.nbatch; ++i) nb *= a.batch_ext[i];
+  if (tiles <= 0 || tiles > 0x7FFFFFFFL || nb <= 0 || nb > 65535) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, 1, (unsigned)nb), dim3(kThreads), smem, s, a);
+  return hipGetLastError();
+}
+
+template <int BM, int BN, typename AT, typename BT>
+hipError_t launch_bf16_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t s) {
+  constexpr size_t sm = bf16_smem<BM, BN>();
+  if (akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, true>, sm, BM, BN, a, s);
+  if (akc && !bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, false>, sm, BM, BN, a, s);
+  if (!akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, true>, sm, BM, BN, a, s);
+  return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, false>, sm, BM, BN, a, s);
+}
+
+template <int BM, int BN>
+hipError_t launch_f32_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t s) {
+  constexpr size_t sm = f32_smem<BM, BN>();
+  if (akc && bkc) return launch(gemm_f32_kernel<BM, BN, true, true>, sm, BM, BN, a, s);
+  if (akc && !bkc) return launch(gemm_f32_kernel<BM, BN, true, false>, sm, BM, BN, a, s);
+  if (!akc && bkc) return launch(gemm_f32_kernel<BM, BN, false, true>, sm, BM, BN, a, s);
+  return launch(gemm_f32_kernel<BM, BN, false, false>, sm, BM, BN, a, s);
+}
+
+bool a_kcontig(const GemmDesc& d) { return d.a.s_k == 1 || d.K == 1; }
+bool b_kcontig(const GemmDesc& d) { return d.b.s_k == 1 || d.K == 1; }
+bool big_tile(const GemmDesc& d) {
+  // 256x256 tiles only when they still fill the chip (>= 256 workgroups)
+  double nb = 1;
+  for (int i = 0; i < d.nbatch; ++i) nb *= (double)d.batch_ext[i];
+  const double tiles = ((d.M + 255) / 256) * (double)((d.N + 255) / 256) * nb;
+  return tiles >= 256;
+}
+
+}  // namespace
+
+const char* gemm_kernel_name(const GemmDesc& d) {
+  const bool f32 = d.a.prec == Prec::Single && d.b.prec == Prec::Single;
+  const bool big = big_tile(d);
+  if (f32) return big ? "gemm_f32_kernel<256,256>" : "gemm_f32_kernel<128,128>";
+  return big ? "gemm_bf16_kernel<256,256>" : "gemm_bf16_kernel<128,128>";
+}
+
+hipError_t launch_gemm(const GemmDesc& d, const GemmArgs& a, hipStream_t s) {
+  const bool akc = a_kcontig(d), bkc = b_kcontig(d);
+  const bool big = big_tile(d);
+  const bool af = d.a.prec == Prec::Single, bf = d.b.prec == Prec::Single;
+  if (af && bf) return big ? launch_f32_layout<256, 256>(akc, bkc, a, s) : launch_f32_layout<128, 128>(akc, bkc, a, s);
+  if (!af && !bf)
+    return big ? launch_bf16_layout<256, 256, unsigned short, unsigned short>(akc, bkc, a, s)
+               : launch_bf16_layout<128, 128, unsigned short, unsigned short>(akc, bkc, a, s);
+  if (af && !bf)
+    return big ? launch_bf16_layout<256, 256, float, unsigned short>(akc, bkc, a, s)
+               : launch_bf16_layout<128, 128, float, unsigned short>(akc, bkc, a, s);
+  return big ? launch_bf16_layout<256, 256, unsigned short, float>(akc, bkc, a, s)
+             : launch_bf16_layout<128, 128, unsigned short, float>(akc, bkc, a, s);
+}
+
+}  // namespace ocannl

@@ -1,0 +1,30 @@
+// Launch interface of the hand-written CDNA4 MFMA contraction kernels (gemm.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "plan.hpp"
+
+namespace ocannl {
+
+// Device-side view of one strided-batched contraction.
+struct GemmArgs {
+  const void* a;
+  const void* b;
+  void* c;
+  int64_t M, N, K;
+  int64_t a_row, a_k, b_row, b_k, c_row;   // element strides; C is unit-stride along N
+  int nbatch;
+  int64_t batch_ext[3];
+  int64_t a_batch[3], b_batch[3], c_batch[3];
+  int accumulate;    // beta = 1
+  int c_is_bf16;
+};
+
+// Picks the kernel instance for the operand precisions / layouts and launches it on `stream`.
+// Returns hipErrorInvalidValue for a combination the planner should not have produced.
+hipError_t launch_gemm(const GemmDesc& desc, const GemmArgs& args, hipStream_t stream);
+
+// Name of the instance launch_gemm would pick (for kernel_info and profiles).
+const char* gemm_kernel_name(const GemmDesc& desc);
+
+}  // namespace ocannl

@@ -1,0 +1,474 @@
+#include "plan.hpp"
+
+#include <algorithm>
+#include <functional>
+#include <set>
+
+namespace ocannl {
+namespace {
+
+struct Access {
+  int node;
+  const Indices* idcs;
+  bool write;
+  int vec_len;   // >0 for Set_from_vec writes
+};
+
+void scalar_accesses(const Scalar& s, std::vector<Access>& out, bool& foreign_local_write,
+                     std::set<ScopeId>& declared);
+void block_accesses(const Block& b, std::vector<Access>& out, bool& whole_array_write,
+                    bool& foreign_local_write, std::set<ScopeId>& declared) {
+  for (auto& sp : b) {
+    const Stmt& s = *sp;
+    switch (s.kind) {
+      case Stmt::Comment: break;
+      case Stmt::For: block_accesses(s.body, out, whole_array_write, foreign_local_write, declared); break;
+      case Stmt::ZeroOut: whole_array_write = true; break;
+      case Stmt::Set:
+        out.push_back({s.node, &s.idcs, true, 0});
+        scalar_accesses(*s.value, out, foreign_local_write, declared);
+        break;
+      case Stmt::SetVec:
+        out.push_back({s.node, &s.idcs, true, s.length});
+        scalar_accesses(*s.value, out, foreign_local_write, declared);
+        break;
+      case Stmt::SetLocal:
+        if (!declared.count(s.scope)) foreign_local_write = true;
+        scalar_accesses(*s.value, out, foreign_local_write, declared);
+        break;
+      case Stmt::DeclareLocal: declared.insert(s.scope); break;
+    }
+  }
+}
+
+void scalar_accesses(const Scalar& s, std::vector<Access>& out, bool& flw, std::set<ScopeId>& declared) {
+  switch (s.kind) {
+    case Scalar::Get: case Scalar::GetMerge: out.push_back({s.node, &s.idcs, false, 0}); break;
+    case Scalar::GetDyn:
+      out.push_back({s.node, &s.idcs, false, 0});
+      scalar_accesses(*s.a, out, flw, declared);
+      break;
+    case Scalar::LocalScope: {
+      declared.insert(s.scope);
+      bool whole = false;
+      block_accesses(s.body, out, whole, flw, declared);
+      break;
+    }
+    case Scalar::Un: scalar_accesses(*s.a, out, flw, declared); break;
+    case Scalar::Bin: scalar_accesses(*s.a, out, flw, declared); scalar_accesses(*s.b, out, flw, declared); break;
+    case Scalar::Tern:
+      scalar_accesses(*s.a, out, flw, declared); scalar_accesses(*s.b, out, flw, declared);
+      scalar_accesses(*s.c, out, flw, declared);
+      break;
+    default: break;
+  }
+}
+
+// Axis at which `idcs` is driven by `sym` alone: Iterator sym, or a one-term Affine c*sym+o.
+int axis_of(const Indices& idcs, int sym) {
+  for (size_t p = 0; p < idcs.size(); ++p) {
+    const AxisIndex& a = idcs[p];
+    if (a.kind == AxisIndex::Iter && a.sym == sym) return (int)p;
+    if (a.kind == AxisIndex::Affine && a.terms.size() == 1 && a.terms[0].second == sym && a.terms[0].first != 0)
+      return (int)p;
+  }
+  return -1;
+}
+
+// A chain symbol is parallel when every array written below the chain is touched, in every access
+// (reads included), through one and the same index expression driven by that symbol on one and the
+// same axis: different values of the symbol then work on disjoint slices.
+bool symbol_is_parallel(int sym, const std::vector<Access>& acc) {
+  std::set<int> written;
+  for (auto& a : acc) if (a.write) written.insert(a.node);
+  for (int w : written) {
+    int axis = -1;
+    const AxisIndex* expr = nullptr;
+    for (auto& a : acc) {
+      if (a.node != w) continue;
+      int p = axis_of(*a.idcs, sym);
+      if (p < 0) return false;
+      const AxisIndex& e = (*a.idcs)[p];
+      if (a.vec_len > 0 && p == (int)a.idcs->size() - 1) {
+        // a vector write covers [e, e+len): needs a stride of at least len along sym
+        if (!(e.kind == AxisIndex::Affine && std::abs(e.terms[0].first) >= a.vec_len)) return false;
+      }
+      // the symbol must not also appear on another axis of this access
+      for (size_t q = 0; q < a.idcs->size(); ++q)
+        if ((int)q != p && (*a.idcs)[q].mentions(sym)) return false;
+      if (axis < 0) { axis = p; expr = &e; }
+      else if (axis != p || !(*expr == e)) return false;
+    }
+  }
+  return true;
+}
+
+bool same_indices(const Indices& a, const Indices& b) { return a == b; }
+
+int64_t row_major_stride(const Node& n, size_t axis) {
+  int64_t s = 1;
+  for (size_t q = axis + 1; q < n.dims.size(); ++q) s *= n.dims[q];
+  return s;
+}
+
+struct Strides {
+  std::map<int, int64_t> by_sym;
+  int64_t offset = 0;
+  std::vector<std::pair<int, int64_t>> statics;
+  bool ok = true;
+};
+
+Strides strides_of(const Routine& r, int node, const Indices& idcs) {
+  Strides st;
+  const Node& n = r.node(node);
+  for (size_t p = 0; p < idcs.size(); ++p) {
+    const int64_t rs = row_major_stride(n, p);
+    const AxisIndex& a = idcs[p];
+    if (a.kind == AxisIndex::Fixed) st.offset += a.fixed * rs;
+    else if (a.kind == AxisIndex::Iter) {
+      if (r.is_static(a.sym)) st.statics.emplace_back(a.sym, rs);
+      else st.by_sym[a.sym] += rs;
+    } else {
+      for (auto& t : a.terms) {
+        if (r.is_static(t.second)) st.statics.emplace_back(t.second, t.first * rs);
+        else st.by_sym[t.second] += t.first * rs;
+      }
+      st.offset += a.offset * rs;
+    }
+  }
+  return st;
+}
+
+int64_t get_stride(const Strides& s, int sym) {
+  auto it = s.by_sym.find(sym);
+  return it == s.by_sym.end() ? 0 : it->second;
+}
+
+bool mfma_prec(Prec p) { return p == Prec::Single || p == Prec::Bfloat16; }
+
+// Recognises `for.. { c[L] := fma(a[A], b[B], c[L]) }` (either operand order; also
+// `(a*b) + c`), fills a strided-batched GEMM descriptor.  Returns false to leave the phase generic.
+bool match_contraction(const Routine& r, Phase& ph, const PlanOptions& opt) {
+  if (!opt.enable_mfma) return false;
+  if (ph.inner.size() != 1 || ph.inner[0]->kind != Stmt::Set) return false;
+  const Stmt& set = *ph.inner[0];
+  const Scalar& v = *set.value;
+  const Scalar *pa = nullptr, *pb = nullptr, *pc = nullptr;
+  if (v.kind == Scalar::Tern && v.tern == Ternop::Fma) { pa = v.a.get(); pb = v.b.get(); pc = v.c.get(); }
+  else if (v.kind == Scalar::Bin && v.bin == Binop::Add) {
+    const Scalar* l = v.a.get(); const Scalar* rr = v.b.get();
+    if (rr->kind == Scalar::Bin && rr->bin == Binop::Mul) { pc = l; pa = rr->a.get(); pb = rr->b.get(); }
+    else if (l->kind == Scalar::Bin && l->bin == Binop::Mul) { pc = rr; pa = l->a.get(); pb = l->b.get(); }
+    else return false;
+  } else return false;
+  if (pa->kind != Scalar::Get || pb->kind != Scalar::Get || pc->kind != Scalar::Get) return false;
+  if (pc->node != set.node || !same_indices(pc->idcs, set.idcs)) return false;
+  if (pa->node == set.node || pb->node == set.node) return false;
+  const Node &na = r.node(pa->node), &nb = r.node(pb->node), &nc = r.node(set.node);
+  if (!mfma_prec(na.prec) || !mfma_prec(nb.prec) || !mfma_prec(nc.prec)) return false;
+
+  Strides sa = strides_of(r, pa->node, pa->idcs), sb = strides_of(r, pb->node, pb->idcs),
+          sc = strides_of(r, set.node, set.idcs);
+
+  struct Sym { int sym; int64_t ext, a, b, c; };
+  std::vector<Sym> batch, ms, ns, ks;
+  auto add_chain = [&](int sym, int64_t from, int64_t ext) -> bool {
+    if (from != 0) return false;
+    if (ext == 1) return true;  // degenerate loops contribute nothing
+    Sym s{sym, ext, get_stride(sa, sym), get_stride(sb, sym), get_stride(sc, sym)};
+    if (s.a < 0 || s.b < 0 || s.c < 0) return false;
+    const bool ia = s.a != 0, ib = s.b != 0, ic = s.c != 0;
+    if (ic && ia && ib) batch.push_back(s);
+    else if (ic && ia) ms.push_back(s);
+    else if (ic && ib) ns.push_back(s);
+    else if (ia && ib) ks.push_back(s);
+    else return false;
+    return true;
+  };
+  for (size_t i = 0; i < ph.par_syms.size(); ++i)
+    if (!add_chain(ph.par_syms[i], ph.par_from[i], ph.par_ext[i])) return false;
+  for (size_t i = 0; i < ph.seq_syms.size(); ++i)
+    if (!add_chain(ph.seq_syms[i], ph.seq_from[i], ph.seq_to[i] - ph.seq_from[i] + 1)) return false;
+
+  // merge symbols of one class that are contiguous in all three tensors
+  auto merge = [&](std::vector<Sym>& v, bool by_a) {
+    std::sort(v.begin(), v.end(), [&](const Sym& x, const Sym& y) {
+      return by_a ? x.a > y.a : x.c > y.c; });
+    for (size_t i = 0; i + 1 < v.size();) {
+      Sym &o = v[i], &in = v[i + 1];
+      if (o.a == in.ext * in.a && o.b == in.ext * in.b && o.c == in.ext * in.c) {
+        in.ext *= o.ext;
+        v.erase(v.begin() + i);
+      } else ++i;
+    }
+  };
+  merge(batch, false); merge(ms, false); merge(ns, false); merge(ks, true);
+  // surplus M / N symbols become batch dimensions (the other operand is re-read: stride 0)
+  while (ms.size() > 1) { batch.push_back(ms.front()); ms.erase(ms.begin()); }
+  while (ns.size() > 1) { batch.push_back(ns.front()); ns.erase(ns.begin()); }
+  if (ks.size() > 1 || batch.size() > 3) return false;
+
+  GemmDesc g;
+  g.M = ms.empty() ? 1 : ms[0].ext;
+  g.N = ns.empty() ? 1 : ns[0].ext;
+  g.K = ks.empty() ? 1 : ks[0].ext;
+  g.a.node = pa->node; g.a.prec = na.prec; g.a.offset = sa.offset; g.a.static_terms = sa.statics;
+  g.b.node = pb->node; g.b.prec = nb.prec; g.b.offset = sb.offset; g.b.static_terms = sb.statics;
+  g.c.node = set.node; g.c.prec = nc.prec; g.c.offset = sc.offset; g.c.static_terms = sc.statics;
+  g.a.s_row = ms.empty() ? 0 : ms[0].a;  g.a.s_k = ks.empty() ? 0 : ks[0].a;
+  g.b.s_row = ns.empty() ? 0 : ns[0].b;  g.b.s_k = ks.empty() ? 0 : ks[0].b;
+  g.c.s_row = ms.empty() ? 0 : ms[0].c;  g.c.s_k = ns.empty() ? 0 : ns[0].c;
+  g.nbatch = (int)batch.size();
+  for (int i = 0; i < g.nbatch; ++i) {
+    g.batch_ext[i] = batch[i].ext;
+    g.a.s_batch[i] = batch[i].a; g.b.s_batch[i] = batch[i].b; g.c.s_batch[i] = batch[i].c;
+  }
+  if (g.flops() < (double)opt.min_mfma_flops) return false;
+  if (g.M < 16 || g.N < 16 || g.K < 8) return false;   // matrix-vector shapes stay generic
+
+  // C must be contiguous along N; if it is contiguous along M instead, compute the transpose.
+  if (g.c.s_k != 1) {
+    if (g.c.s_row != 1) return false;
+    std::swap(g.a, g.b);
+    std::swap(g.M, g.N);
+    std::swap(g.c.s_row, g.c.s_k);
+  }
+  // each operand: unit stride along K or along its row dimension; vector-load alignment
+  const bool f32_compute = g.a.prec == Prec::Single && g.b.prec == Prec::Single;
+  auto operand_ok = [&](const GemmOperand& o, int64_t rows) {
+    // staging moves 8-element (bf16 compute) or 4-element (fp32 compute) chunks
+    const int vec = f32_compute ? 4 : 8;
+    if (o.s_k != 1 && o.s_row != 1) return false;
+    const int64_t ld = o.s_k == 1 ? o.s_row : o.s_k;
+    if (rows > 1 && g.K > 1 && ld % vec) return false;
+    if (o.offset % vec) return false;
+    for (auto& t : o.static_terms) if (t.second % vec) return false;
+    for (int i = 0; i < g.nbatch; ++i) if (o.s_batch[i] % vec) return false;
+    const int64_t contig = o.s_k == 1 ? g.K : rows;
+    if (contig % vec) return false;
+    return true;
+  };
+  if (!operand_ok(g.a, g.M) || !operand_ok(g.b, g.N)) return false;
+  {
+    const int vec = 4;
+    if (g.c.s_row % vec || g.c.offset % vec || g.N % vec) return false;
+    for (auto& t : g.c.static_terms) if (t.second % vec) return false;
+    for (int i = 0; i < g.nbatch; ++i) if (g.c.s_batch[i] % vec) return false;
+  }
+  g.accumulate = !ph.fused_zero_init;
+  ph.kind = Phase::Contraction;
+  ph.gemm = g;
+  ph.flops = g.flops();
+  return true;
+}
+
+// Is the phase `lhs[L] := accum(lhs[L], e)` / `fma(a, b, lhs[L])` with an associative, commutative
+// accum and `e` free of lhs?  Then sequential chain loops may be split across lanes.
+bool reduction_shape(const Routine& r, const Phase& ph, Binop* accum_out) {
+  if (ph.inner.size() != 1 || ph.inner[0]->kind != Stmt::Set) return false;
+  const Stmt& set = *ph.inner[0];
+  const Scalar& v = *set.value;
+  auto is_self = [&](const Scalar& s) {
+    return s.kind == Scalar::Get && s.node == set.node && same_indices(s.idcs, set.idcs); };
+  std::function<bool(const Scalar&)> reads_lhs = [&](const Scalar& s) -> bool {
+    switch (s.kind) {
+      case Scalar::Get: case Scalar::GetMerge: return s.node == set.node;
+      case Scalar::GetDyn: return s.node == set.node || reads_lhs(*s.a);
+      case Scalar::LocalScope: {
+        std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+        block_accesses(s.body, acc, w, f, d);
+        for (auto& a : acc) if (a.node == set.node) return true;
+        return false;
+      }
+      case Scalar::Un: return reads_lhs(*s.a);
+      case Scalar::Bin: return reads_lhs(*s.a) || reads_lhs(*s.b);
+      case Scalar::Tern: return reads_lhs(*s.a) || reads_lhs(*s.b) || reads_lhs(*s.c);
+      default: return false;
+    }
+  };
+  if (v.kind == Scalar::Tern && v.tern == Ternop::Fma) {
+    if (!is_self(*v.c) || reads_lhs(*v.a) || reads_lhs(*v.b)) return false;
+    *accum_out = Binop::Add;
+    return true;
+  }
+  if (v.kind == Scalar::Bin && (v.bin == Binop::Add || v.bin == Binop::Max || v.bin == Binop::Min)) {
+    if (is_self(*v.a) && !reads_lhs(*v.b)) { *accum_out = v.bin; return true; }
+    if (is_self(*v.b) && !reads_lhs(*v.a)) { *accum_out = v.bin; return true; }
+  }
+  (void)r;
+  return false;
+}
+
+void choose_coop(const Routine& r, Phase& ph, const PlanOptions& opt) {
+  ph.coop_lanes = 1;
+  if (!opt.enable_coop || ph.seq_syms.empty()) return;
+  Binop accum;
+  if (!reduction_shape(r, ph, &accum)) return;
+  const Stmt& set = *ph.inner[0];
+  const Prec p = r.node(set.node).prec;
+  if (!(p == Prec::Single || p == Prec::Double || p == Prec::Bfloat16 || p == Prec::Half)) return;
+  const int rc = ph.seq_syms.back();
+  const int64_t rext = ph.seq_to.back() - ph.seq_from.back() + 1;
+  int64_t P = 1, R = 1;
+  for (auto e : ph.par_ext) P *= e;
+  for (size_t i = 0; i < ph.seq_syms.size(); ++i) R *= ph.seq_to[i] - ph.seq_from[i] + 1;
+  // does the innermost sequential symbol walk some operand with unit stride?
+  std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+  scalar_accesses(*set.value, acc, f, d);
+  bool unit = false;
+  for (auto& a : acc) {
+    if (a.node == set.node) continue;
+    Strides st = strides_of(r, a.node, *a.idcs);
+    if (get_stride(st, rc) == 1) unit = true;
+  }
+  (void)w;
+  auto pow2_floor = [](int64_t x) { int64_t p2 = 1; while (p2 * 2 <= x) p2 *= 2; return p2; };
+  if (unit && rext >= 16) ph.coop_lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
+  else if (P < 16384 && R >= 256 && rext >= 2) ph.coop_lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
+}
+
+// Algorithmic bytes of a generic phase: every distinct (node, index tuple) read once, every
+// written element once; extents taken from the chain loops (inner loops count for reads).
+void account_bytes(const Routine& r, Phase& ph) {
+  std::map<int, int64_t> ext;
+  for (size_t i = 0; i < ph.par_syms.size(); ++i) ext[ph.par_syms[i]] = ph.par_ext[i];
+  for (size_t i = 0; i < ph.seq_syms.size(); ++i) ext[ph.seq_syms[i]] = ph.seq_to[i] - ph.seq_from[i] + 1;
+  std::function<void(const Block&)> inner_loops = [&](const Block& b) {
+    for (auto& s : b) {
+      if (s->kind == Stmt::For) { ext[s->sym] = s->to - s->from + 1; inner_loops(s->body); }
+      std::function<void(const Scalar&)> sc = [&](const Scalar& x) {
+        if (x.kind == Scalar::LocalScope) inner_loops(x.body);
+        if (x.a) sc(*x.a); if (x.b) sc(*x.b); if (x.c) sc(*x.c);
+      };
+      if (s->value) sc(*s->value);
+    }
+  };
+  inner_loops(ph.inner);
+  std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+  block_accesses(ph.inner, acc, w, f, d);
+  std::set<std::pair<int, std::string>> seen;
+  double bytes = 0;
+  for (auto& a : acc) {
+    std::set<int> syms;
+    std::string key = a.write ? "w" : "r";
+    for (auto& ix : *a.idcs) {
+      if (ix.kind == AxisIndex::Iter) { syms.insert(ix.sym); key += "i" + std::to_string(ix.sym); }
+      else if (ix.kind == AxisIndex::Affine) { for (auto& t : ix.terms) { syms.insert(t.second); key += "a" + std::to_string(t.second); } }
+      else key += "f" + std::to_string(ix.fixed);
+      key += ",";
+    }
+    if (!seen.insert({a.node, key}).second) continue;
+    double n = 1;
+    for (int s : syms) { auto it = ext.find(s); if (it != ext.end()) n *= (double)it->second; }
+    const Node& nd = r.node(a.node);
+    n = std::min(n, (double)nd.num_elems());
+    if (a.vec_len > 0) n *= a.vec_len;
+    bytes += n * prec_in_bytes(nd.prec);
+  }
+  ph.bytes = bytes;
+}
+
+Block strip_comments(const Block& b, std::string* last_comment) {
+  Block out;
+  for (auto& s : b) {
+    if (s->kind == Stmt::Comment) { if (last_comment) *last_comment = s->text; }
+    else out.push_back(s);
+  }
+  return out;
+}
+
+}  // namespace
+
+Plan make_plan(Routine& r, const PlanOptions& opt) {
+  Plan plan;
+  std::string label;
+  Block top = r.body;
+  for (size_t ti = 0; ti < top.size(); ++ti) {
+    StmtP sp = top[ti];
+    if (sp->kind == Stmt::Comment) { label = sp->text; continue; }
+    Phase ph;
+    ph.label = label;
+    ph.stmt = sp;
+    if (sp->kind == Stmt::ZeroOut) {
+      const Node& n = r.node(sp->node);
+      if (n.mode == Mode::Virtual) continue;
+      ph.kind = Phase::Fill;
+      ph.fill_node = sp->node;
+      ph.bytes = (double)n.size_in_bytes();
+      plan.phases.push_back(std::move(ph));
+      continue;
+    }
+    if (sp->kind == Stmt::DeclareLocal || sp->kind == Stmt::SetLocal)
+      throw InvalidArgument("hip backend: scalar locals at routine scope are not supported (routine " + r.name + ")");
+    // perfect-nest chain
+    std::vector<const Stmt*> chain;
+    Block inner;
+    if (sp->kind == Stmt::For) {
+      const Stmt* cur = sp.get();
+      for (;;) {
+        chain.push_back(cur);
+        Block body = strip_comments(cur->body, nullptr);
+        if (body.size() == 1 && body[0]->kind == Stmt::For) { cur = body[0].get(); continue; }
+        inner = body;
+        break;
+      }
+    } else {
+      inner = {sp};
+    }
+    std::vector<Access> acc;
+    bool whole = false, foreign = false;
+    std::set<ScopeId> declared;
+    block_accesses(inner, acc, whole, foreign, declared);
+    for (const Stmt* l : chain) {
+      const int64_t ext = l->to - l->from + 1;
+      if (ext <= 0) { chain.clear(); inner.clear(); break; }   // zero-trip loop: nothing runs
+    }
+    if (chain.empty() && inner.empty()) continue;
+    for (const Stmt* l : chain) {
+      const int64_t ext = l->to - l->from + 1;
+      const bool par = !whole && !foreign && symbol_is_parallel(l->sym, acc);
+      if (par) { ph.par_syms.push_back(l->sym); ph.par_from.push_back(l->from); ph.par_ext.push_back(ext); }
+      else { ph.seq_syms.push_back(l->sym); ph.seq_from.push_back(l->from); ph.seq_to.push_back(l->to); }
+    }
+    ph.inner = inner;
+
+    // fold a directly preceding Zero_out of the accumulation target into this phase when the nest
+    // overwrites the whole array: every axis is a full-range parallel iterator or has extent 1.
+    Binop accum;
+    if (!plan.phases.empty() && plan.phases.back().kind == Phase::Fill && reduction_shape(r, ph, &accum) &&
+        accum == Binop::Add && plan.phases.back().fill_node == inner[0]->node) {
+      const Stmt& set = *inner[0];
+      const Node& n = r.node(set.node);
+      bool full = true;
+      for (size_t p = 0; p < set.idcs.size() && full; ++p) {
+        const AxisIndex& a = set.idcs[p];
+        if (a.kind == AxisIndex::Fixed) full = n.dims[p] == 1;
+        else if (a.kind == AxisIndex::Iter) {
+          full = false;
+          for (size_t i = 0; i < ph.par_syms.size(); ++i)
+            if (ph.par_syms[i] == a.sym) full = ph.par_from[i] == 0 && ph.par_ext[i] == n.dims[p];
+        } else full = false;
+      }
+      if (full) { ph.fused_zero_init = true; plan.phases.pop_back(); }
+    }
+
+    if (!match_contraction(r, ph, opt)) {
+      ph.kind = Phase::Generic;
+      choose_coop(r, ph, opt);
+      account_bytes(r, ph);
+    } else {
+      const GemmDesc& g = ph.gemm;
+      auto op_bytes = [&](const GemmOperand& o, double rows, double cols) {
+        double n = rows * cols;
+        for (int i = 0; i < g.nbatch; ++i) if (o.s_batch[i]) n *= (double)g.batch_ext[i];
+        return n * prec_in_bytes(o.prec);
+      };
+      ph.bytes = op_bytes(g.a, (double)g.M, (double)g.K) + op_bytes(g.b, (double)g.N, (double)g.K) +
+                 op_bytes(g.c, (double)g.M, (double)g.N) * (g.accumulate ? 2 : 1);
+    }
+    plan.phases.push_back(std::move(ph));
+  }
+  return plan;
+}
+
+}  // namespace ocannl

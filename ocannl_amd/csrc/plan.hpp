@@ -1,0 +1,78 @@
+// Planner: splits a routine's loop nest into device kernels.
+//
+// The reference's GPU backends print the whole routine as ONE serial function run by one thread
+// (arrayjit/lib/cuda_backend.ml:359-360,1043).  Here every top-level statement of the routine
+// (arrayjit/lib/low_level.mli:22-51) becomes a *phase*; each phase is classified as
+//   * Fill         -- Zero_out of a node (c_syntax.ml:468-479)
+//   * Contraction  -- an accumulating `c[..] := fma(a[..], b[..], c[..])` nest
+//                     (arrayjit/lib/assignments.ml:431-432, low_level.ml:1631-1634) big enough for
+//                     the hand-written MFMA kernels
+//   * Generic      -- anything else: a generated kernel with one thread (or one cooperating lane
+//                     group) per point of the nest's parallel index space.
+#pragma once
+#include <string>
+#include <vector>
+
+#include "llir.hpp"
+
+namespace ocannl {
+
+// One strided operand of a contraction, in elements.
+struct GemmOperand {
+  int node = -1;
+  Prec prec = Prec::Single;
+  int64_t offset = 0;                                  // constant part of the element offset
+  std::vector<std::pair<int, int64_t>> static_terms;   // (static symbol, stride): added at launch
+  int64_t s_row = 0;     // stride along M (A, C) or N (B)
+  int64_t s_k = 0;       // stride along K (A, B); for C: stride along N
+  int64_t s_batch[3] = {0, 0, 0};
+};
+
+// C[batch, m, n] (+)= sum_k A[batch, m, k] * B[batch, n, k], all strides explicit.
+struct GemmDesc {
+  GemmOperand a, b, c;
+  int64_t M = 1, N = 1, K = 1;
+  int nbatch = 0;
+  int64_t batch_ext[3] = {1, 1, 1};
+  bool accumulate = false;   // beta = 1: add into existing C (gradient accumulation `=+`)
+  double flops() const {
+    double f = 2.0 * (double)M * (double)N * (double)K;
+    for (int i = 0; i < nbatch; ++i) f *= (double)batch_ext[i];
+    return f;
+  }
+};
+
+struct Phase {
+  enum Kind { Generic, Fill, Contraction } kind = Generic;
+  std::string label;          // human-readable, from the nearest preceding comment
+  // Generic
+  StmtP stmt;                 // the statement this phase runs
+  std::vector<int> par_syms;  // parallel loop symbols, slowest first
+  std::vector<int64_t> par_from, par_ext;
+  std::vector<int> seq_syms;  // chain symbols that stay sequential inside a thread, outer first
+  std::vector<int64_t> seq_from, seq_to;
+  Block inner;                // body below the perfect-nest chain
+  int coop_lanes = 1;         // >1: that many adjacent lanes share one output (tree-combined)
+  bool fused_zero_init = false;  // the preceding Zero_out of the target was folded in (beta = 0)
+  // Fill
+  int fill_node = -1;
+  // Contraction
+  GemmDesc gemm;
+  // accounting (algorithmic): distinct elements read + written, and flops
+  double bytes = 0, flops = 0;
+};
+
+struct PlanOptions {
+  int64_t min_mfma_flops = 1 << 22;   // below this a contraction stays a generic kernel
+  bool enable_mfma = true;
+  bool enable_coop = true;
+};
+
+struct Plan {
+  std::vector<Phase> phases;
+  std::vector<Node> scratch;   // nodes invented by the planner (de-virtualised contraction results)
+};
+
+Plan make_plan(Routine& r, const PlanOptions& opt);
+
+}  // namespace ocannl

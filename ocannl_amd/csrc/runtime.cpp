@@ -1,0 +1,681 @@
+// Runtime behind the C ABI: devices, the pool table, events, copies, hiprtc compilation, linking
+// and launching.  Mirrors the responsibilities of the reference CUDA backend
+// (arrayjit/lib/cuda_backend.ml) without sharing its structure: one HIP stream per device, slabs
+// from hipMalloc, kernels from hiprtc modules plus the precompiled MFMA kernels of this library.
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <cstring>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "../../include/ocannl_hip.h"
+#include "codegen.hpp"
+#include "gemm.hpp"
+#include "llir.hpp"
+#include "plan.hpp"
+
+using namespace ocannl;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+struct RuntimeError : std::runtime_error { using std::runtime_error::runtime_error; };
+
+void hip_check(hipError_t e, const char* what) {
+  if (e != hipSuccess) throw RuntimeError(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+}  // namespace
+
+struct ocannl_hip_device {
+  int ordinal = 0;
+  hipStream_t stream = nullptr;
+  std::map<int, std::pair<void*, uint64_t>> pools;   // pool_id -> (base, size)
+  uint64_t used = 0;
+  uint64_t scratch_used = 0;
+  int live_events = 0;
+  int live_routines = 0;
+  hipDeviceProp_t props{};
+  void make_current() const { hip_check(hipSetDevice(ordinal), "hipSetDevice"); }
+  void* resolve(int pool_id, uint64_t offset, uint64_t bytes, const char* what) const {
+    auto it = pools.find(pool_id);
+    if (it == pools.end()) throw InvalidArgument(std::string(what) + ": unknown pool_id " + std::to_string(pool_id));
+    if (offset + bytes > it->second.second)
+      throw InvalidArgument(std::string(what) + ": range [" + std::to_string(offset) + ", +" + std::to_string(bytes) +
+                            ") exceeds pool " + std::to_string(pool_id) + " of " + std::to_string(it->second.second) + " bytes");
+    return static_cast<char*>(it->second.first) + offset;
+  }
+};
+
+struct ocannl_hip_event {
+  hipEvent_t ev = nullptr;
+  ocannl_hip_device* dev = nullptr;
+};
+
+namespace {
+
+struct CompiledRoutine {
+  Routine r;
+  Plan plan;
+  GeneratedModule mod;
+  std::vector<char> binary;   // gfx950 code object of the generated kernels (empty if none)
+};
+
+std::mutex g_mu;
+bool g_inited = false;
+std::vector<std::unique_ptr<ocannl_hip_device>> g_devices;
+
+std::vector<char> hiprtc_compile(const std::string& src, const std::string& name) {
+  hiprtcProgram prog;
+  if (hiprtcCreateProgram(&prog, src.c_str(), (name + ".hip").c_str(), 0, nullptr, nullptr) != HIPRTC_SUCCESS)
+    throw RuntimeError("hiprtcCreateProgram failed");
+  // No packed-FP32 instructions: they are generated from ordinary float code at -O3 otherwise.
+  const char* opts[] = {"--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                        "-ffp-contract=off"};
+  hiprtcResult rc = hiprtcCompileProgram(prog, (int)(sizeof opts / sizeof *opts), opts);
+  if (rc != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    hiprtcGetProgramLogSize(prog, &n);
+    std::string log(n, '\0');
+    if (n) hiprtcGetProgramLog(prog, &log[0]);
+    hiprtcDestroyProgram(&prog);
+    // mirrors Cc_backend's "generated code failed to compile" (arrayjit/lib/cc_backend.ml:105-117)
+    throw InvalidArgument("hip backend: generated code for " + name + " failed to compile (" +
+                          hiprtcGetErrorString(rc) + ")\n" + log);
+  }
+  size_t n = 0;
+  hiprtcGetCodeSize(prog, &n);
+  std::vector<char> bin(n);
+  hiprtcGetCode(prog, bin.data());
+  hiprtcDestroyProgram(&prog);
+  return bin;
+}
+
+PlanOptions parse_options(const char* options) {
+  PlanOptions o;
+  if (!options) return o;
+  std::stringstream ss(options);
+  std::string kv;
+  while (std::getline(ss, kv, ';')) {
+    if (kv.empty()) continue;
+    auto eq = kv.find('=');
+    if (eq == std::string::npos) throw InvalidArgument("compile options: expected key=value, got '" + kv + "'");
+    const std::string k = kv.substr(0, eq), v = kv.substr(eq + 1);
+    if (k == "mfma") o.enable_mfma = v != "0";
+    else if (k == "coop") o.enable_coop = v != "0";
+    else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
+    else throw InvalidArgument("compile options: unknown key '" + k + "'");
+  }
+  return o;
+}
+
+}  // namespace
+
+struct ocannl_hip_code {
+  std::vector<CompiledRoutine> routines;
+};
+
+struct ocannl_hip_routine {
+  ocannl_hip_device* dev = nullptr;
+  const CompiledRoutine* code = nullptr;
+  std::shared_ptr<void> keep_code;   // context_lifetime: keeps module + code alive (cuda_backend.ml:1046-1051)
+  hipModule_t module = nullptr;
+  void* scratch = nullptr;
+  uint64_t scratch_bytes = 0;
+  std::map<int, void*> node_ptr;
+  std::map<int, int64_t> statics;    // symbol -> current value
+  struct Launch {
+    int phase;
+    hipFunction_t fn = nullptr;
+    std::vector<void*> ptr_vals;       // storage for pointer arguments
+    std::vector<uint32_t> idx_vals;    // storage for static-index arguments
+    std::vector<int> idx_syms;
+    std::vector<void*> args;
+    unsigned grid = 1, block = 256;
+    void* fill_ptr = nullptr; uint64_t fill_bytes = 0;
+  };
+  std::vector<Launch> launches;
+  std::vector<hipEvent_t> timing_events;
+};
+
+namespace {
+
+template <class F>
+int guarded(F&& f) {
+  try {
+    f();
+    return OCANNL_HIP_OK;
+  } catch (const UserError& e) { g_last_error = e.what(); return OCANNL_HIP_E_USER;
+  } catch (const InvalidArgument& e) { g_last_error = e.what(); return OCANNL_HIP_E_INVALID;
+  } catch (const std::exception& e) { g_last_error = e.what(); return OCANNL_HIP_E_RUNTIME; }
+}
+
+void copy_out(const std::string& s, char* buf, size_t cap) {
+  if (!buf || cap == 0) throw InvalidArgument("output buffer is null");
+  const size_t n = std::min(s.size(), cap - 1);
+  std::memcpy(buf, s.data(), n);
+  buf[n] = '\0';
+}
+
+void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
+  ocannl_hip_device& dev = *rt.dev;
+  dev.make_current();
+  const Routine& r = rt.code->r;
+  // static indices: range check, then publish (cuda_backend.ml:1015-1030)
+  for (auto& s : r.statics) {
+    const int64_t v = rt.statics[s.sym];
+    if (v < 0)
+      throw UserError("hip backend: static index " + sym_ident(s.sym) + " is negative: " + std::to_string(v));
+    if (s.range >= 0 && v >= s.range)
+      throw UserError("hip backend: static index " + sym_ident(s.sym) + " is too big: " + std::to_string(v) +
+                      " (range 0.." + std::to_string(s.range - 1) + ")");
+  }
+  const bool timed = kernel_ms != nullptr;
+  if (timed) {
+    if (cap < (int)rt.launches.size()) throw InvalidArgument("run_timed: kernel_ms too small");
+    while (rt.timing_events.size() < rt.launches.size() + 1) {
+      hipEvent_t e;
+      hip_check(hipEventCreate(&e), "hipEventCreate");
+      rt.timing_events.push_back(e);
+    }
+    hip_check(hipEventRecord(rt.timing_events[0], dev.stream), "hipEventRecord");
+  }
+  for (size_t li = 0; li < rt.launches.size(); ++li) {
+    auto& l = rt.launches[li];
+    const Phase& ph = rt.code->plan.phases[l.phase];
+    if (ph.kind == Phase::Fill) {
+      hip_check(hipMemsetAsync(l.fill_ptr, 0, l.fill_bytes, dev.stream), "hipMemsetAsync");
+    } else if (ph.kind == Phase::Generic) {
+      for (size_t i = 0; i < l.idx_syms.size(); ++i) l.idx_vals[i] = (uint32_t)rt.statics[l.idx_syms[i]];
+      hip_check(hipModuleLaunchKernel(l.fn, l.grid, 1, 1, l.block, 1, 1, 0, dev.stream, l.args.data(), nullptr),
+                "hipModuleLaunchKernel");
+    } else {
+      const GemmDesc& g = ph.gemm;
+      auto base = [&](const GemmOperand& o) -> char* {
+        int64_t off = o.offset;
+        for (auto& t : o.static_terms) off += rt.statics[t.first] * t.second;
+        return static_cast<char*>(rt.node_ptr.at(o.node)) + off * prec_in_bytes(o.prec);
+      };
+      GemmArgs a{};
+      a.a = base(g.a); a.b = base(g.b); a.c = base(g.c);
+      a.M = g.M; a.N = g.N; a.K = g.K;
+      a.a_row = g.a.s_row; a.a_k = g.a.s_k; a.b_row = g.b.s_row; a.b_k = g.b.s_k; a.c_row = g.c.s_row;
+      a.nbatch = g.nbatch;
+      for (int i = 0; i < 3; ++i) {
+        a.batch_ext[i] = g.batch_ext[i];
+        a.a_batch[i] = g.a.s_batch[i]; a.b_batch[i] = g.b.s_batch[i]; a.c_batch[i] = g.c.s_batch[i];
+      }
+      a.accumulate = g.accumulate ? 1 : 0;
+      a.c_is_bf16 = g.c.prec == Prec::Bfloat16;
+      hip_check(launch_gemm(g, a, dev.stream), "launch_gemm");
+    }
+    if (timed) hip_check(hipEventRecord(rt.timing_events[li + 1], dev.stream), "hipEventRecord");
+  }
+  if (timed) {
+    hip_check(hipStreamSynchronize(dev.stream), "hipStreamSynchronize");
+    for (size_t li = 0; li < rt.launches.size(); ++li)
+      hip_check(hipEventElapsedTime(&kernel_ms[li], rt.timing_events[li], rt.timing_events[li + 1]), "hipEventElapsedTime");
+  }
+}
+
+}  // namespace
+
+// ================================================================================================
+extern "C" {
+
+const char* ocannl_hip_last_error(void) { return g_last_error.c_str(); }
+
+int ocannl_hip_init(void) {
+  return guarded([] {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_inited) return;
+    hip_check(hipInit(0), "hipInit");
+    int n = 0;
+    hip_check(hipGetDeviceCount(&n), "hipGetDeviceCount");
+    g_devices.resize(n);
+    g_inited = true;
+  });
+}
+
+int ocannl_hip_num_devices(int* count) {
+  return guarded([&] {
+    if (!count) throw InvalidArgument("num_devices: null output");
+    if (!g_inited) { int rc = ocannl_hip_init(); if (rc) throw RuntimeError(g_last_error); }
+    *count = (int)g_devices.size();
+  });
+}
+
+int ocannl_hip_get_device(int ordinal, ocannl_hip_device** out) {
+  return guarded([&] {
+    if (!out) throw InvalidArgument("get_device: null output");
+    if (!g_inited) { int rc = ocannl_hip_init(); if (rc) throw RuntimeError(g_last_error); }
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (ordinal < 0 || ordinal >= (int)g_devices.size())
+      throw InvalidArgument("get_device: ordinal " + std::to_string(ordinal) + " out of range (" +
+                            std::to_string(g_devices.size()) + " devices)");
+    if (!g_devices[ordinal]) {
+      auto d = std::make_unique<ocannl_hip_device>();
+      d->ordinal = ordinal;
+      d->make_current();
+      hip_check(hipGetDeviceProperties(&d->props, ordinal), "hipGetDeviceProperties");
+      if (std::string(d->props.gcnArchName).rfind("gfx950", 0) != 0)
+        throw RuntimeError(std::string("hip backend: device is ") + d->props.gcnArchName + ", this library is built for gfx950 only");
+      hip_check(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+      g_devices[ordinal] = std::move(d);
+    }
+    *out = g_devices[ordinal].get();
+  });
+}
+
+int ocannl_hip_get_name(ocannl_hip_device* dev, char* buf, size_t cap) {
+  return guarded([&] {
+    if (!dev) throw InvalidArgument("get_name: null device");
+    copy_out("hip:" + std::to_string(dev->ordinal), buf, cap);
+  });
+}
+
+int ocannl_hip_static_properties(char* buf, size_t cap) {
+  return guarded([&] {
+    if (!g_inited) { int rc = ocannl_hip_init(); if (rc) throw RuntimeError(g_last_error); }
+    std::ostringstream s;
+    s << "(";
+    for (size_t i = 0; i < g_devices.size(); ++i) {
+      hipDeviceProp_t p;
+      hip_check(hipGetDeviceProperties(&p, (int)i), "hipGetDeviceProperties");
+      s << "((device " << i << ") (name \"" << p.name << "\") (arch " << p.gcnArchName << ") (total_global_mem "
+        << p.totalGlobalMem << ") (multiprocessor_count " << p.multiProcessorCount << ") (warp_size " << p.warpSize
+        << ") (max_shared_memory_per_block " << p.sharedMemPerBlock << ") (clock_rate_khz " << p.clockRate
+        << ") (memory_clock_rate_khz " << p.memoryClockRate << ") (memory_bus_width " << p.memoryBusWidth
+        << ") (l2_cache_size " << p.l2CacheSize << "))";
+    }
+    s << ")";
+    copy_out(s.str(), buf, cap);
+  });
+}
+
+int ocannl_hip_get_used_memory(ocannl_hip_device* dev, uint64_t* bytes) {
+  return guarded([&] {
+    if (!dev || !bytes) throw InvalidArgument("get_used_memory: null argument");
+    *bytes = dev->used + dev->scratch_used;
+  });
+}
+
+int ocannl_hip_get_debug_info(ocannl_hip_device* dev, char* buf, size_t cap) {
+  return guarded([&] {
+    if (!dev) throw InvalidArgument("get_debug_info: null device");
+    std::ostringstream s;
+    s << "((pools " << dev->pools.size() << ") (pool_bytes " << dev->used << ") (scratch_bytes " << dev->scratch_used
+      << ") (live_events " << dev->live_events << ") (live_routines " << dev->live_routines << "))";
+    copy_out(s.str(), buf, cap);
+  });
+}
+
+int ocannl_hip_await(ocannl_hip_device* dev) {
+  return guarded([&] {
+    if (!dev) throw InvalidArgument("await: null device");
+    dev->make_current();
+    hip_check(hipStreamSynchronize(dev->stream), "hipStreamSynchronize");
+  });
+}
+
+int ocannl_hip_is_idle(ocannl_hip_device* dev, int* idle) {
+  return guarded([&] {
+    if (!dev || !idle) throw InvalidArgument("is_idle: null argument");
+    dev->make_current();
+    hipError_t e = hipStreamQuery(dev->stream);
+    if (e == hipSuccess) *idle = 1;
+    else if (e == hipErrorNotReady) *idle = 0;
+    else hip_check(e, "hipStreamQuery");
+  });
+}
+
+int ocannl_hip_all_work(ocannl_hip_device* dev, ocannl_hip_event** out) {
+  return guarded([&] {
+    if (!dev || !out) throw InvalidArgument("all_work: null argument");
+    dev->make_current();
+    auto ev = std::make_unique<ocannl_hip_event>();
+    ev->dev = dev;
+    hip_check(hipEventCreateWithFlags(&ev->ev, hipEventDisableTiming), "hipEventCreateWithFlags");
+    hip_check(hipEventRecord(ev->ev, dev->stream), "hipEventRecord");
+    dev->live_events++;
+    *out = ev.release();
+  });
+}
+
+int ocannl_hip_sync(ocannl_hip_event* ev) {
+  return guarded([&] {
+    if (!ev) throw InvalidArgument("sync: null event");
+    ev->dev->make_current();
+    hip_check(hipEventSynchronize(ev->ev), "hipEventSynchronize");
+  });
+}
+
+int ocannl_hip_is_done(ocannl_hip_event* ev, int* done) {
+  return guarded([&] {
+    if (!ev || !done) throw InvalidArgument("is_done: null argument");
+    ev->dev->make_current();
+    hipError_t e = hipEventQuery(ev->ev);
+    if (e == hipSuccess) *done = 1;
+    else if (e == hipErrorNotReady) *done = 0;
+    else hip_check(e, "hipEventQuery");
+  });
+}
+
+int ocannl_hip_will_wait_for(ocannl_hip_device* dev, ocannl_hip_event* ev) {
+  return guarded([&] {
+    if (!dev || !ev) throw InvalidArgument("will_wait_for: null argument");
+    dev->make_current();
+    hip_check(hipStreamWaitEvent(dev->stream, ev->ev, 0), "hipStreamWaitEvent");
+  });
+}
+
+void ocannl_hip_event_free(ocannl_hip_event* ev) {
+  if (!ev) return;
+  if (ev->ev) (void)hipEventDestroy(ev->ev);
+  ev->dev->live_events--;
+  delete ev;
+}
+
+int ocannl_hip_alloc_pool(ocannl_hip_device* dev, int pool_id, uint64_t size, uint64_t alignment) {
+  return guarded([&] {
+    if (!dev) throw InvalidArgument("alloc_pool: null device");
+    if (alignment > 256) throw InvalidArgument("alloc_pool: alignment above 256 bytes is not supported");
+    dev->make_current();
+    auto it = dev->pools.find(pool_id);
+    if (it != dev->pools.end()) {   // regrowth: release the old slab first
+      hip_check(hipStreamSynchronize(dev->stream), "hipStreamSynchronize");
+      hip_check(hipFree(it->second.first), "hipFree");
+      dev->used -= it->second.second;
+      dev->pools.erase(it);
+    }
+    void* p = nullptr;
+    hip_check(hipMalloc(&p, size ? size : 1), "hipMalloc");
+    dev->pools[pool_id] = {p, size};
+    dev->used += size;
+  });
+}
+
+int ocannl_hip_free_pool(ocannl_hip_device* dev, int pool_id) {
+  return guarded([&] {
+    if (!dev) throw InvalidArgument("free_pool: null device");
+    auto it = dev->pools.find(pool_id);
+    if (it == dev->pools.end()) throw InvalidArgument("free_pool: unknown pool_id " + std::to_string(pool_id));
+    dev->make_current();
+    hip_check(hipStreamSynchronize(dev->stream), "hipStreamSynchronize");
+    hip_check(hipFree(it->second.first), "hipFree");
+    dev->used -= it->second.second;
+    dev->pools.erase(it);
+  });
+}
+
+int ocannl_hip_memset_zero(ocannl_hip_device* dev, int pool_id, uint64_t offset, uint64_t size) {
+  return guarded([&] {
+    if (!dev) throw InvalidArgument("memset_zero: null device");
+    dev->make_current();
+    void* p = dev->resolve(pool_id, offset, size, "memset_zero");
+    if (size) hip_check(hipMemsetAsync(p, 0, size, dev->stream), "hipMemsetAsync");
+  });
+}
+
+int ocannl_hip_from_host(ocannl_hip_device* dev, int pool_id, uint64_t offset, const void* src, uint64_t bytes) {
+  return guarded([&] {
+    if (!dev || (!src && bytes)) throw InvalidArgument("from_host: null argument");
+    dev->make_current();
+    void* p = dev->resolve(pool_id, offset, bytes, "from_host");
+    if (bytes) hip_check(hipMemcpyAsync(p, src, bytes, hipMemcpyHostToDevice, dev->stream), "hipMemcpyAsync(H2D)");
+  });
+}
+
+int ocannl_hip_to_host(ocannl_hip_device* dev, int pool_id, uint64_t offset, void* dst, uint64_t bytes) {
+  return guarded([&] {
+    if (!dev || (!dst && bytes)) throw InvalidArgument("to_host: null argument");
+    dev->make_current();
+    void* p = dev->resolve(pool_id, offset, bytes, "to_host");
+    if (bytes) hip_check(hipMemcpyAsync(dst, p, bytes, hipMemcpyDeviceToHost, dev->stream), "hipMemcpyAsync(D2H)");
+  });
+}
+
+int ocannl_hip_device_to_device(ocannl_hip_device* dst, int dst_pool, uint64_t dst_off, ocannl_hip_device* src,
+                                int src_pool, uint64_t src_off, uint64_t bytes) {
+  return guarded([&] {
+    if (!dst || !src) throw InvalidArgument("device_to_device: null device");
+    if (dst_pool < 0) {   // into the merge buffer = pool 0, grown on demand
+      auto it = dst->pools.find(0);
+      if (it == dst->pools.end() || it->second.second < bytes) {
+        int rc = ocannl_hip_alloc_pool(dst, 0, bytes, 256);
+        if (rc) throw RuntimeError(g_last_error);
+      }
+      dst_pool = 0; dst_off = 0;
+    }
+    void* d = dst->resolve(dst_pool, dst_off, bytes, "device_to_device(dst)");
+    void* s = src->resolve(src_pool, src_off, bytes, "device_to_device(src)");
+    dst->make_current();
+    if (dst->ordinal == src->ordinal) {
+      if (d == s) return;
+      hip_check(hipMemcpyAsync(d, s, bytes, hipMemcpyDeviceToDevice, dst->stream), "hipMemcpyAsync(D2D)");
+    } else {
+      hip_check(hipMemcpyPeerAsync(d, dst->ordinal, s, src->ordinal, bytes, dst->stream), "hipMemcpyPeerAsync");
+    }
+  });
+}
+
+int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, ocannl_hip_code** out) {
+  return guarded([&] {
+    if (!llir || !out) throw InvalidArgument("compile: null argument");
+    PlanOptions opt = parse_options(options);
+    auto code = std::make_unique<ocannl_hip_code>();
+    std::vector<Routine> rs = parse_routines(llir, len);
+    for (auto& r : rs) {
+      CompiledRoutine cr;
+      cr.r = std::move(r);
+      cr.plan = make_plan(cr.r, opt);
+      cr.mod = generate_module(cr.r, cr.plan);
+      if (!cr.mod.kernels.empty()) cr.binary = hiprtc_compile(cr.mod.source, cr.r.name);
+      code->routines.push_back(std::move(cr));
+    }
+    *out = code.release();
+  });
+}
+
+int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** out) {
+  return ocannl_hip_compile_opts(llir, len, nullptr, out);
+}
+
+void ocannl_hip_code_free(ocannl_hip_code* code) { delete code; }
+
+static const CompiledRoutine& routine_at(ocannl_hip_code* code, int index) {
+  if (!code) throw InvalidArgument("null code");
+  if (index < 0 || index >= (int)code->routines.size()) throw InvalidArgument("routine index out of range");
+  return code->routines[index];
+}
+
+int ocannl_hip_code_num_routines(ocannl_hip_code* code, int* n) {
+  return guarded([&] { if (!code || !n) throw InvalidArgument("null argument"); *n = (int)code->routines.size(); });
+}
+
+int ocannl_hip_code_routine_name(ocannl_hip_code* code, int index, char* buf, size_t cap) {
+  return guarded([&] { copy_out(routine_at(code, index).r.name, buf, cap); });
+}
+
+int ocannl_hip_code_kparams(ocannl_hip_code* code, int index, ocannl_hip_kparam* params, int cap, int* count) {
+  return guarded([&] {
+    const CompiledRoutine& cr = routine_at(code, index);
+    std::vector<ocannl_hip_kparam> ks;
+    if (cr.r.merge_node >= 0) ks.push_back({2, cr.r.merge_node, cr.r.node(cr.r.merge_node).size_in_bytes()});
+    for (auto& s : cr.r.statics) ks.push_back({1, s.sym, s.range});
+    for (int id : cr.r.node_order) {
+      const Node& n = cr.r.node(id);
+      if (n.mode == Mode::Ctx) ks.push_back({0, id, n.size_in_bytes()});
+    }
+    if (count) *count = (int)ks.size();
+    if (params) {
+      if (cap < (int)ks.size()) throw InvalidArgument("kparams: buffer too small");
+      std::copy(ks.begin(), ks.end(), params);
+    }
+  });
+}
+
+int ocannl_hip_code_source(ocannl_hip_code* code, char* buf, size_t cap, size_t* needed) {
+  return guarded([&] {
+    if (!code) throw InvalidArgument("null code");
+    std::string all;
+    for (auto& cr : code->routines) all += cr.mod.source;
+    if (needed) *needed = all.size() + 1;
+    if (buf) copy_out(all, buf, cap);
+  });
+}
+
+int ocannl_hip_code_num_kernels(ocannl_hip_code* code, int index, int* n) {
+  return guarded([&] { if (!n) throw InvalidArgument("null argument"); *n = (int)routine_at(code, index).plan.phases.size(); });
+}
+
+int ocannl_hip_code_kernel_info(ocannl_hip_code* code, int index, int kernel, ocannl_hip_kernel_info* info) {
+  return guarded([&] {
+    const CompiledRoutine& cr = routine_at(code, index);
+    if (!info || kernel < 0 || kernel >= (int)cr.plan.phases.size()) throw InvalidArgument("kernel index out of range");
+    const Phase& ph = cr.plan.phases[kernel];
+    std::memset(info, 0, sizeof *info);
+    info->kind = ph.kind == Phase::Generic ? 0 : ph.kind == Phase::Fill ? 1 : 2;
+    info->coop_lanes = ph.coop_lanes;
+    info->flops = ph.flops;
+    info->bytes = ph.bytes;
+    std::string name;
+    if (ph.kind == Phase::Contraction) {
+      info->m = ph.gemm.M; info->n = ph.gemm.N; info->k = ph.gemm.K;
+      info->batch = 1;
+      for (int i = 0; i < ph.gemm.nbatch; ++i) info->batch *= ph.gemm.batch_ext[i];
+      name = gemm_kernel_name(ph.gemm);
+    } else if (ph.kind == Phase::Fill) {
+      name = "fill_zero:" + cr.r.node(ph.fill_node).ident;
+    } else {
+      for (auto& k : cr.mod.kernels) if (k.phase_index == kernel) name = k.name;
+    }
+    copy_out(name, info->name, sizeof info->name);
+  });
+}
+
+int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, const ocannl_hip_node_loc* locs, int n_locs,
+                    ocannl_hip_routine** out) {
+  return guarded([&] {
+    if (!dev || !out) throw InvalidArgument("link: null argument");
+    const CompiledRoutine& cr = routine_at(code, index);
+    if (n_locs > 0 && !locs) throw InvalidArgument("link: null locs");
+    dev->make_current();
+    auto rt = std::make_unique<ocannl_hip_routine>();
+    rt->dev = dev;
+    rt->code = &cr;
+    if (cr.r.merge_node >= 0) throw UserError("hip backend: merge-buffer routines need a second device and are not supported");
+    // ctx nodes from the caller's table
+    std::map<int, const ocannl_hip_node_loc*> by_id;
+    for (int i = 0; i < n_locs; ++i) by_id[locs[i].node_id] = &locs[i];
+    // local nodes (and planner scratch): one private arena, 256-byte aligned sub-buffers
+    uint64_t arena = 0;
+    std::map<int, uint64_t> local_off;
+    for (auto& kv : cr.r.nodes) {
+      const Node& n = kv.second;
+      if (n.mode != Mode::Local) continue;
+      local_off[n.id] = arena;
+      arena += ((uint64_t)n.size_in_bytes() + 255) / 256 * 256;
+    }
+    if (arena) {
+      hip_check(hipMalloc(&rt->scratch, arena), "hipMalloc(scratch)");
+      rt->scratch_bytes = arena;
+      dev->scratch_used += arena;
+    }
+    for (auto& kv : cr.r.nodes) {
+      const Node& n = kv.second;
+      if (n.mode == Mode::Virtual) continue;
+      if (n.mode == Mode::Local) { rt->node_ptr[n.id] = static_cast<char*>(rt->scratch) + local_off[n.id]; continue; }
+      auto it = by_id.find(n.id);
+      if (it == by_id.end())
+        throw UserError("hip backend link: node " + n.ident + " (id " + std::to_string(n.id) + ") missing from context");
+      rt->node_ptr[n.id] = dev->resolve(it->second->pool_id, it->second->offset, (uint64_t)n.size_in_bytes(), "link");
+    }
+    for (auto& s : cr.r.statics) rt->statics[s.sym] = 0;
+    if (!cr.binary.empty()) hip_check(hipModuleLoadData(&rt->module, cr.binary.data()), "hipModuleLoadData");
+    // launch records
+    size_t next_generic = 0;
+    for (size_t pi = 0; pi < cr.plan.phases.size(); ++pi) {
+      const Phase& ph = cr.plan.phases[pi];
+      ocannl_hip_routine::Launch l;
+      l.phase = (int)pi;
+      if (ph.kind == Phase::Fill) {
+        l.fill_ptr = rt->node_ptr.at(ph.fill_node);
+        l.fill_bytes = (uint64_t)cr.r.node(ph.fill_node).size_in_bytes();
+      } else if (ph.kind == Phase::Generic) {
+        const GeneratedKernel& gk = cr.mod.kernels.at(next_generic++);
+        if (gk.phase_index != (int)pi) throw InvalidArgument("link: kernel table out of step with the plan");
+        hip_check(hipModuleGetFunction(&l.fn, rt->module, gk.name.c_str()), "hipModuleGetFunction");
+        const uint64_t blocks = (gk.threads + gk.block - 1) / gk.block;
+        if (blocks == 0 || blocks > 0x7FFFFFFFull) throw UserError("hip backend: phase too large for one launch: " + gk.name);
+        l.grid = (unsigned)blocks;
+        l.block = (unsigned)gk.block;
+        size_t np = 0, ni = 0;
+        for (auto& p : gk.params) (p.kind == KernelParam::NodePtr ? np : ni)++;
+        l.ptr_vals.reserve(np); l.idx_vals.reserve(ni);
+        for (auto& p : gk.params) {
+          if (p.kind == KernelParam::NodePtr) { l.ptr_vals.push_back(rt->node_ptr.at(p.id)); }
+          else { l.idx_vals.push_back(0); l.idx_syms.push_back(p.id); }
+        }
+        size_t ip = 0, ii = 0;
+        for (auto& p : gk.params) {
+          if (p.kind == KernelParam::NodePtr) l.args.push_back(&l.ptr_vals[ip++]);
+          else l.args.push_back(&l.idx_vals[ii++]);
+        }
+      }
+      rt->launches.push_back(std::move(l));
+    }
+    // argument storage moved with the Launch objects: rebuild the pointers into it
+    for (auto& l : rt->launches) {
+      if (l.args.empty()) continue;
+      const GeneratedKernel* gk = nullptr;
+      for (auto& k : cr.mod.kernels) if (k.phase_index == l.phase) gk = &k;
+      size_t ip = 0, ii = 0, ai = 0;
+      for (auto& p : gk->params) l.args[ai++] = p.kind == KernelParam::NodePtr ? (void*)&l.ptr_vals[ip++] : (void*)&l.idx_vals[ii++];
+    }
+    dev->live_routines++;
+    *out = rt.release();
+  });
+}
+
+void ocannl_hip_routine_free(ocannl_hip_routine* rt) {
+  if (!rt) return;
+  (void)hipSetDevice(rt->dev->ordinal);
+  (void)hipStreamSynchronize(rt->dev->stream);
+  for (auto e : rt->timing_events) (void)hipEventDestroy(e);
+  if (rt->module) (void)hipModuleUnload(rt->module);
+  if (rt->scratch) { (void)hipFree(rt->scratch); rt->dev->scratch_used -= rt->scratch_bytes; }
+  rt->dev->live_routines--;
+  delete rt;
+}
+
+int ocannl_hip_routine_set_static(ocannl_hip_routine* rt, int symbol, int64_t value) {
+  return guarded([&] {
+    if (!rt) throw InvalidArgument("set_static: null routine");
+    auto it = rt->statics.find(symbol);
+    if (it == rt->statics.end()) throw InvalidArgument("set_static: routine has no static index " + sym_ident(symbol));
+    it->second = value;
+  });
+}
+
+int ocannl_hip_routine_run(ocannl_hip_routine* rt) {
+  return guarded([&] {
+    if (!rt) throw InvalidArgument("run: null routine");
+    enqueue(*rt, nullptr, 0);
+  });
+}
+
+int ocannl_hip_routine_run_timed(ocannl_hip_routine* rt, float* kernel_ms, int cap) {
+  return guarded([&] {
+    if (!rt || !kernel_ms) throw InvalidArgument("run_timed: null argument");
+    enqueue(*rt, kernel_ms, cap);
+  });
+}
+
+}  // extern "C"

@@ -1,0 +1,100 @@
+"""GPU parity tests: the HIP library (through the C ABI) against the CPU checker on identical
+seeded inputs.  Tolerances follow the stated bar: fp32 within 1e-4 relative, bf16 within 2e-2,
+loss curves over 100 steps within 1e-3."""
+import numpy as np
+import pytest
+
+from ocannl_amd import llir as L
+from ocannl_amd import workloads as W
+from parity import HipRun, OracleRun, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _small_contraction():
+    L.reset_symbols(0)
+    a = L.Node(1, "a", "single", (3, 5)); b = L.Node(2, "b", "single", (5, 4)); c = L.Node(3, "c", "single", (4, 3))
+    d = L.Node(4, "d", "single", (4, 3))
+    i, j, k = L.fresh_symbol(), L.fresh_symbol(), L.fresh_symbol()
+    sc = L.Scope(L.Node(9, "n2", "single", (1,), mode="virtual"), 1)
+    body = [
+        L.Comment("c fwd"),
+        L.For(i, 0, 3, [L.For(j, 0, 2, [L.Set(c, (L.It(i), L.It(j)), L.Unop("relu", L.LocalScope(sc, [
+            L.SetLocal(sc, L.Const(0.0)),
+            L.For(k, 0, 4, [L.SetLocal(sc, L.Ternop("fma", L.Get(a, (L.It(j), L.It(k))), L.Get(b, (L.It(k), L.It(i))),
+                                                    L.GetLocal(sc)))])])))])]),
+        L.ZeroOut(d),
+        L.For(i, 0, 3, [L.For(j, 0, 2, [L.For(k, 0, 4, [L.Set(d, (L.It(i), L.It(j)), L.Ternop(
+            "fma", L.Get(a, (L.It(j), L.It(k))), L.Get(b, (L.It(k), L.It(i))), L.Get(d, (L.It(i), L.It(j)))))])])]),
+    ]
+    return L.Routine("c_fwd", body), (a, b, c, d)
+
+
+def test_small_contraction_bit_exact():
+    # the generated kernels keep the reference's sequential summation order: fp32 bit equality
+    r, (a, b, c, d) = _small_contraction()
+    rng = np.random.default_rng(0)
+    init = {1: rng.standard_normal((3, 5)).astype(np.float32), 2: rng.standard_normal((5, 4)).astype(np.float32)}
+    hip, ora = HipRun(r, init), OracleRun(r, init)
+    hip.step(); ora.step()
+    for n in (c, d):
+        assert np.array_equal(hip.get(n).view(np.uint32), ora.get(n).view(np.uint32))
+    hip.close()
+
+
+@pytest.mark.parametrize("inline", [True, False])
+def test_moons_mlp_loss_curve(inline):
+    w = W.moons_mlp(inline=inline)
+    sym = w.statics["batch_n"].sym
+    hip, ora = HipRun(w.routine, w.init), OracleRun(w.routine, w.init)
+    lh, lo = [], []
+    for step in range(100):
+        st = {sym: step % w.statics["batch_n"].range}
+        hip.step(st); ora.step(st)
+        lh.append(float(hip.get(w.nodes["loss"])[0])); lo.append(float(ora.get(w.nodes["loss"])[0]))
+    lh, lo = np.array(lh), np.array(lo)
+    assert np.max(np.abs(lh - lo)) <= 1e-3, (lh[:5], lo[:5])
+    for name in ("w1", "b1", "w2", "b2", "w3"):
+        assert rel_err(hip.get(w.nodes[name]), ora.get(w.nodes[name]), "single") <= 1e-3, name
+    hip.close()
+
+
+def test_static_index_range_is_checked():
+    from ocannl_amd import backend as B
+    w = W.moons_mlp()
+    hip = HipRun(w.routine, w.init)
+    with pytest.raises(B.User_error):
+        hip.step({w.statics["batch_n"].sym: w.statics["batch_n"].range})
+    with pytest.raises(B.User_error):
+        hip.step({w.statics["batch_n"].sym: -1})
+    hip.close()
+
+
+@pytest.mark.parametrize("prec,out_prec,tol", [("single", "single", 1e-4), ("bfloat16", "single", 2e-2),
+                                                ("bfloat16", "bfloat16", 2e-2)])
+@pytest.mark.parametrize("order", ["last", "first"])
+def test_dense_contraction_mfma_small(prec, out_prec, tol, order):
+    w = W.dense_contraction(b=256, i=192, o=128, prec=prec, out_prec=out_prec, reduce_order=order)
+    rng = np.random.default_rng(5)
+    # gradients accumulate into existing contents
+    w.init[w.nodes["dx"].id] = W.as_prec(rng.standard_normal((256, 192)).astype(np.float32), out_prec)
+    w.init[w.nodes["dw"].id] = W.as_prec(rng.standard_normal((128, 192)).astype(np.float32), out_prec)
+    hip = HipRun(w.routine, w.init, options="min_mfma_flops=1")
+    kinds = [k["kind"] for k in hip.code.kernels()]
+    assert kinds.count("mfma") == 3, hip.code.kernels()
+    ora = OracleRun(w.routine, w.init)
+    hip.step(); ora.step()
+    for name in ("y", "dx", "dw"):
+        got, want = hip.get(w.nodes[name]), ora.get(w.nodes[name])
+        if out_prec == "bfloat16":
+            # the checker rounds the running sum to bf16 after every step; compare both to fp64
+            x = W.to_float(w.init[w.nodes["x"].id], prec); wt = W.to_float(w.init[w.nodes["w"].id], prec)
+            dy = W.to_float(w.init[w.nodes["dy"].id], prec)
+            exact = {"y": x @ wt.T, "dx": W.to_float(w.init[w.nodes["dx"].id], out_prec) + dy @ wt,
+                     "dw": W.to_float(w.init[w.nodes["dw"].id], out_prec) + dy.T @ x}[name]
+            scale = np.max(np.abs(exact))
+            assert np.max(np.abs(W.to_float(got, out_prec) - exact)) / scale <= tol, name
+            assert np.max(np.abs(W.to_float(want, out_prec) - exact)) / scale <= 5 * tol, name
+        else:
+            assert rel_err(got, want, out_prec) <= tol, name
+    hip.close()
