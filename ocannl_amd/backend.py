@@ -75,7 +75,7 @@ EXPORTS = (
     "ocannl_hip_code_routine_name", "ocannl_hip_code_kparams", "ocannl_hip_code_source",
     "ocannl_hip_code_num_kernels", "ocannl_hip_code_kernel_info", "ocannl_hip_link",
     "ocannl_hip_routine_free", "ocannl_hip_routine_set_static", "ocannl_hip_routine_run",
-    "ocannl_hip_routine_run_timed",
+    "ocannl_hip_routine_run_timed", "ocannl_hip_routine_profile_kernel", "ocannl_hip_routine_profile_read",
 )
 
 _lib = None
@@ -128,6 +128,8 @@ def load_library() -> ctypes.CDLL:
         "ocannl_hip_routine_set_static": (i32, [vp, i32, i64]),
         "ocannl_hip_routine_run": (i32, [vp]),
         "ocannl_hip_routine_run_timed": (i32, [vp, P(ctypes.c_float), i32]),
+        "ocannl_hip_routine_profile_kernel": (i32, [vp, i32]),
+        "ocannl_hip_routine_profile_read": (i32, [vp, P(ctypes.c_double), P(i64)]),
     }
     for name in EXPORTS:
         fn = getattr(lib, name)   # AttributeError if the library lacks a declared symbol
@@ -347,6 +349,14 @@ class Routine:
     def run(self) -> None:
         """``Task.run``: checks static indices, enqueues the kernels; asynchronous."""
         _check(load_library().ocannl_hip_routine_run(self._h))
+
+    def profile_kernel(self, kernel_index: int) -> None:
+        _check(load_library().ocannl_hip_routine_profile_kernel(self._h, kernel_index))
+
+    def profile_read(self):
+        ms, n = ctypes.c_double(), ctypes.c_int64()
+        _check(load_library().ocannl_hip_routine_profile_read(self._h, ctypes.byref(ms), ctypes.byref(n)))
+        return ms.value, n.value
 
     def run_timed(self) -> List[float]:
         n = len(self.code.kernels(self.index))

@@ -379,6 +379,162 @@ Block strip_comments(const Block& b, std::string* last_comment) {
 
 }  // namespace
 
+// Chain/inner split and parallel classification of one top-level statement.
+// Returns false when the statement runs nothing (a zero-trip loop).
+static bool analyze_nest(const Routine& r, const StmtP& sp, Phase& ph) {
+  (void)r;
+  std::vector<const Stmt*> chain;
+  Block inner;
+  if (sp->kind == Stmt::For) {
+    const Stmt* cur = sp.get();
+    for (;;) {
+      chain.push_back(cur);
+      Block body = strip_comments(cur->body, nullptr);
+      if (body.size() == 1 && body[0]->kind == Stmt::For) { cur = body[0].get(); continue; }
+      inner = body;
+      break;
+    }
+  } else {
+    inner = {sp};
+  }
+  for (const Stmt* l : chain)
+    if (l->to - l->from + 1 <= 0) return false;
+  std::vector<Access> acc;
+  bool whole = false, foreign = false;
+  std::set<ScopeId> declared;
+  block_accesses(inner, acc, whole, foreign, declared);
+  for (const Stmt* l : chain) {
+    const int64_t ext = l->to - l->from + 1;
+    const bool par = !whole && !foreign && symbol_is_parallel(l->sym, acc);
+    if (par) { ph.par_syms.push_back(l->sym); ph.par_from.push_back(l->from); ph.par_ext.push_back(ext); }
+    else { ph.seq_syms.push_back(l->sym); ph.seq_from.push_back(l->from); ph.seq_to.push_back(l->to); }
+  }
+  ph.inner = inner;
+  return true;
+}
+
+static void set_contraction_bytes(Phase& ph) {
+  const GemmDesc& g = ph.gemm;
+  auto op_bytes = [&](const GemmOperand& o, double rows, double cols) {
+    double n = rows * cols;
+    for (int i = 0; i < g.nbatch; ++i) if (o.s_batch[i]) n *= (double)g.batch_ext[i];
+    return n * prec_in_bytes(o.prec);
+  };
+  ph.bytes = op_bytes(g.a, (double)g.M, (double)g.K) + op_bytes(g.b, (double)g.N, (double)g.K) +
+             op_bytes(g.c, (double)g.M, (double)g.N) * (g.accumulate ? 2 : 1);
+}
+
+// De-virtualisation.  The optimiser inlines a contraction that is read once into its consumer as
+//   v { v := 0; for k.. { v := fma(a[..], b[..], v) } }
+// (arrayjit/lib/low_level.ml:1165-1316; test/einsum/inline_permuted_view-c_fwd.ll.expected).  When
+// such a reduction is large enough for the MFMA kernels it is given a scratch tensor indexed by the
+// enclosing loop symbols it depends on, computed by a contraction phase of its own, and the
+// consumer reads the scratch element instead.
+static void devirtualise(Routine& r, const StmtP& sp, const PlanOptions& opt, Plan& plan, const std::string& label) {
+  if (!opt.enable_mfma) return;
+  // enclosing perfect chain
+  std::vector<const Stmt*> chain;
+  Block inner;
+  if (sp->kind == Stmt::For) {
+    const Stmt* cur = sp.get();
+    for (;;) {
+      chain.push_back(cur);
+      Block body = strip_comments(cur->body, nullptr);
+      if (body.size() == 1 && body[0]->kind == Stmt::For) { cur = body[0].get(); continue; }
+      inner = body;
+      break;
+    }
+  } else inner = {sp};
+  if (inner.size() != 1 || inner[0]->kind != Stmt::Set) return;
+  for (const Stmt* l : chain) if (l->from != 0 || l->to < l->from) return;
+
+  std::vector<Scalar*> found;
+  std::function<void(Scalar&)> walk = [&](Scalar& s) {
+    if (s.kind == Scalar::LocalScope) { found.push_back(&s); return; }
+    if (s.a) walk(*s.a);
+    if (s.b) walk(*s.b);
+    if (s.c) walk(*s.c);
+  };
+  walk(*inner[0]->value);
+  for (Scalar* ls : found) {
+    Block body = strip_comments(ls->body, nullptr);
+    if (body.size() != 2 || body[0]->kind != Stmt::SetLocal || !(body[0]->scope == ls->scope)) continue;
+    if (body[0]->value->kind != Scalar::Const || body[0]->value->cst != 0.0) continue;
+    if (body[1]->kind != Stmt::For) continue;
+    std::vector<const Stmt*> red;
+    const Stmt* cur = body[1].get();
+    const Stmt* upd = nullptr;
+    for (;;) {
+      red.push_back(cur);
+      Block b2 = strip_comments(cur->body, nullptr);
+      if (b2.size() != 1) break;
+      if (b2[0]->kind == Stmt::For) { cur = b2[0].get(); continue; }
+      if (b2[0]->kind == Stmt::SetLocal && b2[0]->scope == ls->scope) upd = b2[0].get();
+      break;
+    }
+    if (!upd) continue;
+    const Scalar& v = *upd->value;
+    if (!(v.kind == Scalar::Tern && v.tern == Ternop::Fma && v.c->kind == Scalar::GetLocal && v.c->scope == ls->scope)) continue;
+    if (v.a->kind != Scalar::Get || v.b->kind != Scalar::Get) continue;
+    // enclosing symbols the operands depend on
+    std::vector<const Stmt*> dep;
+    double flops = 2.0;
+    for (const Stmt* l : chain) {
+      bool used = false;
+      for (auto& ix : v.a->idcs) used |= ix.mentions(l->sym);
+      for (auto& ix : v.b->idcs) used |= ix.mentions(l->sym);
+      if (used) { dep.push_back(l); flops *= (double)(l->to + 1); }
+    }
+    bool ok = true;
+    for (const Stmt* l : red) { if (l->from != 0 || l->to < 0) ok = false; flops *= (double)(l->to - l->from + 1); }
+    if (!ok || flops < (double)opt.min_mfma_flops) continue;
+
+    // scratch node + candidate nest
+    int new_id = 1;
+    for (auto& kv : r.nodes) new_id = std::max(new_id, kv.first + 1);
+    Node t;
+    t.id = new_id;
+    t.ident = "ctr" + std::to_string(new_id) + "_" + r.node(ls->scope.node).ident;
+    t.prec = Prec::Single;
+    t.mode = Mode::Local;
+    for (const Stmt* l : dep) t.dims.push_back(l->to + 1);
+    if (t.dims.empty()) t.dims.push_back(1);
+    Indices tix;
+    for (const Stmt* l : dep) { AxisIndex a; a.kind = AxisIndex::Iter; a.sym = l->sym; tix.push_back(a); }
+    if (dep.empty()) { AxisIndex a; a.kind = AxisIndex::Fixed; a.fixed = 0; tix.push_back(a); }
+
+    auto self = std::make_shared<Scalar>();
+    self->kind = Scalar::Get; self->node = t.id; self->idcs = tix;
+    auto fma = std::make_shared<Scalar>();
+    fma->kind = Scalar::Tern; fma->tern = Ternop::Fma; fma->arg_prec = v.arg_prec;
+    fma->a = v.a; fma->b = v.b; fma->c = self;
+    auto set = std::make_shared<Stmt>();
+    set->kind = Stmt::Set; set->node = t.id; set->idcs = tix; set->value = fma;
+    StmtP nest = set;
+    auto wrap = [&](const Stmt* l) {
+      auto f = std::make_shared<Stmt>();
+      f->kind = Stmt::For; f->sym = l->sym; f->from = l->from; f->to = l->to; f->body = {nest};
+      nest = f;
+    };
+    for (auto it = red.rbegin(); it != red.rend(); ++it) wrap(*it);
+    for (auto it = dep.rbegin(); it != dep.rend(); ++it) wrap(*it);
+
+    r.nodes.emplace(t.id, t);
+    Phase ph;
+    ph.label = label + " (contraction of " + r.node(ls->scope.node).ident + ")";
+    ph.stmt = nest;
+    ph.fused_zero_init = true;
+    if (!analyze_nest(r, nest, ph) || !match_contraction(r, ph, opt)) { r.nodes.erase(t.id); continue; }
+    set_contraction_bytes(ph);
+    plan.phases.push_back(std::move(ph));
+    plan.scratch.push_back(t);
+    // the consumer now reads the scratch element
+    Scalar repl;
+    repl.kind = Scalar::Get; repl.node = t.id; repl.idcs = tix;
+    *ls = repl;
+  }
+}
+
 Plan make_plan(Routine& r, const PlanOptions& opt) {
   Plan plan;
   std::string label;
@@ -400,44 +556,17 @@ Plan make_plan(Routine& r, const PlanOptions& opt) {
     }
     if (sp->kind == Stmt::DeclareLocal || sp->kind == Stmt::SetLocal)
       throw InvalidArgument("hip backend: scalar locals at routine scope are not supported (routine " + r.name + ")");
-    // perfect-nest chain
-    std::vector<const Stmt*> chain;
-    Block inner;
-    if (sp->kind == Stmt::For) {
-      const Stmt* cur = sp.get();
-      for (;;) {
-        chain.push_back(cur);
-        Block body = strip_comments(cur->body, nullptr);
-        if (body.size() == 1 && body[0]->kind == Stmt::For) { cur = body[0].get(); continue; }
-        inner = body;
-        break;
-      }
-    } else {
-      inner = {sp};
-    }
-    std::vector<Access> acc;
-    bool whole = false, foreign = false;
-    std::set<ScopeId> declared;
-    block_accesses(inner, acc, whole, foreign, declared);
-    for (const Stmt* l : chain) {
-      const int64_t ext = l->to - l->from + 1;
-      if (ext <= 0) { chain.clear(); inner.clear(); break; }   // zero-trip loop: nothing runs
-    }
-    if (chain.empty() && inner.empty()) continue;
-    for (const Stmt* l : chain) {
-      const int64_t ext = l->to - l->from + 1;
-      const bool par = !whole && !foreign && symbol_is_parallel(l->sym, acc);
-      if (par) { ph.par_syms.push_back(l->sym); ph.par_from.push_back(l->from); ph.par_ext.push_back(ext); }
-      else { ph.seq_syms.push_back(l->sym); ph.seq_from.push_back(l->from); ph.seq_to.push_back(l->to); }
-    }
-    ph.inner = inner;
+    const size_t before = plan.phases.size();
+    devirtualise(r, sp, opt, plan, label);
+    const bool devirt = plan.phases.size() != before;
+    if (!analyze_nest(r, sp, ph)) continue;
 
     // fold a directly preceding Zero_out of the accumulation target into this phase when the nest
     // overwrites the whole array: every axis is a full-range parallel iterator or has extent 1.
     Binop accum;
-    if (!plan.phases.empty() && plan.phases.back().kind == Phase::Fill && reduction_shape(r, ph, &accum) &&
-        accum == Binop::Add && plan.phases.back().fill_node == inner[0]->node) {
-      const Stmt& set = *inner[0];
+    if (!devirt && !plan.phases.empty() && plan.phases.back().kind == Phase::Fill && reduction_shape(r, ph, &accum) &&
+        accum == Binop::Add && plan.phases.back().fill_node == ph.inner[0]->node) {
+      const Stmt& set = *ph.inner[0];
       const Node& n = r.node(set.node);
       bool full = true;
       for (size_t p = 0; p < set.idcs.size() && full; ++p) {
@@ -457,14 +586,7 @@ Plan make_plan(Routine& r, const PlanOptions& opt) {
       choose_coop(r, ph, opt);
       account_bytes(r, ph);
     } else {
-      const GemmDesc& g = ph.gemm;
-      auto op_bytes = [&](const GemmOperand& o, double rows, double cols) {
-        double n = rows * cols;
-        for (int i = 0; i < g.nbatch; ++i) if (o.s_batch[i]) n *= (double)g.batch_ext[i];
-        return n * prec_in_bytes(o.prec);
-      };
-      ph.bytes = op_bytes(g.a, (double)g.M, (double)g.K) + op_bytes(g.b, (double)g.N, (double)g.K) +
-                 op_bytes(g.c, (double)g.M, (double)g.N) * (g.accumulate ? 2 : 1);
+      set_contraction_bytes(ph);
     }
     plan.phases.push_back(std::move(ph));
   }

@@ -142,6 +142,9 @@ struct ocannl_hip_routine {
   };
   std::vector<Launch> launches;
   std::vector<hipEvent_t> timing_events;
+  int profile_kernel = -1;
+  std::vector<hipEvent_t> profile_events;   // pairs (start, stop), reused after each read
+  size_t profile_used = 0;
 };
 
 namespace {
@@ -189,6 +192,15 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
   for (size_t li = 0; li < rt.launches.size(); ++li) {
     auto& l = rt.launches[li];
     const Phase& ph = rt.code->plan.phases[l.phase];
+    const bool bracket = !timed && rt.profile_kernel == (int)li;
+    if (bracket) {
+      while (rt.profile_events.size() < rt.profile_used + 2) {
+        hipEvent_t e;
+        hip_check(hipEventCreate(&e), "hipEventCreate");
+        rt.profile_events.push_back(e);
+      }
+      hip_check(hipEventRecord(rt.profile_events[rt.profile_used], dev.stream), "hipEventRecord");
+    }
     if (ph.kind == Phase::Fill) {
       hip_check(hipMemsetAsync(l.fill_ptr, 0, l.fill_bytes, dev.stream), "hipMemsetAsync");
     } else if (ph.kind == Phase::Generic) {
@@ -216,6 +228,10 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
       hip_check(launch_gemm(g, a, dev.stream), "launch_gemm");
     }
     if (timed) hip_check(hipEventRecord(rt.timing_events[li + 1], dev.stream), "hipEventRecord");
+    if (bracket) {
+      hip_check(hipEventRecord(rt.profile_events[rt.profile_used + 1], dev.stream), "hipEventRecord");
+      rt.profile_used += 2;
+    }
   }
   if (timed) {
     hip_check(hipStreamSynchronize(dev.stream), "hipStreamSynchronize");
@@ -649,6 +665,7 @@ void ocannl_hip_routine_free(ocannl_hip_routine* rt) {
   (void)hipSetDevice(rt->dev->ordinal);
   (void)hipStreamSynchronize(rt->dev->stream);
   for (auto e : rt->timing_events) (void)hipEventDestroy(e);
+  for (auto e : rt->profile_events) (void)hipEventDestroy(e);
   if (rt->module) (void)hipModuleUnload(rt->module);
   if (rt->scratch) { (void)hipFree(rt->scratch); rt->dev->scratch_used -= rt->scratch_bytes; }
   rt->dev->live_routines--;
@@ -675,6 +692,31 @@ int ocannl_hip_routine_run_timed(ocannl_hip_routine* rt, float* kernel_ms, int c
   return guarded([&] {
     if (!rt || !kernel_ms) throw InvalidArgument("run_timed: null argument");
     enqueue(*rt, kernel_ms, cap);
+  });
+}
+
+int ocannl_hip_routine_profile_kernel(ocannl_hip_routine* rt, int kernel_index) {
+  return guarded([&] {
+    if (!rt) throw InvalidArgument("profile_kernel: null routine");
+    if (kernel_index >= (int)rt->launches.size()) throw InvalidArgument("profile_kernel: kernel index out of range");
+    rt->profile_kernel = kernel_index;
+  });
+}
+
+int ocannl_hip_routine_profile_read(ocannl_hip_routine* rt, double* total_ms, int64_t* launches) {
+  return guarded([&] {
+    if (!rt || !total_ms || !launches) throw InvalidArgument("profile_read: null argument");
+    rt->dev->make_current();
+    hip_check(hipStreamSynchronize(rt->dev->stream), "hipStreamSynchronize");
+    double sum = 0;
+    for (size_t i = 0; i + 1 < rt->profile_used; i += 2) {
+      float ms = 0;
+      hip_check(hipEventElapsedTime(&ms, rt->profile_events[i], rt->profile_events[i + 1]), "hipEventElapsedTime");
+      sum += ms;
+    }
+    *total_ms = sum;
+    *launches = (int64_t)(rt->profile_used / 2);
+    rt->profile_used = 0;
   });
 }
 

@@ -315,13 +315,35 @@ class Graph:
         out: List[L.Stmt] = [L.Comment(f"{loss.label} forward and gradient update")]
         out += self.forward(loss)
         out.append(L.Comment(f"{loss.label} zero grads and backprop"))
+        seen = set()
         for t in order:
-            if t.grad is not None:
+            if t.grad is not None and t.grad.id not in seen:
+                seen.add(t.grad.id)
                 out.append(L.ZeroOut(t.grad))
                 if not getattr(t.grad, "_touched", False):
                     t.grad.zero_initialized_by_code = True
                 t.grad._touched = True
         out += L.loop_over_dims(loss.grad.dims, lambda ix: [L.Set(loss.grad, ix, L.Const(1.0))])
+        for t in reversed(order):
+            if t.bwd is not None:
+                out += t.bwd()
+        return out
+
+    def backprop_from(self, root: T, comment: str = "backprop") -> List[L.Stmt]:
+        """Backprop with the root gradient supplied by the caller (a context node that is not
+        zeroed): zero every other gradient, then the gradient assignments in reverse order."""
+        root.grad.mode = "ctx"
+        self.forced_ctx.add(root.grad.id)
+        order = self.topo(root)
+        out: List[L.Stmt] = [L.Comment(comment)]
+        seen = set()
+        for t in order:
+            if t.grad is not None and t.grad is not root.grad and t.grad.id not in seen:
+                seen.add(t.grad.id)
+                out.append(L.ZeroOut(t.grad))
+                if not getattr(t.grad, "_touched", False):
+                    t.grad.zero_initialized_by_code = True
+                t.grad._touched = True
         for t in reversed(order):
             if t.bwd is not None:
                 out += t.bwd()
@@ -712,3 +734,79 @@ def make_routine(g: Graph, name: str, body: List[L.Stmt], statics: Sequence[L.St
     if inline:
         body = inline_single_use(g, body, keep=outputs)
     return L.Routine(name, body, list(statics))
+
+
+# ------------------------------------------------------------------------------------------------
+# further operations used by the language-model configurations
+# ------------------------------------------------------------------------------------------------
+
+def rename(t: T, mapping: Dict[str, str]) -> T:
+    """The same tensor under other axis labels (e.g. keys indexed by ``t`` instead of ``s``)."""
+    return T(t.value, tuple(mapping.get(a, a) for a in t.axes), t.grad, (t,), label=t.label)
+
+
+def gather_rows(g: Graph, table: T, ids: T, table_axis: str, ident: str = "embed") -> T:
+    """Embedding lookup in the form the optimiser's one-hot rewrite produces
+    (arrayjit/lib/low_level.ml:2193-2215): ``where(in_range(id), table[.., @dyn id, ..], 0)`` with
+    the guard evaluated in double; the table gradient keeps the one-hot contraction
+    ``g_table[e, v] += g[.., e] * (v == id[..])``."""
+    out_axes = tuple(ids.axes) + tuple(a for a in table.axes if a != table_axis)
+    ext = dict(zip(ids.axes, ids.dims))
+    ext.update(dict(zip(table.axes, table.dims)))
+    classes = ext[table_axis]
+    v, gr = g._result(ident, out_axes, ext, None, table.grad is not None)
+    res = T(v, out_axes, gr, (table, ids), label=ident)
+    dyn_axis = table.axes.index(table_axis)
+
+    def value(idx):
+        iv = L.Get(ids.value, tuple(idx[a] for a in ids.axes))
+        lower = L.Binop("lt", L.Const(-1.0), iv)
+        upper = L.Binop("lt", iv, L.Const(float(classes)))
+        integral = L.Binop("eq", iv, L.Unop("trunc", iv, "double"))
+        guard = L.Binop("and", L.Binop("and", lower, upper), integral)
+        tix = tuple(L.Fixed(0) if a == table_axis else idx[a] for a in table.axes)
+        gather = L.GetDynamic(table.value, tix, dyn_axis, iv, ids.value.prec)
+        return L.Ternop("where", guard, gather, L.Const(0.0), "double")
+
+    space = [(a, ext[a]) for a in out_axes]
+    res.fwd = g.lower(v, out_axes, space, value)
+
+    def bwd():
+        if table.grad is None:
+            return []
+        sp = space + [(table_axis, classes)]
+
+        def rhs(idx):
+            onehot = L.Binop("eq", L.EmbedIndex(idx[table_axis]), L.Get(ids.value, tuple(idx[a] for a in ids.axes)))
+            return L.Binop("mul", L.Get(gr, tuple(idx[a] for a in out_axes)), onehot)
+
+        return g.lower(table.grad, table.axes, sp, rhs, accum="add", init_neutral=False)
+
+    res.bwd = bwd
+    return res
+
+
+def softmax(g: Graph, x: T, axis: str, ident: str = "softmax") -> T:
+    """``Nn_blocks.softmax`` (lib/nn_blocks.ml:137-143): max over the axis, exp of the shifted
+    values, division by their sum."""
+    rest = tuple(a for a in x.axes if a != axis)
+    max_vals = g.reduce(x, rest, accum="max", ident=ident + "_max")
+    exp_vals = g.unary("exp", g.sub(x, max_vals, x.axes, ident=ident + "_shift"), ident=ident + "_exp")
+    denom = g.reduce(exp_vals, rest, ident=ident + "_sum")
+    return g.div(exp_vals, denom, x.axes, ident=ident)
+
+
+def layer_norm(g: Graph, x: T, axis: str, label: str, epsilon: float = 1e-5):
+    """``Nn_blocks.layer_norm`` exactly as written (lib/nn_blocks.ml:251-258): note that ``mean``
+    there is the SUM over the axis and ``centered = (x - mean) / dim``."""
+    rest = tuple(a for a in x.axes if a != axis)
+    d = dict(zip(x.axes, x.dims))[axis]
+    gamma = g.param(f"gamma_{label}", (axis,), (d,))
+    beta = g.param(f"beta_{label}", (axis,), (d,))
+    mean = g.reduce(x, rest, ident=f"mean_{label}")
+    centered = g.div(g.sub(x, mean, x.axes), ConstT(float(d)), x.axes, ident=f"centered_{label}")
+    variance = g.reduce(g.mul(centered, centered, x.axes), rest, ident=f"variance_{label}")
+    std_dev = g.unary("sqrt", g.add(variance, ConstT(epsilon), rest), ident=f"std_{label}")
+    normalized = g.div(centered, std_dev, x.axes, ident=f"normalized_{label}")
+    out = g.add(g.mul(gamma, normalized, x.axes), beta, x.axes, ident=f"ln_{label}")
+    return out, [gamma, beta]

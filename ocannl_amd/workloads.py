@@ -169,3 +169,236 @@ def dense_contraction(b: int = 8192, i: int = 4096, o: int = 4096, prec: str = "
     outs = [n for k, n in (("fwd", Y), ("dx", dX), ("dw", dW)) if k in which]
     return Workload(f"dense_{prec}", routine, init, nodes, {}, outs,
                     f"b|i->o contraction b={b} i={i} o={o} {prec} (dest {out_prec}), fwd+dX+dW")
+
+
+# ------------------------------------------------------------------------------------------------
+# config 2: character-level MLP language model
+# ------------------------------------------------------------------------------------------------
+
+def char_mlp(batch: int = 32, vocab: int = 27, context: int = 3, embed: int = 10, hidden: int = 200,
+             lr: float = 1e-3, seed: int = 0, inline: bool = True, n_batches: int = 16) -> Workload:
+    """test/training/mlp_names.ml:145-168 with synthetic tokens: ids -> embedding gather ->
+    ``tanh(emb +* w1 + b1)`` -> logits -> stable log-softmax cross entropy; Adam update.  A fresh
+    batch is a slice of a resident id/target set selected by the static index ``batch_n``."""
+    from .frontend import gather_rows
+    L.reset_symbols(0)
+    g = Graph("single", "single")
+    batch_n = L.StaticSymbol(L.fresh_symbol(), n_batches)
+    ids_all = g.input("input_batch", ("n", "b", "s"), (n_batches, batch, context))
+    tgt_all = g.input("target_batch", ("n", "b", "v"), (n_batches, batch, vocab))
+    ids = _SliceT(ids_all.value, ("b", "s"), (batch, context),
+                  lambda idx: L.Get(ids_all.value, (L.It(batch_n.sym), idx["b"], idx["s"])))
+    ids.value_prec = "single"
+    tgt = _SliceT(tgt_all.value, ("b", "v"), (batch, vocab),
+                  lambda idx: L.Get(tgt_all.value, (L.It(batch_n.sym), idx["b"], idx["v"])))
+    c = g.param("c", ("e", "v"), (embed, vocab))
+    w1 = g.param("w1", ("h", "s", "e"), (hidden, context, embed)); b1 = g.param("b1", ("h",), (hidden,))
+    w2 = g.param("w2", ("v", "h"), (vocab, hidden)); b2 = g.param("b2", ("v",), (vocab,))
+    # the gather reads the id through the slice
+    ids_view = T(ids_all.value, ("b", "s"), None)
+    ids_view._getter = ids._getter
+    ids_view._dims = (batch, context)
+    emb = _gather_slice(g, c, ids, "v", batch, context)
+    hid = g.unary("tanh", g.add(g.einsum(emb, w1, ("b", "h"), ident="emb_w1"), b1, ("b", "h")), ident="hidden")
+    logits = g.add(g.einsum(w2, hid, ("b", "v"), ident="w2h"), b2, ("b", "v"), ident="logits")
+    max_l = g.reduce(logits, ("b",), accum="max", ident="max_l")
+    shifted = g.sub(logits, max_l, ("b", "v"), ident="shifted")
+    lse = g.unary("log", g.reduce(g.unary("exp", shifted), ("b",), ident="sumexp"), ident="lse")
+    log_probs = g.sub(shifted, lse, ("b", "v"), ident="log_probs")
+    nll = g.unary("neg", g.reduce(g.mul(tgt, log_probs, ("b", "v")), ("l",), ident="tgt_lp"), ident="nll")
+    loss = g.div(nll, ConstT(float(batch)), ("l",), ident="batch_loss")
+    loss.label = "batch_loss"
+    params = [c, w1, b1, w2, b2]
+    body = g.grad_update(loss) + g.adam_update(params, lr=lr)
+    routine = make_routine(g, "char_mlp_adam_step", body, [batch_n], inline=inline, outputs=[loss.value])
+    rng = np.random.default_rng(seed)
+    toks = rng.integers(0, vocab, size=(n_batches, batch, context + 1))
+    onehot = np.zeros((n_batches, batch, vocab), np.float32)
+    np.put_along_axis(onehot, toks[..., -1:], 1.0, axis=-1)
+    init = {ids_all.value.id: toks[..., :context].astype(np.float32), tgt_all.value.id: onehot}
+    for p in params:
+        fan = int(np.prod(p.dims[1:])) if len(p.dims) > 1 else p.dims[0]
+        init[p.value.id] = (rng.uniform(-1, 1, p.dims) / np.sqrt(fan)).astype(np.float32)
+    nodes = {p.label: p.value for p in params}
+    nodes["loss"] = loss.value
+    for p in params:
+        nodes["m_" + p.label] = p.adam_m
+        nodes["v_" + p.label] = p.adam_v
+    return Workload("char_mlp", routine, init, nodes, {"batch_n": batch_n}, [loss.value],
+                    f"char MLP LM vocab {vocab} ctx {context} emb {embed} hid {hidden} batch {batch}, Adam lr {lr}")
+
+
+def _gather_slice(g, table, ids_slice, table_axis, batch, context):
+    from .frontend import gather_rows
+    # gather_rows reads ids through `ids.value` with its axes; give it a view whose element read
+    # goes through the slice getter
+    class _IdsView:
+        pass
+    view = T(ids_slice.value, ids_slice.axes, None)
+    view._getter = ids_slice._getter
+    return _gather_rows_with_getter(g, table, view, (batch, context), table_axis)
+
+
+def _gather_rows_with_getter(g, table, ids, ids_dims, table_axis, ident="embed"):
+    out_axes = tuple(ids.axes) + tuple(a for a in table.axes if a != table_axis)
+    ext = dict(zip(ids.axes, ids_dims))
+    ext.update(dict(zip(table.axes, table.dims)))
+    classes = ext[table_axis]
+    v, gr = g._result(ident, out_axes, ext, None, True)
+    res = T(v, out_axes, gr, (table,), label=ident)
+    dyn_axis = table.axes.index(table_axis)
+
+    def value(idx):
+        iv = ids._getter(idx)
+        guard = L.Binop("and", L.Binop("and", L.Binop("lt", L.Const(-1.0), iv), L.Binop("lt", iv, L.Const(float(classes)))),
+                        L.Binop("eq", iv, L.Unop("trunc", iv, "double")))
+        tix = tuple(L.Fixed(0) if a == table_axis else idx[a] for a in table.axes)
+        return L.Ternop("where", guard, L.GetDynamic(table.value, tix, dyn_axis, iv, "single"), L.Const(0.0), "double")
+
+    space = [(a, ext[a]) for a in out_axes]
+    res.fwd = g.lower(v, out_axes, space, value)
+
+    def bwd():
+        sp = space + [(table_axis, classes)]
+        return g.lower(table.grad, table.axes, sp, lambda idx: L.Binop(
+            "mul", L.Get(gr, tuple(idx[a] for a in out_axes)),
+            L.Binop("eq", L.EmbedIndex(idx[table_axis]), ids._getter(idx))), accum="add", init_neutral=False)
+
+    res.bwd = bwd
+    return res
+
+
+# ------------------------------------------------------------------------------------------------
+# config 5: batched attention, forward and backward
+# ------------------------------------------------------------------------------------------------
+
+def attention(b: int = 16, h: int = 16, q: int = 1024, k: int = 1024, d: int = 64, prec: str = "bfloat16",
+              grad_prec: str = "single", seed: int = 0, inline: bool = True, backward: bool = True) -> Workload:
+    """``scores[b,s,h,t] = sum_d Q[b,s,h,d] K[b,t,h,d] / sqrt(d)``, softmax over ``t``,
+    ``out[b,s,h,e] = sum_t attn[b,s,h,t] V[b,t,h,e]`` (lib/nn_blocks.ml:222-236) and the backward
+    contractions from a supplied ``d out``."""
+    from .frontend import softmax
+    L.reset_symbols(0)
+    g = Graph(prec, grad_prec)
+    Q = g.param("q", ("b", "s", "h", "d"), (b, q, h, d)); K = g.param("k", ("b", "t", "h", "d"), (b, k, h, d))
+    V = g.param("v", ("b", "t", "h", "e"), (b, k, h, d))
+    for t in (Q, K, V):
+        t.grad.mode = "ctx"
+    scores = g.div(g.einsum(Q, K, ("b", "s", "h", "t"), ident="qk"), ConstT(float(np.sqrt(d))), ("b", "s", "h", "t"),
+                   ident="scores")
+    attn = softmax(g, scores, "t", ident="attn")
+    out = g.einsum(attn, V, ("b", "s", "h", "e"), ident="attn_out")
+    out.label = "attn_out"
+    body = g.forward(out)
+    outputs = [out.value]
+    if backward:
+        body += g.backprop_from(out)
+        outputs += [Q.grad, K.grad, V.grad]
+    routine = make_routine(g, "attention_fwd_bwd" if backward else "attention_fwd", body, [], inline=inline, outputs=outputs)
+    rng = np.random.default_rng(seed)
+    init = {t.value.id: as_prec(rng.standard_normal(t.dims).astype(np.float32), prec) for t in (Q, K, V)}
+    if backward:
+        init[out.grad.id] = as_prec(rng.standard_normal(out.dims).astype(np.float32), grad_prec)
+    nodes = {"q": Q.value, "k": K.value, "v": V.value, "out": out.value, "attn": attn.value,
+             "dq": Q.grad, "dk": K.grad, "dv": V.grad, "dout": out.grad}
+    return Workload("attention", routine, init, nodes, {}, outputs,
+                    f"attention b={b} h={h} q={q} k={k} d={d} {prec}, fwd{'+bwd' if backward else ''}")
+
+
+# ------------------------------------------------------------------------------------------------
+# config 4: decoder-only transformer training step
+# ------------------------------------------------------------------------------------------------
+
+def transformer(batch: int = 32, seq: int = 256, d_model: int = 512, heads: int = 8, d_ff: int = 2048,
+                layers: int = 4, vocab: int = 4096, prec: str = "bfloat16", grad_prec: str = "single",
+                lr: float = 0.01, seed: int = 0, inline: bool = True) -> Workload:
+    """Decoder-only transformer: ``Nn_blocks.decoder_only`` (lib/nn_blocks.ml:274-296: post-norm
+    blocks of masked multi-head attention and a 2-layer ReLU FFN), wired as in
+    test/training/fsm_transformer.ml:122-139 -- one-hot token input times an embedding matrix plus
+    a learned positional encoding, a final projection to the vocabulary, softmax cross entropy --
+    with ``Train.grad_update`` + ``Train.sgd_update`` compiled as one routine."""
+    from .frontend import layer_norm, rename, softmax
+    L.reset_symbols(0)
+    g = Graph(prec, grad_prec)
+    dk = d_model // heads
+    x_in = g.input("input_batch", ("b", "s", "v"), (batch, seq, vocab))
+    target = g.input("target_batch", ("b", "s", "v"), (batch, seq, vocab))
+    mask = g.input("mask", ("s", "t"), (seq, seq), "single")
+    lrate = g.input("learning_rate", ("one",), (1,), "single")
+    params: List[T] = []
+
+    def P(name, axes, dims):
+        p = g.param(name, axes, dims)
+        params.append(p)
+        return p
+
+    w_embed = P("w_embed", ("m", "v"), (d_model, vocab))
+    pos = P("pos_encoding", ("s", "m"), (seq, d_model))
+    x = g.add(g.einsum(w_embed, x_in, ("b", "s", "m"), ident="embed"), pos, ("b", "s", "m"), ident="embedded")
+    for li in range(layers):
+        lb = f"l{li}"
+        w_q = P(f"w_q_{lb}", ("h", "d", "m"), (heads, dk, d_model))
+        w_k = P(f"w_k_{lb}", ("h", "d", "m"), (heads, dk, d_model))
+        w_v = P(f"w_v_{lb}", ("h", "e", "m"), (heads, dk, d_model))
+        w_o = P(f"w_o_{lb}", ("m", "h", "e"), (d_model, heads, dk))
+        q = g.einsum(w_q, x, ("b", "s", "h", "d"), ident=f"q_{lb}")
+        k = rename(g.einsum(w_k, x, ("b", "s", "h", "d"), ident=f"k_{lb}"), {"s": "t"})
+        v = rename(g.einsum(w_v, x, ("b", "s", "h", "e"), ident=f"v_{lb}"), {"s": "t"})
+        scores = g.div(g.einsum(q, k, ("b", "s", "h", "t"), ident=f"qk_{lb}"), ConstT(float(np.sqrt(dk))),
+                       ("b", "s", "h", "t"), ident=f"scores_{lb}")
+        masked = g.where(mask, scores, ConstT(-1e9), ident=f"masked_{lb}")
+        masked = T(masked.value, ("s", "t", "b", "h"), masked.grad, masked.children, masked.fwd, masked.bwd, masked.label) \
+            if False else masked
+        attn = softmax(g, _reorder(g, masked, ("b", "s", "h", "t")), "t", ident=f"attn_{lb}")
+        att_out = g.einsum(attn, v, ("b", "s", "h", "e"), ident=f"attn_out_{lb}")
+        mha = g.einsum(w_o, att_out, ("b", "s", "m"), ident=f"mha_{lb}")
+        x1, ln1p = layer_norm(g, g.add(x, mha, ("b", "s", "m")), "m", f"ln1_{lb}")
+        params += ln1p
+        w_f1 = P(f"w_ffn1_{lb}", ("f", "m"), (d_ff, d_model)); b_f1 = P(f"b_ffn1_{lb}", ("f",), (d_ff,))
+        w_f2 = P(f"w_ffn2_{lb}", ("m", "f"), (d_model, d_ff))
+        hid = g.unary("relu", g.add(g.einsum(w_f1, x1, ("b", "s", "f"), ident=f"ffn1_{lb}"), b_f1, ("b", "s", "f")),
+                      ident=f"ffn_hid_{lb}")
+        ffn = g.einsum(w_f2, hid, ("b", "s", "m"), ident=f"ffn_{lb}")
+        x, ln2p = layer_norm(g, g.add(x1, ffn, ("b", "s", "m")), "m", f"ln2_{lb}")
+        params += ln2p
+    w_out = P("w_out", ("v", "m"), (vocab, d_model))
+    logits = g.einsum(w_out, x, ("b", "s", "v"), ident="logits")
+    counts = g.unary("exp", logits, ident="counts")
+    probs = g.div(counts, g.reduce(counts, ("b", "s"), ident="counts_sum"), ("b", "s", "v"), ident="probs")
+    output_probs = g.reduce(g.mul(probs, target, ("b", "s", "v")), ("b", "s"), ident="output_probs")
+    tok_loss = g.unary("neg", g.unary("log", output_probs), ident="loss")
+    batch_loss = g.div(g.reduce(tok_loss, ("l",), ident="loss_sum"), ConstT(float(batch * seq)), ("l",), ident="batch_loss")
+    batch_loss.label = "batch_loss"
+    body = g.grad_update(batch_loss) + g.sgd_update(params, lrate)
+    routine = make_routine(g, "transformer_sgd_step", body, [], inline=inline, outputs=[batch_loss.value])
+    rng = np.random.default_rng(seed)
+    toks = rng.integers(0, vocab, size=(batch, seq + 1))
+    oh_in = np.zeros((batch, seq, vocab), np.float32); oh_tg = np.zeros((batch, seq, vocab), np.float32)
+    np.put_along_axis(oh_in, toks[:, :seq, None], 1.0, axis=-1)
+    np.put_along_axis(oh_tg, toks[:, 1:, None], 1.0, axis=-1)
+    init = {x_in.value.id: as_prec(oh_in, prec), target.value.id: as_prec(oh_tg, prec),
+            mask.value.id: np.tril(np.ones((seq, seq), np.float32)),
+            lrate.value.id: np.array([lr], np.float32)}
+    for p in params:
+        if p.label.startswith("gamma"):
+            vals = np.ones(p.dims, np.float32)
+        elif p.label.startswith(("beta", "b_")):
+            vals = np.zeros(p.dims, np.float32)
+        else:
+            fan_in = int(np.prod([d_ for a, d_ in zip(p.axes, p.dims) if a in ("m", "v", "f", "e") and a != p.axes[0]])) or p.dims[-1]
+            vals = (rng.uniform(-1, 1, p.dims) * np.sqrt(3.0 / max(fan_in, 1))).astype(np.float32)
+        init[p.value.id] = as_prec(vals, prec)
+    nodes = {p.label: p.value for p in params}
+    nodes.update({"loss": batch_loss.value, "logits": logits.value})
+    wl = Workload("transformer", routine, init, nodes, {}, [batch_loss.value],
+                  f"decoder-only transformer x{layers}: d_model {d_model}, {heads} heads, d_ff {d_ff}, seq {seq}, "
+                  f"batch {batch}, vocab {vocab}, {prec} values / {grad_prec} grads, SGD lr {lr}")
+    wl.params = params
+    return wl
+
+
+def _reorder(g: Graph, t: T, axes):
+    """Guarantee the axis order of a tensor (where() orders axes by first appearance)."""
+    if tuple(t.axes) == tuple(axes):
+        return t
+    return g.nary(t.label + "_perm", [t], axes, lambda x: x, [lambda gr, v, x: gr])
