@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X arrayjit backend on the reference's headline configurations.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A "step" is one run of the compiled routine (for the training configurations: forward + backprop
++ optimiser update compiled as ONE routine, as ``Train.to_routine`` does) on synthetic inputs that
+are resident in device memory before the timed region starts.  Prints one JSON line.
+
+workloads: transformer (BASELINE config 4, default), dense_bf16 / dense_f32 (config 3),
+attention (config 5), char_mlp (config 2), moons (config 1).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+import numpy as np  # noqa: E402
+
+PEAKS = {"mfma_bf16": 2500.0, "mfma_f32": 157.3, "hbm": 8000.0}   # TFLOP/s, TFLOP/s, GB/s (published)
+
+
+def build_workload(name: str):
+    from ocannl_amd import workloads as W
+    if name == "transformer":
+        return W.transformer(), "train_steps_per_sec", "steps/s", "bf16"
+    if name == "dense_bf16":
+        return W.dense_contraction(prec="bfloat16", out_prec="single"), "train_steps_per_sec", "steps/s", "bf16"
+    if name == "dense_f32":
+        return W.dense_contraction(prec="single", out_prec="single"), "train_steps_per_sec", "steps/s", "f32"
+    if name == "attention":
+        return W.attention(), "train_steps_per_sec", "steps/s", "bf16"
+    if name == "char_mlp":
+        return W.char_mlp(), "train_steps_per_sec", "steps/s", "f32"
+    if name == "moons":
+        return W.moons_mlp(), "train_steps_per_sec", "steps/s", "f32"
+    raise SystemExit(f"unknown workload {name}")
+
+
+def cpu_baseline(name: str):
+    """The CPU checker (the restated `cc` backend: generated C, gcc -O3 -march=native, one core,
+    in process) timed on a bounded sample of the same workload, scaled to steps/s of the full
+    configuration.  Reported next to the GPU number; it is not a target."""
+    from ocannl_amd import workloads as W
+    from parity import OracleRun
+
+    def time_steps(w, n, statics=None):
+        o = OracleRun(w.routine, w.init)
+        o.step(statics)   # first call: page in
+        t = time.perf_counter()
+        for _ in range(n):
+            o.step(statics)
+        return (time.perf_counter() - t) / n
+
+    if name == "transformer":
+        # per-step time is linear in the batch; layers add a constant each: two samples at batch 1
+        kw = dict(seq=256, d_model=512, heads=8, d_ff=2048, vocab=4096, prec="bfloat16", grad_prec="single")
+        t0 = time_steps(W.transformer(batch=1, layers=0, **kw), 1)
+        t1 = time_steps(W.transformer(batch=1, layers=1, **kw), 1)
+        full = 32.0 * (t0 + 4.0 * (t1 - t0))
+        return {"value": 1.0 / full, "unit": "steps/s", "cores": 1, "kind": "port",
+                "sample": f"batch 1 of 32 with 0 and 1 of 4 layers ({t0:.2f} s, {t1:.2f} s per step), "
+                          "extrapolated: 32 x (t0 + 4 x (t1 - t0))"}
+    if name in ("dense_bf16", "dense_f32"):
+        prec = "bfloat16" if name == "dense_bf16" else "single"
+        t = time_steps(W.dense_contraction(b=64, prec=prec, out_prec="single"), 1)
+        return {"value": 1.0 / (t * 128.0), "unit": "steps/s", "cores": 1, "kind": "port",
+                "sample": f"b=64 of 8192 rows ({t:.2f} s per step), scaled x128"}
+    if name == "attention":
+        t = time_steps(W.attention(b=1, h=1), 1)
+        return {"value": 1.0 / (t * 256.0), "unit": "steps/s", "cores": 1, "kind": "port",
+                "sample": f"1 of 256 (batch, head) pairs ({t:.2f} s per step), scaled x256"}
+    if name == "char_mlp":
+        w = W.char_mlp()
+        t = time_steps(w, 2000, {w.statics["batch_n"].sym: 0})
+        return {"value": 1.0 / t, "unit": "steps/s", "cores": 1, "kind": "port", "sample": "2000 full steps"}
+    w = W.moons_mlp()
+    t = time_steps(w, 20000, {w.statics["batch_n"].sym: 0})
+    return {"value": 1.0 / t, "unit": "steps/s", "cores": 1, "kind": "port", "sample": "20000 full steps"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="transformer")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernel-table", action="store_true", help="print per-kernel times to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)")
+
+    from ocannl_amd import backend as B
+    from parity import HipRun
+
+    w, metric, unit, dtype = build_workload(args.workload)
+    t_c = time.perf_counter()
+    hip = HipRun(w.routine, w.init)
+    compile_s = time.perf_counter() - t_c
+    kernels = hip.code.kernels()
+    statics = {s.sym: 0 for s in w.statics.values()}
+    nb = next(iter(w.statics.values())).range if w.statics else 1
+
+    def step(i):
+        hip.step({sym: i % nb for sym in statics} if statics else None)
+
+    for i in range(max(args.warmup, 1)):
+        step(i)
+    B.await_(hip.ctx.dev)
+
+    # per-kernel times (HIP events on the device stream, outside the timed region): find the
+    # dominant kernel = the kernel name with the largest summed time per step
+    per = np.zeros(len(kernels))
+    n_prof = 3
+    for _ in range(n_prof):
+        per += np.array(hip.rt.run_timed())
+    per /= n_prof
+    by_name = {}
+    for k, ms in zip(kernels, per):
+        d = by_name.setdefault(k["name"] if k["kind"] == "mfma" else ("generated" if k["kind"] == "generated" else "fill"),
+                               {"ms": 0.0, "flops": 0.0, "bytes": 0.0, "n": 0, "kind": k["kind"], "idx": []})
+        d["ms"] += ms; d["flops"] += k["flops"]; d["bytes"] += k["bytes"]; d["n"] += 1
+    mfma_ms = sum(d["ms"] for d in by_name.values() if d["kind"] == "mfma")
+    mfma_fl = sum(d["flops"] for d in by_name.values() if d["kind"] == "mfma")
+    gen_ms = sum(ms for k, ms in zip(kernels, per) if k["kind"] != "mfma")
+    gen_by = sum(k["bytes"] for k in kernels if k["kind"] != "mfma")
+    # dominant single kernel NAME among mfma instantiations, or the longest generated kernel
+    cands = {n: d for n, d in by_name.items() if d["kind"] == "mfma"}
+    longest_gen = max(((ms, i) for i, (k, ms) in enumerate(zip(kernels, per)) if k["kind"] == "generated"), default=(0.0, -1))
+    if cands and max(d["ms"] for d in cands.values()) >= longest_gen[0]:
+        dom_name = max(cands, key=lambda n: cands[n]["ms"])
+        dom_idx = [i for i, k in enumerate(kernels) if k["kind"] == "mfma" and k["name"] == dom_name]
+        bound = "mfma"
+    else:
+        dom_idx = [longest_gen[1]]
+        dom_name = kernels[longest_gen[1]]["name"]
+        bound = "hbm"
+    if args.kernel_table:
+        for k, ms in sorted(zip(kernels, per), key=lambda x: -x[1])[:40]:
+            print(f"{ms*1e3:9.1f} us  {k['kind']:9s} {k['name'][:70]:70s} flops={k['flops']:.3g} bytes={k['bytes']:.3g} "
+                  f"mnk={k['m']}x{k['n']}x{k['k']}x{k['batch']} coop={k['coop_lanes']}", file=sys.stderr)
+
+    # ---- timed region: exactly K steps, device idle on both sides; the dominant kernel's launches
+    #      are bracketed with HIP events on the stream they run on
+    hip.rt.profile_kernel(-1)
+    for i in dom_idx:
+        hip.rt.profile_kernel(i)
+    hip.rt.profile_read()
+    B.await_(hip.ctx.dev)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    B.await_(hip.ctx.dev)
+    dt = time.perf_counter() - t0
+    dom_ms, dom_launches = hip.rt.profile_read()
+    hip.rt.profile_kernel(-1)
+    loss = None
+    if "loss" in w.nodes:
+        from ocannl_amd import workloads as W
+        loss = float(W.to_float(hip.get(w.nodes["loss"]), w.nodes["loss"].prec).ravel()[0])
+
+    avg_ms = dom_ms / max(dom_launches, 1)
+    if bound == "mfma":
+        per_launch = sum(kernels[i]["flops"] for i in dom_idx) / len(dom_idx)
+        achieved = per_launch / (avg_ms * 1e-3) / 1e12
+        f32 = "gemm_f32" in dom_name
+        peak = PEAKS["mfma_f32"] if f32 else PEAKS["mfma_bf16"]
+        roof = {"bound": "mfma", "kernel": dom_name, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+                "frac": achieved / peak, "traffic": None, "launches_per_step": len(dom_idx),
+                "avg_launch_ms": avg_ms, "flops_per_launch": per_launch}
+    else:
+        per_launch = kernels[dom_idx[0]]["bytes"]
+        achieved = per_launch / (avg_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": PEAKS["hbm"], "unit": "GB/s",
+                "frac": achieved / PEAKS["hbm"], "traffic": None, "launches_per_step": 1, "avg_launch_ms": avg_ms,
+                "bytes_per_launch": per_launch}
+
+    out = {
+        "metric": metric, "value": args.steps / dt, "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {w.description}", "routine": w.routine.name,
+                   "kernels_per_step": len(kernels), "compile_s": round(compile_s, 2)},
+        "roofline": roof,
+        "einsum_tflops": (mfma_fl / (mfma_ms * 1e-3) / 1e12) if mfma_ms > 0 else None,
+        "einsum_ms_per_step": mfma_ms,
+        "pointwise_gbps": (gen_by / (gen_ms * 1e-3) / 1e9) if gen_ms > 0 else None,
+        "pointwise_ms_per_step": gen_ms,
+        "final_loss": loss,
+    }
+    hip.close()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

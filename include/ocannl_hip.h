@@ -132,8 +132,9 @@ int ocannl_hip_routine_run(ocannl_hip_routine* routine);
    per-kernel milliseconds (cap >= number of kernels).  For measurement only. */
 int ocannl_hip_routine_run_timed(ocannl_hip_routine* routine, float* kernel_ms, int cap);
 
-/* Measurement inside a timed region: bracket only kernel `kernel_index` (-1: none) of every following
-   ocannl_hip_routine_run with HIP events on the device stream, without synchronising. */
+/* Measurement inside a timed region: also bracket kernel `kernel_index` of every following
+   ocannl_hip_routine_run with HIP events on the device stream, without synchronising; may be called
+   for several kernels, -1 clears the selection. */
 int ocannl_hip_routine_profile_kernel(ocannl_hip_routine* routine, int kernel_index);
 /* Synchronises, returns the summed duration and the number of bracketed launches since the last read. */
 int ocannl_hip_routine_profile_read(ocannl_hip_routine* routine, double* total_ms, int64_t* launches);

@@ -21,6 +21,8 @@
 // fp32 compute uses v_mfma_f32_32x32x2_f32 with the same staging.
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
+
 #include "gemm.hpp"
 
 namespace ocannl {
@@ -188,19 +190,24 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_kernel(const GemmArgs g) {
 
   Stager<BM, AT, A_KC> sa;
   Stager<BN, BT, B_KC> sb;
-  sa.load(A, lda, m0, 0, g.M, g.K, tid);
-  sb.load(B, ldb, n0, 0, g.N, g.K, tid);
+  // split-K: blockIdx.y owns a contiguous range of K steps
+  const long all_steps = (g.K + kBK - 1) / kBK;
+  const long per_split = (all_steps + g.splits - 1) / g.splits;
+  const long kbeg = (long)blockIdx.y * per_split * kBK;
+  const long kend = (kbeg + per_split * kBK) < g.K ? (kbeg + per_split * kBK) : g.K;
+  sa.load(A, lda, m0, kbeg, g.M, kend, tid);
+  sb.load(B, ldb, n0, kbeg, g.N, kend, tid);
   sa.store(As0, tid);
   sb.store(Bs0, tid);
   __syncthreads();
 
-  const long ksteps = (g.K + kBK - 1) / kBK;
+  const long ksteps = kend > kbeg ? (kend - kbeg + kBK - 1) / kBK : 0;
   for (long ks = 0; ks < ksteps; ++ks) {
     const int cur = ks & 1;
     const bool more = ks + 1 < ksteps;
     if (more) {
-      sa.load(A, lda, m0, (ks + 1) * kBK, g.M, g.K, tid);
-      sb.load(B, ldb, n0, (ks + 1) * kBK, g.N, g.K, tid);
+      sa.load(A, lda, m0, kbeg + (ks + 1) * kBK, g.M, kend, tid);
+      sb.load(B, ldb, n0, kbeg + (ks + 1) * kBK, g.N, kend, tid);
     }
     const unsigned short* as = As0 + cur * BM * kStride + (wm0 + (lane & 31)) * kStride + (lane >> 5) * 8;
     const unsigned short* bs = Bs0 + cur * BN * kStride + (wn0 + (lane & 31)) * kStride + (lane >> 5) * 8;
@@ -239,7 +246,9 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_kernel(const GemmArgs g) {
         if (m >= g.M) continue;
         const long off = co + m * ldc + n;
         float v = acc[i][j][e];
-        if (g.c_is_bf16) {
+        if (g.splits > 1) {   // partial sums go to the workspace [batch][split][M][N]
+          g.ws[(((long)blockIdx.z * g.splits + blockIdx.y) * g.M + m) * g.N + n] = v;
+        } else if (g.c_is_bf16) {
           unsigned short* C = static_cast<unsigned short*>(g.c);
           if (g.accumulate) v += __uint_as_float(((unsigned)C[off]) << 16);
           C[off] = (unsigned short)f2bf(v);
@@ -347,19 +356,24 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g) {
 
   StagerF<BM, A_KC> sa;
   StagerF<BN, B_KC> sb;
-  sa.load(A, lda, m0, 0, g.M, g.K, tid);
-  sb.load(B, ldb, n0, 0, g.N, g.K, tid);
+  // split-K: blockIdx.y owns a contiguous range of K steps
+  const long all_steps = (g.K + kBKf - 1) / kBKf;
+  const long per_split = (all_steps + g.splits - 1) / g.splits;
+  const long kbeg = (long)blockIdx.y * per_split * kBKf;
+  const long kend = (kbeg + per_split * kBKf) < g.K ? (kbeg + per_split * kBKf) : g.K;
+  sa.load(A, lda, m0, kbeg, g.M, kend, tid);
+  sb.load(B, ldb, n0, kbeg, g.N, kend, tid);
   sa.store(As0, tid);
   sb.store(Bs0, tid);
   __syncthreads();
 
-  const long ksteps = (g.K + kBKf - 1) / kBKf;
+  const long ksteps = kend > kbeg ? (kend - kbeg + kBKf - 1) / kBKf : 0;
   for (long ks = 0; ks < ksteps; ++ks) {
     const int cur = ks & 1;
     const bool more = ks + 1 < ksteps;
     if (more) {
-      sa.load(A, lda, m0, (ks + 1) * kBKf, g.M, g.K, tid);
-      sb.load(B, ldb, n0, (ks + 1) * kBKf, g.N, g.K, tid);
+      sa.load(A, lda, m0, kbeg + (ks + 1) * kBKf, g.M, kend, tid);
+      sb.load(B, ldb, n0, kbeg + (ks + 1) * kBKf, g.N, kend, tid);
     }
     const float* as = As0 + cur * BM * kStride + (wm0 + (lane & 31)) * kStride + (lane >> 5) * 4;
     const float* bs = Bs0 + cur * BN * kStride + (wn0 + (lane & 31)) * kStride + (lane >> 5) * 4;
@@ -399,7 +413,9 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g) {
         if (m >= g.M) continue;
         const long off = co + m * ldc + n;
         float v = acc[i][j][e];
-        if (g.c_is_bf16) {
+        if (g.splits > 1) {   // partial sums go to the workspace [batch][split][M][N]
+          g.ws[(((long)blockIdx.z * g.splits + blockIdx.y) * g.M + m) * g.N + n] = v;
+        } else if (g.c_is_bf16) {
           unsigned short* C = static_cast<unsigned short*>(g.c);
           if (g.accumulate) v += __uint_as_float(((unsigned)C[off]) << 16);
           C[off] = (unsigned short)f2bf(v);
@@ -418,8 +434,63 @@ constexpr size_t bf16_smem() { return 2ull * (BM + BN) * (kBK + kPad) * sizeof(u
 template <int BM, int BN>
 constexpr size_t f32_smem() { return 2ull * (BM + BN) * (kBKf + kPadf) * sizeof(float); }
 
+// Sums the split-K partials in split order (deterministic) and applies them to C.
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const GemmArgs g) {
+  const long n4 = g.N / 4;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= g.M * n4) return;
+  const long m = idx / n4, n = (idx % n4) * 4;
+  long ao, bo, co;
+  decode_batch(g, blockIdx.z, ao, bo, co);
+  f32x4 sum = {0, 0, 0, 0};
+  for (int sp = 0; sp < g.splits; ++sp)
+    sum += *reinterpret_cast<const f32x4*>(g.ws + (((long)blockIdx.z * g.splits + sp) * g.M + m) * g.N + n);
+  const long off = co + m * g.c_row + n;
+  if (g.c_is_bf16) {
+    unsigned short* C = static_cast<unsigned short*>(g.c);
+    for (int q = 0; q < 4; ++q) {
+      float v = sum[q];
+      if (g.accumulate) v += __uint_as_float(((unsigned)C[off + q]) << 16);
+      C[off + q] = (unsigned short)f2bf(v);
+    }
+  } else {
+    float* C = static_cast<float*>(g.c);
+    f32x4 v = sum;
+    if (g.accumulate) v += *reinterpret_cast<const f32x4*>(C + off);
+    *reinterpret_cast<f32x4*>(C + off) = v;
+  }
+}
+
+long batch_count(const GemmDesc& d) {
+  long nb = 1;
+  for (int i = 0; i < d.nbatch; ++i) nb *= d.batch_ext[i];
+  return nb;
+}
+
+bool big_tile(const GemmDesc& d) {
+  // 256x256 tiles only when they still fill the chip (>= 256 workgroups)
+  const double tiles = ((d.M + 255) / 256) * (double)((d.N + 255) / 256) * (double)batch_count(d);
+  return tiles >= 256;
+}
+
+// Split K when the output has too few tiles to occupy the 256 CUs and K is long enough that every
+// split still runs at least four K stages.
+int split_count(const GemmDesc& d) {
+  const int tile = big_tile(d) ? 256 : 128;
+  const bool f32 = d.a.prec == Prec::Single && d.b.prec == Prec::Single;
+  const long bk = f32 ? kBKf : kBK;
+  const long tiles = ((d.M + tile - 1) / tile) * ((d.N + tile - 1) / tile) * batch_count(d);
+  if (tiles >= 192) return 1;
+  const long ksteps = (d.K + bk - 1) / bk;
+  long want = (256 + tiles - 1) / tiles;
+  long cap = ksteps / 4;
+  long s = want < cap ? want : cap;
+  if (s > 64) s = 64;
+  return s < 2 ? 1 : (int)s;
+}
+
 template <typename K>
-hipError_t launch(K kernel, size_t smem, int BM, int BN, const GemmArgs& a, hipStream_t s) {
+hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t s) {
   static thread_local const void* configured[64];
   static thread_local int n_configured = 0;
   bool done = false;
@@ -433,7 +504,12 @@ hipError_t launch(K kernel, size_t smem, int BM, int BN, const GemmArgs& a, hipS
   long nb = 1;
   for (int i = 0; i < a.nbatch; ++i) nb *= a.batch_ext[i];
   if (tiles <= 0 || tiles > 0x7FFFFFFFL || nb <= 0 || nb > 65535) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, 1, (unsigned)nb), dim3(kThreads), smem, s, a);
+  if (a.splits > 1 && !a.ws) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)a.splits, (unsigned)nb), dim3(kThreads), smem, s, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || a.splits <= 1) return e;
+  const long groups = a.M * (a.N / 4);
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((groups + 255) / 256), 1, (unsigned)nb), dim3(256), 0, s, a);
   return hipGetLastError();
 }
 
@@ -457,24 +533,32 @@ hipError_t launch_f32_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t 
 
 bool a_kcontig(const GemmDesc& d) { return d.a.s_k == 1 || d.K == 1; }
 bool b_kcontig(const GemmDesc& d) { return d.b.s_k == 1 || d.K == 1; }
-bool big_tile(const GemmDesc& d) {
-  // 256x256 tiles only when they still fill the chip (>= 256 workgroups)
-  double nb = 1;
-  for (int i = 0; i < d.nbatch; ++i) nb *= (double)d.batch_ext[i];
-  const double tiles = ((d.M + 255) / 256) * (double)((d.N + 255) / 256) * nb;
-  return tiles >= 256;
-}
 
 }  // namespace
 
 const char* gemm_kernel_name(const GemmDesc& d) {
-  const bool f32 = d.a.prec == Prec::Single && d.b.prec == Prec::Single;
-  const bool big = big_tile(d);
-  if (f32) return big ? "gemm_f32_kernel<256,256>" : "gemm_f32_kernel<128,128>";
-  return big ? "gemm_bf16_kernel<256,256>" : "gemm_bf16_kernel<128,128>";
+  // the instantiation as a profiler prints it (without namespaces)
+  static thread_local char buf[128];
+  const bool af = d.a.prec == Prec::Single, bf = d.b.prec == Prec::Single;
+  const int tile = big_tile(d) ? 256 : 128;
+  const char* tf[2] = {"false", "true"};
+  if (af && bf)
+    snprintf(buf, sizeof buf, "gemm_f32_kernel<%d, %d, %s, %s>", tile, tile, tf[a_kcontig(d)], tf[b_kcontig(d)]);
+  else
+    snprintf(buf, sizeof buf, "gemm_bf16_kernel<%d, %d, %s, %s, %s, %s>", tile, tile, af ? "float" : "unsigned short",
+             bf ? "float" : "unsigned short", tf[a_kcontig(d)], tf[b_kcontig(d)]);
+  return buf;
 }
 
-hipError_t launch_gemm(const GemmDesc& d, const GemmArgs& a, hipStream_t s) {
+size_t gemm_workspace_bytes(const GemmDesc& d) {
+  const int sp = split_count(d);
+  return sp > 1 ? (size_t)sp * (size_t)batch_count(d) * (size_t)d.M * (size_t)d.N * sizeof(float) : 0;
+}
+
+hipError_t launch_gemm(const GemmDesc& d, const GemmArgs& a_in, void* workspace, hipStream_t s) {
+  GemmArgs a = a_in;
+  a.splits = split_count(d);
+  a.ws = static_cast<float*>(workspace);
   const bool akc = a_kcontig(d), bkc = b_kcontig(d);
   const bool big = big_tile(d);
   const bool af = d.a.prec == Prec::Single, bf = d.b.prec == Prec::Single;

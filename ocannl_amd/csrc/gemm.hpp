@@ -18,11 +18,17 @@ struct GemmArgs {
   int64_t a_batch[3], b_batch[3], c_batch[3];
   int accumulate;    // beta = 1
   int c_is_bf16;
+  int splits;        // split-K factor (set by launch_gemm)
+  float* ws;         // split-K workspace [batch][split][M][N] (set by launch_gemm)
 };
 
 // Picks the kernel instance for the operand precisions / layouts and launches it on `stream`.
 // Returns hipErrorInvalidValue for a combination the planner should not have produced.
-hipError_t launch_gemm(const GemmDesc& desc, const GemmArgs& args, hipStream_t stream);
+// `workspace` must hold gemm_workspace_bytes(desc) bytes (may be null when that is 0).
+hipError_t launch_gemm(const GemmDesc& desc, const GemmArgs& args, void* workspace, hipStream_t stream);
+
+// Bytes of split-K workspace this contraction needs (0 when K is not split).
+size_t gemm_workspace_bytes(const GemmDesc& desc);
 
 // Name of the instance launch_gemm would pick (for kernel_info and profiles).
 const char* gemm_kernel_name(const GemmDesc& desc);

@@ -128,6 +128,7 @@ struct ocannl_hip_routine {
   hipModule_t module = nullptr;
   void* scratch = nullptr;
   uint64_t scratch_bytes = 0;
+  void* gemm_ws = nullptr;           // split-K workspace inside the scratch arena
   std::map<int, void*> node_ptr;
   std::map<int, int64_t> statics;    // symbol -> current value
   struct Launch {
@@ -142,7 +143,7 @@ struct ocannl_hip_routine {
   };
   std::vector<Launch> launches;
   std::vector<hipEvent_t> timing_events;
-  int profile_kernel = -1;
+  std::vector<char> profile_mask;           // kernels bracketed with events in plain runs
   std::vector<hipEvent_t> profile_events;   // pairs (start, stop), reused after each read
   size_t profile_used = 0;
 };
@@ -192,7 +193,7 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
   for (size_t li = 0; li < rt.launches.size(); ++li) {
     auto& l = rt.launches[li];
     const Phase& ph = rt.code->plan.phases[l.phase];
-    const bool bracket = !timed && rt.profile_kernel == (int)li;
+    const bool bracket = !timed && li < rt.profile_mask.size() && rt.profile_mask[li];
     if (bracket) {
       while (rt.profile_events.size() < rt.profile_used + 2) {
         hipEvent_t e;
@@ -225,7 +226,7 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
       }
       a.accumulate = g.accumulate ? 1 : 0;
       a.c_is_bf16 = g.c.prec == Prec::Bfloat16;
-      hip_check(launch_gemm(g, a, dev.stream), "launch_gemm");
+      hip_check(launch_gemm(g, a, rt.gemm_ws, dev.stream), "launch_gemm");
     }
     if (timed) hip_check(hipEventRecord(rt.timing_events[li + 1], dev.stream), "hipEventRecord");
     if (bracket) {
@@ -599,8 +600,14 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
       local_off[n.id] = arena;
       arena += ((uint64_t)n.size_in_bytes() + 255) / 256 * 256;
     }
+    uint64_t ws_bytes = 0;
+    for (auto& ph : cr.plan.phases)
+      if (ph.kind == Phase::Contraction) ws_bytes = std::max<uint64_t>(ws_bytes, gemm_workspace_bytes(ph.gemm));
+    const uint64_t ws_off = arena;
+    arena += (ws_bytes + 255) / 256 * 256;
     if (arena) {
       hip_check(hipMalloc(&rt->scratch, arena), "hipMalloc(scratch)");
+      if (ws_bytes) rt->gemm_ws = static_cast<char*>(rt->scratch) + ws_off;
       rt->scratch_bytes = arena;
       dev->scratch_used += arena;
     }
@@ -699,7 +706,9 @@ int ocannl_hip_routine_profile_kernel(ocannl_hip_routine* rt, int kernel_index) 
   return guarded([&] {
     if (!rt) throw InvalidArgument("profile_kernel: null routine");
     if (kernel_index >= (int)rt->launches.size()) throw InvalidArgument("profile_kernel: kernel index out of range");
-    rt->profile_kernel = kernel_index;
+    if (kernel_index < 0) { rt->profile_mask.clear(); return; }
+    rt->profile_mask.resize(rt->launches.size(), 0);
+    rt->profile_mask[kernel_index] = 1;
   });
 }
 

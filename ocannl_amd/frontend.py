@@ -236,14 +236,15 @@ class Graph:
 
     einsum = mul
 
-    def div(self, a, b, out_axes=None, ident="div"):
+    def div(self, a, b, out_axes=None, ident="div", prec=None):
         out_axes = out_axes or self._union_axes(a, b)
-        return self.nary(ident, [a, b], out_axes, lambda x, y: L.Binop("div", x, y),
+        return self.nary(ident, [a, b], out_axes, lambda x, y: L.Binop("div", x, y), prec=prec, grad_fns=
                          [lambda g, v, x, y: L.Binop("div", g, y),
                           lambda g, v, x, y: L.Binop("mul", g, L.Binop(
                               "div", L.Binop("mul", L.Const(-1.0), x), L.Binop("mul", y, y)))])
 
-    def unary(self, op: str, a: T, ident: Optional[str] = None):
+
+    def unary(self, op: str, a: T, ident: Optional[str] = None, prec=None):
         rules = {   # tensor/operation.ml:163-296
             "relu": lambda g, v, x: L.Binop("relu_gate", x, g),
             "exp": lambda g, v, x: L.Binop("mul", g, v),
@@ -254,9 +255,9 @@ class Graph:
             "recip": lambda g, v, x: L.Binop("mul", g, L.Binop("mul", L.Const(-1.0), L.Binop("mul", v, v))),
             "id": lambda g, v, x: g,
         }
-        return self.nary(ident or op, [a], a.axes, lambda x: L.Unop(op, x) if op != "id" else x, [rules[op]])
+        return self.nary(ident or op, [a], a.axes, lambda x: L.Unop(op, x) if op != "id" else x, [rules[op]], prec=prec)
 
-    def reduce(self, a: T, out_axes: Sequence[str], accum: str = "add", ident: Optional[str] = None):
+    def reduce(self, a: T, out_axes: Sequence[str], accum: str = "add", ident: Optional[str] = None, prec=None):
         """``einsum1`` / ``einmax1`` (tensor/operation.ml:504-508,583-593)."""
         if accum == "add":
             gfn = lambda g, v, x: g
@@ -265,7 +266,7 @@ class Graph:
         else:
             raise ValueError(accum)
         return self.nary(ident or ("sum" if accum == "add" else accum), [a], out_axes, lambda x: x, [gfn],
-                         accum=accum)
+                         accum=accum, prec=prec)
 
     def where(self, cond: T, a, b, ident="where"):
         """tensor/operation.ml:455-464: no gradient to the predicate."""

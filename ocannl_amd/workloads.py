@@ -347,8 +347,6 @@ def transformer(batch: int = 32, seq: int = 256, d_model: int = 512, heads: int 
         scores = g.div(g.einsum(q, k, ("b", "s", "h", "t"), ident=f"qk_{lb}"), ConstT(float(np.sqrt(dk))),
                        ("b", "s", "h", "t"), ident=f"scores_{lb}")
         masked = g.where(mask, scores, ConstT(-1e9), ident=f"masked_{lb}")
-        masked = T(masked.value, ("s", "t", "b", "h"), masked.grad, masked.children, masked.fwd, masked.bwd, masked.label) \
-            if False else masked
         attn = softmax(g, _reorder(g, masked, ("b", "s", "h", "t")), "t", ident=f"attn_{lb}")
         att_out = g.einsum(attn, v, ("b", "s", "h", "e"), ident=f"attn_out_{lb}")
         mha = g.einsum(w_o, att_out, ("b", "s", "m"), ident=f"mha_{lb}")
@@ -365,9 +363,12 @@ def transformer(batch: int = 32, seq: int = 256, d_model: int = 512, heads: int 
     logits = g.einsum(w_out, x, ("b", "s", "v"), ident="logits")
     counts = g.unary("exp", logits, ident="counts")
     probs = g.div(counts, g.reduce(counts, ("b", "s"), ident="counts_sum"), ("b", "s", "v"), ident="probs")
-    output_probs = g.reduce(g.mul(probs, target, ("b", "s", "v")), ("b", "s"), ident="output_probs")
-    tok_loss = g.unary("neg", g.unary("log", output_probs), ident="loss")
-    batch_loss = g.div(g.reduce(tok_loss, ("l",), ident="loss_sum"), ConstT(float(batch * seq)), ("l",), ident="batch_loss")
+    # the loss reduction is kept in single precision (Tn.update_prec on the loss nodes): a bfloat16
+    # running sum of 8192 token losses saturates
+    output_probs = g.reduce(g.mul(probs, target, ("b", "s", "v")), ("b", "s"), ident="output_probs", prec="single")
+    tok_loss = g.unary("neg", g.unary("log", output_probs, prec="single"), ident="loss", prec="single")
+    batch_loss = g.div(g.reduce(tok_loss, ("l",), ident="loss_sum", prec="single"), ConstT(float(batch * seq)), ("l",),
+                       ident="batch_loss", prec="single")
     batch_loss.label = "batch_loss"
     body = g.grad_update(batch_loss) + g.sgd_update(params, lrate)
     routine = make_routine(g, "transformer_sgd_step", body, [], inline=inline, outputs=[batch_loss.value])

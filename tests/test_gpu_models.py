@@ -77,7 +77,7 @@ def test_transformer_step(prec, tol, steps):
     assert sum(k["kind"] == "mfma" for k in hip.code.kernels()) >= 10
     for _ in range(steps):
         hip.step(); ora.step()
-        lh = float(W.to_float(hip.get(w.nodes["loss"]), prec)[0]); lo = float(ora.get(wr.nodes["loss"])[0])
+        lh = float(W.to_float(hip.get(w.nodes["loss"]), w.nodes["loss"].prec)[0]); lo = float(ora.get(wr.nodes["loss"])[0])
         assert abs(lh - lo) <= tol * max(abs(lo), 1.0), (lh, lo)
     for name in ("w_embed", "w_q_l0", "w_ffn2_l1", "w_out", "gamma_ln1_l0", "pos_encoding"):
         assert _err(W.to_float(hip.get(w.nodes[name]), prec), ora.get(wr.nodes[name]), prec) <= tol, name

@@ -98,3 +98,52 @@ def test_dense_contraction_mfma_small(prec, out_prec, tol, order):
         else:
             assert rel_err(got, want, out_prec) <= tol, name
     hip.close()
+
+
+@pytest.mark.parametrize("prec,tol", [("bfloat16", 2e-2), ("single", 1e-4)])
+def test_dense_contraction_full_size_sampled_rows(prec, tol):
+    """BASELINE config 3 at full size (b=8192, i=o=4096): too large for the serial checker, so a
+    random sample of output rows is recomputed in float64 on the host from the same inputs."""
+    b, i, o = 8192, 4096, 4096
+    w = W.dense_contraction(b=b, i=i, o=o, prec=prec, out_prec="single")
+    hip = HipRun(w.routine, w.init)
+    assert [k["kind"] for k in hip.code.kernels()] == ["mfma"] * 3
+    hip.step()
+    x = W.to_float(w.init[w.nodes["x"].id], prec); wt = W.to_float(w.init[w.nodes["w"].id], prec)
+    dy = W.to_float(w.init[w.nodes["dy"].id], prec)
+    rng = np.random.default_rng(11)
+    rows = np.sort(rng.choice(b, 48, replace=False)); orows = np.sort(rng.choice(o, 48, replace=False))
+    y = hip.get(w.nodes["y"]).astype(np.float64)
+    want = x[rows] @ wt.T
+    assert np.max(np.abs(y[rows] - want)) / np.max(np.abs(want)) <= tol
+    dx = hip.get(w.nodes["dx"]).astype(np.float64)
+    want = dy[rows] @ wt
+    assert np.max(np.abs(dx[rows] - want)) / np.max(np.abs(want)) <= tol
+    dw = hip.get(w.nodes["dw"]).astype(np.float64)
+    want = dy[:, orows].T @ x
+    assert np.max(np.abs(dw[orows] - want)) / np.max(np.abs(want)) <= tol
+    # linearity in the accumulating gradients: a second run adds the same amount again
+    hip.step()
+    dx2 = hip.get(w.nodes["dx"]).astype(np.float64)
+    assert np.max(np.abs(dx2[rows] - 2 * dx[rows])) / np.max(np.abs(dx[rows])) <= 1e-5
+    hip.close()
+
+
+@pytest.mark.parametrize("prec,tol", [("single", 1e-4), ("bfloat16", 2e-2)])
+def test_split_k_weight_gradient_shape(prec, tol):
+    """Small output, long reduction (the dW shape): K is split over workgroups and the partials are
+    summed in a fixed order; two runs must agree bit for bit."""
+    w = W.dense_contraction(b=4096, i=128, o=128, prec=prec, out_prec="single", which=("dw",), reduce_order="first")
+    rng = np.random.default_rng(3)
+    w.init[w.nodes["dw"].id] = rng.standard_normal((128, 128)).astype(np.float32)
+    hip = HipRun(w.routine, w.init, "min_mfma_flops=1")
+    assert [k["kind"] for k in hip.code.kernels()] == ["mfma"]
+    hip.step()
+    got = hip.get(w.nodes["dw"]).astype(np.float64)
+    x = W.to_float(w.init[w.nodes["x"].id], prec); dy = W.to_float(w.init[w.nodes["dy"].id], prec)
+    want = w.init[w.nodes["dw"].id].astype(np.float64) + dy.T @ x
+    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) <= tol
+    hip2 = HipRun(w.routine, w.init, "min_mfma_flops=1")
+    hip2.step()
+    assert np.array_equal(hip2.get(w.nodes["dw"]).view(np.uint32), hip.get(w.nodes["dw"]).view(np.uint32))
+    hip.close(); hip2.close()
