@@ -22,6 +22,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <utility>
 
 #include "gemm.hpp"
 
@@ -32,6 +33,17 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Compile-time loop: the accumulator array is only ever indexed by constants, so it stays in
+// registers whatever the unroller decides.
+template <int N, typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl<N>(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
 
 constexpr int kThreads = 256;
 constexpr int kBK = 64;        // K elements per stage (bf16 compute)
@@ -45,30 +57,35 @@ __device__ __forceinline__ unsigned f2bf(float f) {   // round to nearest even, 
 }
 __device__ __forceinline__ unsigned pack2(float lo, float hi) { return f2bf(lo) | (f2bf(hi) << 16); }
 
-// 8 consecutive source elements -> 8 bf16 in a uint4
-template <typename T>
-__device__ __forceinline__ u32x4 load8(const T* p);
-template <>
-__device__ __forceinline__ u32x4 load8<unsigned short>(const unsigned short* p) {
-  return *reinterpret_cast<const u32x4*>(p);
-}
-template <>
-__device__ __forceinline__ u32x4 load8<float>(const float* p) {
-  const f32x4 x = *reinterpret_cast<const f32x4*>(p);
-  const f32x4 y = *reinterpret_cast<const f32x4*>(p + 4);
-  u32x4 r;
-  r.x = pack2(x.x, x.y); r.y = pack2(x.z, x.w); r.z = pack2(y.x, y.y); r.w = pack2(y.z, y.w);
-  return r;
-}
+// Raw staging type of 8 consecutive source elements: bf16 sources travel as one 16-byte vector,
+// fp32 sources as two; the fp32 -> bf16 rounding happens when the registers are written to LDS, so
+// that the global loads stay in flight while the previous tile is being multiplied.
+template <typename T> struct Raw8;
+template <> struct Raw8<unsigned short> {
+  u32x4 v;
+  __device__ __forceinline__ void zero() { v = u32x4{0, 0, 0, 0}; }
+  __device__ __forceinline__ void load(const unsigned short* p) { v = *reinterpret_cast<const u32x4*>(p); }
+  __device__ __forceinline__ u32x4 bf16() const { return v; }
+};
+template <> struct Raw8<float> {
+  f32x4 lo, hi;
+  __device__ __forceinline__ void zero() { lo = f32x4{0, 0, 0, 0}; hi = lo; }
+  __device__ __forceinline__ void load(const float* p) {
+    lo = *reinterpret_cast<const f32x4*>(p);
+    hi = *reinterpret_cast<const f32x4*>(p + 4);
+  }
+  __device__ __forceinline__ u32x4 bf16() const {
+    return u32x4{pack2(lo.x, lo.y), pack2(lo.z, lo.w), pack2(hi.x, hi.y), pack2(hi.z, hi.w)};
+  }
+};
 
+// Batch index -> element offsets.  Written with constant array indices only: a runtime index into
+// the by-value argument struct would force the whole struct into scratch memory.
 __device__ __forceinline__ void decode_batch(const GemmArgs& g, long z, long& ao, long& bo, long& co) {
   ao = bo = co = 0;
-  for (int i = g.nbatch - 1; i >= 0; --i) {
-    const long e = g.batch_ext[i];
-    const long q = z % e;
-    z /= e;
-    ao += q * g.a_batch[i]; bo += q * g.b_batch[i]; co += q * g.c_batch[i];
-  }
+  if (g.nbatch > 2) { const long e = g.batch_ext[2], q = z % e; z /= e; ao += q * g.a_batch[2]; bo += q * g.b_batch[2]; co += q * g.c_batch[2]; }
+  if (g.nbatch > 1) { const long e = g.batch_ext[1], q = z % e; z /= e; ao += q * g.a_batch[1]; bo += q * g.b_batch[1]; co += q * g.c_batch[1]; }
+  if (g.nbatch > 0) { const long e = g.batch_ext[0], q = z % e; ao += q * g.a_batch[0]; bo += q * g.b_batch[0]; co += q * g.c_batch[0]; }
 }
 
 // XCD-aware tile order: consecutive hardware workgroup ids land on different XCDs; give XCD x the
@@ -88,14 +105,17 @@ __device__ __forceinline__ void tile_of_block(long wg, long tiles_m, long tiles_
   tn = r / gm;
 }
 
-// ---- staging one operand tile: global -> registers ---------------------------------------------
-// ROWS x kBK tile starting at (row0, k0).  K-contiguous: thread owns chunks of 8 k at one row.
-// Row-contiguous: thread owns 8(k) x 8(row) blocks, transposed in registers.
+// ---- staging one operand tile: global -> registers -> LDS --------------------------------------
+// ROWS x kBK tile starting at (row0, k0).  K-contiguous: a thread owns chunks of 8 k at one row.
+// Row-contiguous: a thread owns 8(k) x 8(row) blocks which it transposes in registers on the way to
+// LDS; adjacent lanes take adjacent k-groups of the same rows, so that both the global loads (eight
+// 128-byte row pieces per instruction) and the LDS writes (eight lanes fill one padded row) are
+// conflict-free.
 template <int ROWS, typename T, bool KC>
 struct Stager {
-  static constexpr int kChunks = ROWS * (kBK / 8) / kThreads;   // 16-byte LDS chunks per thread
-  static constexpr int kBlocks = (ROWS + kThreads - 1) / kThreads;  // 8x8 blocks per thread (row-contiguous)
-  u32x4 regs[KC ? kChunks : kBlocks * 8];
+  static constexpr int kChunks = ROWS * (kBK / 8) / kThreads;        // 8-element chunks per thread
+  static constexpr int kBlocks = (ROWS + kThreads - 1) / kThreads;   // 8x8 blocks per thread
+  Raw8<T> regs[KC ? kChunks : kBlocks * 8];
 
   __device__ __forceinline__ void load(const T* base, long ld, long row0, long k0, long rows, long K, int tid) {
     if (KC) {
@@ -104,35 +124,19 @@ struct Stager {
         const int c = tid + kThreads * j;
         const long row = row0 + c / (kBK / 8);
         const long k = k0 + (c % (kBK / 8)) * 8;
-        u32x4 v = {0, 0, 0, 0};
-        if (row < rows && k < K) v = load8<T>(base + row * ld + k);
-        regs[j] = v;
+        regs[j].zero();
+        if (row < rows && k < K) regs[j].load(base + row * ld + k);
       }
     } else {
-      // blocks: (kBK/8) k-groups x (ROWS/8) row-chunks; kChunks/8 blocks per thread
 #pragma unroll
       for (int jb = 0; jb < kBlocks; ++jb) {
         const int blk = tid + kThreads * jb;
-        const long row = row0 + (blk % (ROWS / 8)) * 8;
-        const long kg = k0 + (blk / (ROWS / 8)) * 8;
-        u32x4 in[8];
+        const long kg = k0 + (blk % (kBK / 8)) * 8;
+        const long row = row0 + (blk / (kBK / 8)) * 8;
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) {
-          u32x4 v = {0, 0, 0, 0};
-          if (blk < ROWS && row < rows && kg + kk < K) v = load8<T>(base + (kg + kk) * ld + row);
-          in[kk] = v;
-        }
-        // transpose 8x8 of 16-bit: out[m] holds k = 0..7 for row m
-#pragma unroll
-        for (int m = 0; m < 8; ++m) {
-          unsigned w[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const unsigned lo = in[2 * j][m / 2], hi = in[2 * j + 1][m / 2];
-            w[j] = (m & 1) ? ((lo >> 16) | (hi & 0xFFFF0000u)) : ((lo & 0xFFFFu) | (hi << 16));
-          }
-          u32x4 o = {w[0], w[1], w[2], w[3]};
-          regs[jb * 8 + m] = o;
+          regs[jb * 8 + kk].zero();
+          if (blk < ROWS && row < rows && kg + kk < K) regs[jb * 8 + kk].load(base + (kg + kk) * ld + row);
         }
       }
     }
@@ -144,24 +148,63 @@ struct Stager {
 #pragma unroll
       for (int j = 0; j < kChunks; ++j) {
         const int c = tid + kThreads * j;
-        *reinterpret_cast<u32x4*>(lds + (c / (kBK / 8)) * kStride + (c % (kBK / 8)) * 8) = regs[j];
+        *reinterpret_cast<u32x4*>(lds + (c / (kBK / 8)) * kStride + (c % (kBK / 8)) * 8) = regs[j].bf16();
       }
     } else {
 #pragma unroll
       for (int jb = 0; jb < kBlocks; ++jb) {
         const int blk = tid + kThreads * jb;
         if (blk >= ROWS) break;
-        const int row = (blk % (ROWS / 8)) * 8, kg = (blk / (ROWS / 8)) * 8;
+        const int kg = (blk % (kBK / 8)) * 8, row = (blk / (kBK / 8)) * 8;
+        u32x4 in[8];
 #pragma unroll
-        for (int m = 0; m < 8; ++m)
-          *reinterpret_cast<u32x4*>(lds + (row + m) * kStride + kg) = regs[jb * 8 + m];
+        for (int kk = 0; kk < 8; ++kk) in[kk] = regs[jb * 8 + kk].bf16();
+        // transpose 8x8 of 16-bit: out[m] holds k = 0..7 for row m
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+          unsigned w[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const unsigned lo = in[2 * j][m / 2], hi = in[2 * j + 1][m / 2];
+            w[j] = (m & 1) ? ((lo >> 16) | (hi & 0xFFFF0000u)) : ((lo & 0xFFFFu) | (hi << 16));
+          }
+          *reinterpret_cast<u32x4*>(lds + (row + m) * kStride + kg) = u32x4{w[0], w[1], w[2], w[3]};
+        }
       }
     }
   }
 };
 
+// Epilogue for one 32x32 MFMA tile: the lane holds column `n`; register e holds row
+// m_base + 8*(e/4) + e%4.
+__device__ __forceinline__ void store_tile(const GemmArgs& g, const f32x16& t, long m_base, long n, long co) {
+  if (n >= g.N) return;
+  static_for<16>([&](auto ec) {
+    constexpr int e = decltype(ec)::value;
+    const long m = m_base + (e >> 2) * 8 + (e & 3);
+    if (m < g.M) {
+      float v = t[e];
+      const long off = co + m * g.c_row + n;
+      if (g.splits > 1) {   // partial sums go to the workspace [batch][split][M][N]
+        g.ws[(((long)blockIdx.z * g.splits + blockIdx.y) * g.M + m) * g.N + n] = v;
+      } else if (g.c_is_bf16) {
+        unsigned short* C = static_cast<unsigned short*>(g.c);
+        if (g.accumulate) v += __uint_as_float(((unsigned)C[off]) << 16);
+        C[off] = (unsigned short)f2bf(v);
+      } else {
+        float* C = static_cast<float*>(g.c);
+        if (g.accumulate) v += C[off];
+        C[off] = v;
+      }
+    }
+  });
+}
+
+// One wavefront per SIMD for the 256x256 tile (the 256 accumulator registers live in AGPRs and the
+// whole 512-register budget is available); two for the 128x128 tile.
 template <int BM, int BN, typename AT, typename BT, bool A_KC, bool B_KC>
-__global__ void __launch_bounds__(kThreads) gemm_bf16_kernel(const GemmArgs g) {
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, BM >= 256 ? 1 : 2)))
+gemm_bf16_kernel(const GemmArgs g) {
   constexpr int kStride = kBK + kPad;
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   extern __shared__ __align__(16) unsigned short smem[];
@@ -181,34 +224,46 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_kernel(const GemmArgs g) {
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
 
   f32x16 acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  static_for<TM>([&](auto ic) {
+    static_for<TN>([&](auto jc) {
+      static_for<16>([&](auto ec) { acc[decltype(ic)::value][decltype(jc)::value][decltype(ec)::value] = 0.0f; });
+    });
+  });
 
-  Stager<BM, AT, A_KC> sa;
-  Stager<BN, BT, B_KC> sb;
   // split-K: blockIdx.y owns a contiguous range of K steps
   const long all_steps = (g.K + kBK - 1) / kBK;
   const long per_split = (all_steps + g.splits - 1) / g.splits;
   const long kbeg = (long)blockIdx.y * per_split * kBK;
   const long kend = (kbeg + per_split * kBK) < g.K ? (kbeg + per_split * kBK) : g.K;
-  sa.load(A, lda, m0, kbeg, g.M, kend, tid);
-  sb.load(B, ldb, n0, kbeg, g.N, kend, tid);
-  sa.store(As0, tid);
-  sb.store(Bs0, tid);
+  const long ksteps = kend > kbeg ? (kend - kbeg + kBK - 1) / kBK : 0;
+
+  // Software pipeline.  LDS is double buffered; global loads run kPF tiles ahead of the tile being
+  // multiplied, held in kPF register sets.  One set is what the register file affords next to a
+  // 256-register accumulator; the code is written for any depth.
+  constexpr int kPF = (BM >= 256 && sizeof(AT) == 2 && sizeof(BT) == 2) ? 2 : 1;
+  Stager<BM, AT, A_KC> sa[kPF];
+  Stager<BN, BT, B_KC> sb[kPF];
+  sa[0].load(A, lda, m0, kbeg, g.M, kend, tid);
+  sb[0].load(B, ldb, n0, kbeg, g.N, kend, tid);
+  if (kPF > 1) {
+    sa[kPF - 1].load(A, lda, m0, kbeg + kBK, g.M, kend, tid);
+    sb[kPF - 1].load(B, ldb, n0, kbeg + kBK, g.N, kend, tid);
+  }
+  sa[0].store(As0, tid);
+  sb[0].store(Bs0, tid);
   __syncthreads();
 
-  const long ksteps = kend > kbeg ? (kend - kbeg + kBK - 1) / kBK : 0;
-  for (long ks = 0; ks < ksteps; ++ks) {
+  // one K step; `par` = ks % kPF is a compile-time constant so that the register sets are
+  // addressed statically
+  auto step = [&](long ks, auto par_c) __attribute__((always_inline)) {
+    constexpr int par = decltype(par_c)::value;
     const int cur = ks & 1;
-    const bool more = ks + 1 < ksteps;
-    if (more) {
-      sa.load(A, lda, m0, kbeg + (ks + 1) * kBK, g.M, kend, tid);
-      sb.load(B, ldb, n0, kbeg + (ks + 1) * kBK, g.N, kend, tid);
+    // register set `par` held tile ks (already in LDS): refill it with tile ks + kPF
+    if (ks + kPF < ksteps) {
+      sa[par].load(A, lda, m0, kbeg + (ks + kPF) * kBK, g.M, kend, tid);
+      sb[par].load(B, ldb, n0, kbeg + (ks + kPF) * kBK, g.N, kend, tid);
     }
+    __builtin_amdgcn_sched_barrier(0);   // the loads are issued before the MFMA block, not sunk below it
     const unsigned short* as = As0 + cur * BM * kStride + (wm0 + (lane & 31)) * kStride + (lane >> 5) * 8;
     const unsigned short* bs = Bs0 + cur * BN * kStride + (wn0 + (lane & 31)) * kStride + (lane >> 5) * 8;
 #pragma unroll
@@ -218,48 +273,35 @@ __global__ void __launch_bounds__(kThreads) gemm_bf16_kernel(const GemmArgs g) {
       for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(as + i * 32 * kStride + kk * 16);
 #pragma unroll
       for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(bs + j * 32 * kStride + kk * 16);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
+      static_for<TM>([&](auto ic) {
+        static_for<TN>([&](auto jc) {
+          constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        });
+      });
     }
-    if (more) {
-      sa.store(As0 + (cur ^ 1) * BM * kStride, tid);
-      sb.store(Bs0 + (cur ^ 1) * BN * kStride, tid);
+    __builtin_amdgcn_sched_barrier(0);
+    // tile ks + 1 sits in the other register set (or, with one set, in the one just refilled)
+    if (ks + 1 < ksteps) {
+      constexpr int nxt = (par + 1) % kPF;
+      sa[nxt].store(As0 + (cur ^ 1) * BM * kStride, tid);
+      sb[nxt].store(Bs0 + (cur ^ 1) * BN * kStride, tid);
     }
     __syncthreads();
-  }
+  };
+  long ks = 0;
+  for (; ks + kPF <= ksteps; ks += kPF) static_for<kPF>([&](auto p) { step(ks + decltype(p)::value, p); });
+  static_for<kPF>([&](auto p) { if (ks + decltype(p)::value < ksteps) step(ks + decltype(p)::value, p); });
 
   // epilogue: lane holds column (lane % 32); register e holds row 8*(e/4) + 4*(lane/32) + e%4
-  const long ldc = g.c_row;
   const int col = lane & 31, rbase = (lane >> 5) * 4;
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const long n = n0 + wn0 + j * 32 + col;
-      if (n >= g.N) continue;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const long m = m0 + wm0 + i * 32 + (e >> 2) * 8 + rbase + (e & 3);
-        if (m >= g.M) continue;
-        const long off = co + m * ldc + n;
-        float v = acc[i][j][e];
-        if (g.splits > 1) {   // partial sums go to the workspace [batch][split][M][N]
-          g.ws[(((long)blockIdx.z * g.splits + blockIdx.y) * g.M + m) * g.N + n] = v;
-        } else if (g.c_is_bf16) {
-          unsigned short* C = static_cast<unsigned short*>(g.c);
-          if (g.accumulate) v += __uint_as_float(((unsigned)C[off]) << 16);
-          C[off] = (unsigned short)f2bf(v);
-        } else {
-          float* C = static_cast<float*>(g.c);
-          if (g.accumulate) v += C[off];
-          C[off] = v;
-        }
-      }
-    }
-  }
+  static_for<TM>([&](auto ic) {
+    static_for<TN>([&](auto jc) {
+      constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
+      store_tile(g, acc[i][j], m0 + wm0 + i * 32 + rbase, n0 + wn0 + j * 32 + col, co);
+      __builtin_amdgcn_sched_barrier(0);   // keep the tiles' loads/stores from piling up in registers
+    });
+  });
 }
 
 // ---- fp32 compute -------------------------------------------------------------------------------
@@ -326,7 +368,8 @@ struct StagerF {
 };
 
 template <int BM, int BN, bool A_KC, bool B_KC>
-__global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g) {
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, BM >= 256 ? 1 : 2)))
+gemm_f32_kernel(const GemmArgs g) {
   constexpr int kStride = kBKf + kPadf;
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   extern __shared__ __align__(16) unsigned short smem[];
@@ -347,12 +390,11 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g) {
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
 
   f32x16 acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  static_for<TM>([&](auto ic) {
+    static_for<TN>([&](auto jc) {
+      static_for<16>([&](auto ec) { acc[decltype(ic)::value][decltype(jc)::value][decltype(ec)::value] = 0.0f; });
+    });
+  });
 
   StagerF<BM, A_KC> sa;
   StagerF<BN, B_KC> sb;
@@ -384,13 +426,14 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g) {
       for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const f32x4*>(as + i * 32 * kStride + kk * 8);
 #pragma unroll
       for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const f32x4*>(bs + j * 32 * kStride + kk * 8);
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
+      static_for<4>([&](auto qc) {
+        static_for<TM>([&](auto ic) {
+          static_for<TN>([&](auto jc) {
+            constexpr int q = decltype(qc)::value, i = decltype(ic)::value, j = decltype(jc)::value;
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][q], bf[j][q], acc[i][j], 0, 0, 0);
+          });
+        });
+      });
     }
     if (more) {
       sa.store(As0 + (cur ^ 1) * BM * kStride, tid);
@@ -399,34 +442,14 @@ __global__ void __launch_bounds__(kThreads) gemm_f32_kernel(const GemmArgs g) {
     __syncthreads();
   }
 
-  const long ldc = g.c_row;
   const int col = lane & 31, rbase = (lane >> 5) * 4;
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const long n = n0 + wn0 + j * 32 + col;
-      if (n >= g.N) continue;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const long m = m0 + wm0 + i * 32 + (e >> 2) * 8 + rbase + (e & 3);
-        if (m >= g.M) continue;
-        const long off = co + m * ldc + n;
-        float v = acc[i][j][e];
-        if (g.splits > 1) {   // partial sums go to the workspace [batch][split][M][N]
-          g.ws[(((long)blockIdx.z * g.splits + blockIdx.y) * g.M + m) * g.N + n] = v;
-        } else if (g.c_is_bf16) {
-          unsigned short* C = static_cast<unsigned short*>(g.c);
-          if (g.accumulate) v += __uint_as_float(((unsigned)C[off]) << 16);
-          C[off] = (unsigned short)f2bf(v);
-        } else {
-          float* C = static_cast<float*>(g.c);
-          if (g.accumulate) v += C[off];
-          C[off] = v;
-        }
-      }
-    }
-  }
+  static_for<TM>([&](auto ic) {
+    static_for<TN>([&](auto jc) {
+      constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
+      store_tile(g, acc[i][j], m0 + wm0 + i * 32 + rbase, n0 + wn0 + j * 32 + col, co);
+      __builtin_amdgcn_sched_barrier(0);   // keep the tiles' loads/stores from piling up in registers
+    });
+  });
 }
 
 template <int BM, int BN>
