@@ -22,6 +22,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <type_traits>
 #include <utility>
 
 #include "gemm.hpp"
@@ -35,7 +36,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // Compile-time loop: the accumulator array is only ever indexed by constants, so it stays in
-// registers whatever the unroller decides.
+// registers whatever the unroller decides.  The loop bodies are lambdas that must be inlined too
+// (a body left as a call would take the accumulators' address and push them to scratch memory).
+#define OCN_LAMBDA_INLINE __attribute__((always_inline))
 template <int N, typename F, int... I>
 __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
   (f(std::integral_constant<int, I>{}), ...);
@@ -44,6 +47,16 @@ template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl<N>(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
 }
+
+// Phase timestamps for kernel tuning (compiled in only with -DOCANNL_GEMM_TIMING): workgroup w
+// writes the 100 MHz wall clock at stamp i to g_gemm_stamps[8 * w + i].
+#ifdef OCANNL_GEMM_TIMING
+__device__ long long g_gemm_stamps[8 * 4096];
+#define OCANNL_STAMP(i) \
+  do { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && blockIdx.x < 4096) g_gemm_stamps[8 * blockIdx.x + (i)] = wall_clock64(); } while (0)
+#else
+#define OCANNL_STAMP(i) do { } while (0)
+#endif
 
 constexpr int kThreads = 256;
 constexpr int kBK = 64;        // K elements per stage (bf16 compute)
@@ -175,28 +188,88 @@ struct Stager {
   }
 };
 
-// Epilogue for one 32x32 MFMA tile: the lane holds column `n`; register e holds row
-// m_base + 8*(e/4) + e%4.
-__device__ __forceinline__ void store_tile(const GemmArgs& g, const f32x16& t, long m_base, long n, long co) {
-  if (n >= g.N) return;
-  static_for<16>([&](auto ec) {
-    constexpr int e = decltype(ec)::value;
-    const long m = m_base + (e >> 2) * 8 + (e & 3);
-    if (m < g.M) {
-      float v = t[e];
-      const long off = co + m * g.c_row + n;
-      if (g.splits > 1) {   // partial sums go to the workspace [batch][split][M][N]
-        g.ws[(((long)blockIdx.z * g.splits + blockIdx.y) * g.M + m) * g.N + n] = v;
-      } else if (g.c_is_bf16) {
-        unsigned short* C = static_cast<unsigned short*>(g.c);
-        if (g.accumulate) v += __uint_as_float(((unsigned)C[off]) << 16);
-        C[off] = (unsigned short)f2bf(v);
-      } else {
-        float* C = static_cast<float*>(g.c);
-        if (g.accumulate) v += C[off];
-        C[off] = v;
+// ---- epilogue -----------------------------------------------------------------------------------
+// One wave's block of TM x TN accumulator tiles -> memory, one row of tiles (32 x TN*32) at a
+// time.  In a 32x32 tile the lane holds column lane % 32 and register e holds row
+// 8 * (e / 4) + 4 * (lane / 32) + e % 4, so one store instruction writes two 32-element row
+// pieces.  The address of an element splits into a part that is uniform over the wave (tile
+// origin + compile-time row/column: scalar registers) and one 32-bit per-lane offset computed
+// once.  ACC loads the whole row of tiles before the first store, so that TN * 16 reads are in
+// flight; CHECK guards ragged edges.
+enum : int { kOutF32 = 0, kOutBf16 = 1 };
+
+template <int TN, int OUT, bool ACC, bool CHECK>
+__device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, long ld, int lane,
+                                               long rows_left, long cols_left) {
+  using T = typename std::conditional<OUT == kOutBf16, unsigned short, float>::type;
+  T* const base = static_cast<T*>(origin);
+  const unsigned col = lane & 31, rb = (lane >> 5) * 4;
+  const unsigned loff = rb * (unsigned)ld + col;
+  // Pin the tiles to accumulation registers up to this point: without it the register allocator
+  // may move all accumulators of the block into ordinary registers right after the main loop and
+  // spill most of them.
+  static_assert(TN == 2 || TN == 4, "tile rows of 2 or 4 tiles");
+  asm volatile("" : "+a"(acc[0]), "+a"(acc[1]));
+  if constexpr (TN == 4) asm volatile("" : "+a"(acc[2]), "+a"(acc[3]));
+  float old[ACC ? TN : 1][16];
+  if (ACC) {
+    static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
+      static_for<16>([&](auto ec) OCN_LAMBDA_INLINE {
+        constexpr int j = decltype(jc)::value, e = decltype(ec)::value, r = (e >> 2) * 8 + (e & 3);
+        const T* p = base + (long)r * ld + j * 32;
+        float o = 0.0f;
+        if (!CHECK || ((long)(r + rb) < rows_left && (long)(j * 32 + col) < cols_left)) {
+          if (OUT == kOutBf16) o = __uint_as_float(((unsigned)p[loff]) << 16);
+          else o = p[loff];
+        }
+        old[ACC ? j : 0][e] = o;
+      });
+    });
+  }
+  static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
+    static_for<16>([&](auto ec) OCN_LAMBDA_INLINE {
+      constexpr int j = decltype(jc)::value, e = decltype(ec)::value, r = (e >> 2) * 8 + (e & 3);
+      T* p = base + (long)r * ld + j * 32;
+      float v = acc[j][e];
+      if (ACC) v += old[ACC ? j : 0][e];
+      if (!CHECK || ((long)(r + rb) < rows_left && (long)(j * 32 + col) < cols_left)) {
+        if (OUT == kOutBf16) p[loff] = (unsigned short)f2bf(v);
+        else p[loff] = v;
       }
+    });
+    __builtin_amdgcn_sched_barrier(0);   // one tile's registers at a time
+  });
+}
+
+// (m, n) is the origin of the wave's block.  The variant is picked per row of tiles with a
+// wave-uniform switch: that bounds what the compiler can hoist above the branch to one row's
+// registers (hoisting all 256 accumulator reads above one up-front branch spills them).
+template <int TM, int TN>
+__device__ __forceinline__ void epilogue(const GemmArgs& g, f32x16 (&acc)[TM][TN], long m, long n, long co, int lane) {
+  const long rows_left = g.M - m, cols_left = g.N - n;
+  if (rows_left <= 0 || cols_left <= 0) return;
+  const bool full = rows_left >= TM * 32 && cols_left >= TN * 32;
+  const bool to_ws = g.splits > 1;   // split-K partial sums go to the workspace [batch][split][M][N]
+  const bool bf = !to_ws && g.c_is_bf16;
+  const long ld = to_ws ? g.N : g.c_row;
+  const long first = to_ws ? (((long)blockIdx.z * g.splits + blockIdx.y) * g.M + m) * g.N + n : co + m * g.c_row + n;
+  char* const origin = (to_ws ? reinterpret_cast<char*>(g.ws) : static_cast<char*>(g.c)) + first * (bf ? 2 : 4);
+  const int variant = (bf ? 4 : 0) + ((!to_ws && g.accumulate) ? 2 : 0) + (full ? 0 : 1);
+  static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
+    constexpr int i = decltype(ic)::value;
+    void* o = origin + (long)i * 32 * ld * (bf ? 2 : 4);
+    const long rl = rows_left - i * 32;
+    switch (variant) {
+      case 0: store_tile_row<TN, kOutF32, false, false>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 1: store_tile_row<TN, kOutF32, false, true>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 2: store_tile_row<TN, kOutF32, true, false>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 3: store_tile_row<TN, kOutF32, true, true>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 4: store_tile_row<TN, kOutBf16, false, false>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 5: store_tile_row<TN, kOutBf16, false, true>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 6: store_tile_row<TN, kOutBf16, true, false>(acc[i], o, ld, lane, rl, cols_left); break;
+      default: store_tile_row<TN, kOutBf16, true, true>(acc[i], o, ld, lane, rl, cols_left); break;
     }
+    __builtin_amdgcn_sched_barrier(0);
   });
 }
 
@@ -211,7 +284,8 @@ gemm_bf16_kernel(const GemmArgs g) {
   unsigned short* const As0 = smem;
   unsigned short* const Bs0 = smem + 2 * BM * kStride;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  OCANNL_STAMP(0);
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
   const long tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
   long tmi, tni;
@@ -224,9 +298,9 @@ gemm_bf16_kernel(const GemmArgs g) {
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
 
   f32x16 acc[TM][TN];
-  static_for<TM>([&](auto ic) {
-    static_for<TN>([&](auto jc) {
-      static_for<16>([&](auto ec) { acc[decltype(ic)::value][decltype(jc)::value][decltype(ec)::value] = 0.0f; });
+  static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
+    static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
+      static_for<16>([&](auto ec) OCN_LAMBDA_INLINE { acc[decltype(ic)::value][decltype(jc)::value][decltype(ec)::value] = 0.0f; });
     });
   });
 
@@ -252,6 +326,7 @@ gemm_bf16_kernel(const GemmArgs g) {
   sa[0].store(As0, tid);
   sb[0].store(Bs0, tid);
   __syncthreads();
+  OCANNL_STAMP(1);
 
   // one K step; `par` = ks % kPF is a compile-time constant so that the register sets are
   // addressed statically
@@ -273,8 +348,8 @@ gemm_bf16_kernel(const GemmArgs g) {
       for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(as + i * 32 * kStride + kk * 16);
 #pragma unroll
       for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(bs + j * 32 * kStride + kk * 16);
-      static_for<TM>([&](auto ic) {
-        static_for<TN>([&](auto jc) {
+      static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
+        static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
           constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
         });
@@ -290,18 +365,12 @@ gemm_bf16_kernel(const GemmArgs g) {
     __syncthreads();
   };
   long ks = 0;
-  for (; ks + kPF <= ksteps; ks += kPF) static_for<kPF>([&](auto p) { step(ks + decltype(p)::value, p); });
-  static_for<kPF>([&](auto p) { if (ks + decltype(p)::value < ksteps) step(ks + decltype(p)::value, p); });
+  for (; ks + kPF <= ksteps; ks += kPF) static_for<kPF>([&](auto p) OCN_LAMBDA_INLINE { step(ks + decltype(p)::value, p); });
+  static_for<kPF>([&](auto p) OCN_LAMBDA_INLINE { if (ks + decltype(p)::value < ksteps) step(ks + decltype(p)::value, p); });
+  OCANNL_STAMP(2);
 
-  // epilogue: lane holds column (lane % 32); register e holds row 8*(e/4) + 4*(lane/32) + e%4
-  const int col = lane & 31, rbase = (lane >> 5) * 4;
-  static_for<TM>([&](auto ic) {
-    static_for<TN>([&](auto jc) {
-      constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
-      store_tile(g, acc[i][j], m0 + wm0 + i * 32 + rbase, n0 + wn0 + j * 32 + col, co);
-      __builtin_amdgcn_sched_barrier(0);   // keep the tiles' loads/stores from piling up in registers
-    });
-  });
+  epilogue<TM, TN>(g, acc, m0 + wm0, n0 + wn0, co, lane);
+  OCANNL_STAMP(3);
 }
 
 // ---- fp32 compute -------------------------------------------------------------------------------
@@ -377,7 +446,7 @@ gemm_f32_kernel(const GemmArgs g) {
   float* const As0 = fsm;
   float* const Bs0 = fsm + 2 * BM * kStride;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
   const long tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
   long tmi, tni;
@@ -390,9 +459,9 @@ gemm_f32_kernel(const GemmArgs g) {
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
 
   f32x16 acc[TM][TN];
-  static_for<TM>([&](auto ic) {
-    static_for<TN>([&](auto jc) {
-      static_for<16>([&](auto ec) { acc[decltype(ic)::value][decltype(jc)::value][decltype(ec)::value] = 0.0f; });
+  static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
+    static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
+      static_for<16>([&](auto ec) OCN_LAMBDA_INLINE { acc[decltype(ic)::value][decltype(jc)::value][decltype(ec)::value] = 0.0f; });
     });
   });
 
@@ -426,9 +495,9 @@ gemm_f32_kernel(const GemmArgs g) {
       for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const f32x4*>(as + i * 32 * kStride + kk * 8);
 #pragma unroll
       for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const f32x4*>(bs + j * 32 * kStride + kk * 8);
-      static_for<4>([&](auto qc) {
-        static_for<TM>([&](auto ic) {
-          static_for<TN>([&](auto jc) {
+      static_for<4>([&](auto qc) OCN_LAMBDA_INLINE {
+        static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
+          static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
             constexpr int q = decltype(qc)::value, i = decltype(ic)::value, j = decltype(jc)::value;
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][q], bf[j][q], acc[i][j], 0, 0, 0);
           });
@@ -442,14 +511,7 @@ gemm_f32_kernel(const GemmArgs g) {
     __syncthreads();
   }
 
-  const int col = lane & 31, rbase = (lane >> 5) * 4;
-  static_for<TM>([&](auto ic) {
-    static_for<TN>([&](auto jc) {
-      constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
-      store_tile(g, acc[i][j], m0 + wm0 + i * 32 + rbase, n0 + wn0 + j * 32 + col, co);
-      __builtin_amdgcn_sched_barrier(0);   // keep the tiles' loads/stores from piling up in registers
-    });
-  });
+  epilogue<TM, TN>(g, acc, m0 + wm0, n0 + wn0, co, lane);
 }
 
 template <int BM, int BN>

@@ -620,6 +620,14 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
         throw UserError("hip backend link: node " + n.ident + " (id " + std::to_string(n.id) + ") missing from context");
       rt->node_ptr[n.id] = dev->resolve(it->second->pool_id, it->second->offset, (uint64_t)n.size_in_bytes(), "link");
     }
+    // the MFMA kernels read 16-byte chunks relative to the node base
+    for (auto& ph : cr.plan.phases) {
+      if (ph.kind != Phase::Contraction) continue;
+      for (const GemmOperand* op : {&ph.gemm.a, &ph.gemm.b, &ph.gemm.c})
+        if (reinterpret_cast<uintptr_t>(rt->node_ptr.at(op->node)) % 16 != 0)
+          throw UserError("hip backend link: node " + cr.r.node(op->node).ident +
+                          " feeds a matrix-core contraction and must sit at a 16-byte aligned pool offset");
+    }
     for (auto& s : cr.r.statics) rt->statics[s.sym] = 0;
     if (!cr.binary.empty()) hip_check(hipModuleLoadData(&rt->module, cr.binary.data()), "hipModuleLoadData");
     // launch records

@@ -94,3 +94,26 @@ def test_link_reports_missing_node(dev):
     with pytest.raises(B.User_error):
         B.link(dev, B.compile(r), {1: (904, 0)})
     B.free_pool(dev, pool_id=904)
+
+
+def test_link_rejects_misaligned_contraction_operand(dev):
+    # the matrix-core kernels read 16-byte chunks: an operand packed at a 4-byte aligned offset
+    # (what element-size alignment alone would allow) is a user error, reported at link time
+    from ocannl_amd import workloads as W
+    w = W.dense_contraction(b=256, i=128, o=128, prec="single", out_prec="single")
+    code = B.compile(w.routine)
+    assert any(k["kind"] == "mfma" for k in code.kernels())
+    nodes = w.routine.param_nodes()
+    total, locs = 0, {}
+    for n in nodes:
+        locs[n.id] = (905, total)
+        total += (n.size_in_bytes + 255) // 256 * 256
+    B.alloc_pool(dev, pool_id=905, size_in_bytes=total + 256, alignment=256)
+    rt = B.link(dev, code, locs)          # aligned: fine
+    del rt
+    bad = dict(locs)
+    first = nodes[0].id
+    bad[first] = (905, locs[first][1] + 4)
+    with pytest.raises(B.User_error, match="16-byte"):
+        B.link(dev, code, bad)
+    B.free_pool(dev, pool_id=905)
