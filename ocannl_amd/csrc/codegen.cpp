@@ -278,10 +278,19 @@ bool reads_scope_before_set(const ScopeId& target, const Block& body) {
 // statement / scalar printer
 // ------------------------------------------------------------------------------------------------
 
+std::string neutral_literal(Binop accum, bool dbl);
+std::string combine_expr(Binop accum, bool dbl, const std::string& a, const std::string& b);
+
 struct Printer {
   const Routine& r;
   std::set<int> used_nodes;
   std::set<int> used_statics;
+  // when set, this inlined scalar reduction is shared by `coop_lanes` adjacent lanes (lane id in
+  // `lane_`): they stride its innermost loop, accumulate in float and combine by butterfly
+  // shuffles; the enclosing store is done by lane 0
+  const Scalar* coop_scope = nullptr;
+  int coop_lanes = 1;
+  Binop coop_accum = Binop::Add;
   // when set, a read of exactly this (node, indices) prints as `self_name`
   const Stmt* self_set = nullptr;
   std::string self_name;
@@ -308,6 +317,7 @@ struct Printer {
     switch (s.kind) {
       case Scalar::LocalScope: {
         const Prec sp = r.node(s.scope.node).prec;
+        if (&s == coop_scope) return coop_reduction(prec, s, ind, defs);
         Def d; d.scope = s.scope.scope;
         d.lines.push_back(ind + c_typ(sp) + " " + scope_name(s.scope) +
                           (reads_scope_before_set(s.scope, s.body) ? init_zero(sp) : "") + ";");
@@ -377,6 +387,65 @@ struct Printer {
     return "";
   }
 
+  // `v { v := neutral; for k1.. for kn { v := accum(v, e) } }` computed by a group of lanes.
+  std::string coop_reduction(Prec prec, const Scalar& s, const std::string& ind, std::vector<Def>& defs) {
+    const Prec sp = r.node(s.scope.node).prec;
+    const bool dbl = sp == Prec::Double;
+    const Prec accP = dbl ? Prec::Double : Prec::Single;
+    const std::string part = "part" + std::to_string(s.scope.scope) + "_";
+    auto only = [](const Block& b) -> const Stmt* {   // the single non-comment statement
+      const Stmt* one = nullptr;
+      for (auto& x : b) if (x->kind != Stmt::Comment) { if (one) return nullptr; one = x.get(); }
+      return one;
+    };
+    const Stmt* loop = nullptr;
+    for (auto& x : s.body) if (x->kind == Stmt::For) loop = x.get();
+    std::vector<const Stmt*> loops;
+    const Stmt* upd = nullptr;
+    for (const Stmt* cur = loop; cur;) {
+      loops.push_back(cur);
+      const Stmt* in = only(cur->body);
+      if (in && in->kind == Stmt::For) { cur = in; continue; }
+      upd = in;
+      break;
+    }
+    if (!upd || upd->kind != Stmt::SetLocal) throw InvalidArgument("codegen: cooperative scope lost its shape");
+    Def d; d.scope = s.scope.scope;
+    d.lines.push_back(ind + (dbl ? "double " : "float ") + part + " = " + neutral_literal(coop_accum, dbl) + ";");
+    std::string ci = ind;
+    for (size_t i = 0; i < loops.size(); ++i) {
+      const std::string sy = sym_ident(loops[i]->sym);
+      if (i + 1 == loops.size())
+        d.lines.push_back(ci + "for (uint32_t " + sy + " = " + std::to_string(loops[i]->from) + " + lane_; " + sy + " <= " +
+                          std::to_string(loops[i]->to) + "; " + sy + " += " + std::to_string(coop_lanes) + ") {");
+      else
+        d.lines.push_back(ci + "for (uint32_t " + sy + " = " + std::to_string(loops[i]->from) + "; " + sy + " <= " +
+                          std::to_string(loops[i]->to) + "; ++" + sy + ") {");
+      ci += "  ";
+    }
+    auto widen = [&](const std::string& e) { Pair c = convert_precision(sp, accP); return c.first + e + c.second; };
+    auto is_v = [&](const Scalar& x) { return x.kind == Scalar::GetLocal && x.scope == s.scope; };
+    const Scalar& v = *upd->value;
+    std::vector<Def> inner_defs;
+    std::string line;
+    if (v.kind == Scalar::Tern) {
+      const std::string a = scalar(sp, *v.a, ci + "  ", inner_defs), b = scalar(sp, *v.b, ci + "  ", inner_defs);
+      line = part + " = " + (dbl ? "fma(" : "fmaf(") + widen(a) + ", " + widen(b) + ", " + part + ");";
+    } else {
+      const std::string e = scalar(sp, is_v(*v.a) ? *v.b : *v.a, ci + "  ", inner_defs);
+      line = part + " = " + combine_expr(coop_accum, dbl, part, widen(e)) + ";";
+    }
+    with_defs(inner_defs, {line}, ci, d.lines);
+    for (size_t i = 0; i < loops.size(); ++i) { ci.resize(ci.size() - 2); d.lines.push_back(ci + "}"); }
+    for (int o = coop_lanes / 2; o > 0; o >>= 1)
+      d.lines.push_back(ind + part + " = " + combine_expr(coop_accum, dbl, part, "ocn_xshfl(" + part + ", " + std::to_string(o) + ")") + ";");
+    Pair narrow = convert_precision(accP, sp);
+    d.lines.push_back(ind + c_typ(sp) + " " + scope_name(s.scope) + " = " + narrow.first + part + narrow.second + ";");
+    defs.push_back(std::move(d));
+    Pair c = convert_precision(sp, prec);
+    return c.first + scope_name(s.scope) + c.second;
+  }
+
   void with_defs(std::vector<Def>& defs, const std::vector<std::string>& lines, const std::string& ind,
                  std::vector<std::string>& out) {
     if (defs.empty()) { for (auto& l : lines) out.push_back(ind + l); return; }
@@ -418,7 +487,8 @@ struct Printer {
         note(c.node, c.idcs);
         std::vector<Def> defs;
         std::string v = scalar(n.prec, *c.value, ind + "  ", defs);
-        with_defs(defs, {n.ident + "[" + offset_str(c.idcs, n.dims) + "] = " + v + ";"}, ind, out);
+        with_defs(defs, {std::string(coop_scope ? "if (lane_ == 0) " : "") + n.ident + "[" + offset_str(c.idcs, n.dims) +
+                         "] = " + v + ";"}, ind, out);
         break;
       }
       case Stmt::SetVec: {
@@ -549,7 +619,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     Binop accum = Binop::Add;
     bool is_reduction = false;
     const Stmt* set = nullptr;
-    if (!ph.seq_syms.empty() && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set) {
+    if ((!ph.seq_syms.empty() || ph.fused_zero_init) && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set) {
       set = ph.inner[0].get();
       const Scalar& v = *set->value;
       auto is_self = [&](const Scalar& s) { return s.kind == Scalar::Get && s.node == set->node && s.idcs == set->idcs; };
@@ -575,7 +645,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
       for (size_t i = 0; i < ph.seq_syms.size(); ++i) { cur_ind.resize(cur_ind.size() - 2); body.push_back(cur_ind + "}"); }
     };
 
-    if (is_reduction && G > 1) {
+    if (is_reduction && G > 1 && !ph.coop_scope) {
       // lanes of a group stride the innermost sequential loop; partials are combined by butterfly
       // shuffles in a fixed order (deterministic), accumulating in float (double for double).
       const Node& n = r.node(set->node);
@@ -622,17 +692,22 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
       std::string ci = ind;
       open_seq_loops(ci, false);
       pr.self_set = set; pr.self_name = "acc_";
+      if (ph.coop_scope) { pr.coop_scope = ph.coop_scope; pr.coop_lanes = G; pr.coop_accum = ph.coop_accum; }
       std::vector<Printer::Def> defs;
       std::string v = pr.scalar(n.prec, *set->value, ci + "  ", defs);
       pr.with_defs(defs, {"acc_ = " + v + ";"}, ci, body);
       pr.self_set = nullptr;
       close_seq_loops(ci);
-      body.push_back(ind + lhs + " = acc_;");
+      body.push_back(ind + (ph.coop_scope ? "if (lane_ == 0) " : "") + lhs + " = acc_;");
+      pr.coop_scope = nullptr;
     } else {
       if (ph.fused_zero_init) throw InvalidArgument("planner: fused zero-init on a non-reduction phase");
       std::string ci = ind;
       open_seq_loops(ci, false);
+      if (G > 1 && ph.coop_scope) { pr.coop_scope = ph.coop_scope; pr.coop_lanes = G; pr.coop_accum = ph.coop_accum; }
+      else if (G > 1) throw InvalidArgument("planner: lane group without a reduction to share");
       pr.block(ph.inner, ci, body);
+      pr.coop_scope = nullptr;
       close_seq_loops(ci);
     }
 

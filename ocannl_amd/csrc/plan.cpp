@@ -1,11 +1,14 @@
 #include "plan.hpp"
 
 #include <algorithm>
+#include <cmath>
 #include <functional>
 #include <set>
 
 namespace ocannl {
 namespace {
+
+Block strip_comments(const Block& b, std::string* last_comment);
 
 struct Access {
   int node;
@@ -299,9 +302,84 @@ bool reduction_shape(const Routine& r, const Phase& ph, Binop* accum_out) {
   return false;
 }
 
+// The inlined scalar reduction form `v { v := const; for k1.. for kn { v := accum(v, e) } }`
+// (low_level.ml:1165-1316) with e free of v.  Fills the reduction loops (outer first) and the update.
+bool scope_reduction(const Scalar& ls, std::vector<const Stmt*>& loops, const Stmt*& init, const Stmt*& upd,
+                     Binop* accum) {
+  if (ls.kind != Scalar::LocalScope) return false;
+  Block body = strip_comments(ls.body, nullptr);
+  if (body.size() != 2 || body[0]->kind != Stmt::SetLocal || !(body[0]->scope == ls.scope)) return false;
+  if (body[0]->value->kind != Scalar::Const || body[1]->kind != Stmt::For) return false;
+  init = body[0].get();
+  const Stmt* cur = body[1].get();
+  upd = nullptr;
+  for (;;) {
+    loops.push_back(cur);
+    Block b2 = strip_comments(cur->body, nullptr);
+    if (b2.size() != 1) return false;
+    if (b2[0]->kind == Stmt::For) { cur = b2[0].get(); continue; }
+    if (b2[0]->kind == Stmt::SetLocal && b2[0]->scope == ls.scope) upd = b2[0].get();
+    break;
+  }
+  if (!upd) return false;
+  std::function<bool(const Scalar&)> mentions = [&](const Scalar& s) -> bool {
+    if (s.kind == Scalar::GetLocal) return s.scope == ls.scope;
+    if (s.kind == Scalar::LocalScope) return true;   // nested scopes: leave alone
+    return (s.a && mentions(*s.a)) || (s.b && mentions(*s.b)) || (s.c && mentions(*s.c));
+  };
+  auto is_v = [&](const Scalar& s) { return s.kind == Scalar::GetLocal && s.scope == ls.scope; };
+  const Scalar& v = *upd->value;
+  if (v.kind == Scalar::Tern && v.tern == Ternop::Fma && is_v(*v.c) && !mentions(*v.a) && !mentions(*v.b)) {
+    *accum = Binop::Add;
+  } else if (v.kind == Scalar::Bin && (v.bin == Binop::Add || v.bin == Binop::Max || v.bin == Binop::Min) &&
+             ((is_v(*v.a) && !mentions(*v.b)) || (is_v(*v.b) && !mentions(*v.a)))) {
+    *accum = v.bin;
+  } else return false;
+  const double c0 = init->value->cst;
+  if (*accum == Binop::Add && c0 != 0.0) return false;
+  if (*accum == Binop::Max && !(std::isinf(c0) && c0 < 0)) return false;
+  if (*accum == Binop::Min && !(std::isinf(c0) && c0 > 0)) return false;
+  for (const Stmt* l : loops) if (l->to < l->from) return false;
+  return true;
+}
+
+// A pointwise statement whose value holds one inlined scalar reduction: lanes may share it.
+void choose_scope_coop(const Routine& r, Phase& ph) {
+  if (ph.inner.size() != 1 || ph.inner[0]->kind != Stmt::Set) return;
+  std::vector<const Scalar*> found;
+  std::function<void(const Scalar&)> walk = [&](const Scalar& s) {
+    if (s.kind == Scalar::LocalScope) { found.push_back(&s); return; }
+    if (s.a) walk(*s.a);
+    if (s.b) walk(*s.b);
+    if (s.c) walk(*s.c);
+  };
+  walk(*ph.inner[0]->value);
+  if (found.size() != 1) return;
+  std::vector<const Stmt*> loops; const Stmt* init = nullptr; const Stmt* upd = nullptr; Binop accum;
+  if (!scope_reduction(*found[0], loops, init, upd, &accum)) return;
+  const Prec p = r.node(found[0]->scope.node).prec;
+  if (!(p == Prec::Single || p == Prec::Double || p == Prec::Bfloat16 || p == Prec::Half)) return;
+  int64_t P = 1, R = 1;
+  for (auto e : ph.par_ext) P *= e;
+  for (const Stmt* l : loops) R *= l->to - l->from + 1;
+  const int64_t rext = loops.back()->to - loops.back()->from + 1;
+  // one thread per point walks its own row: adjacent threads are a whole row apart, so sharing
+  // the row between adjacent lanes is what makes the reads coalesce
+  std::vector<Access> acc; bool f = false; std::set<ScopeId> d;
+  scalar_accesses(*upd->value, acc, f, d);
+  bool unit = false;
+  for (auto& a : acc) if (get_stride(strides_of(r, a.node, *a.idcs), loops.back()->sym) == 1) unit = true;
+  auto pow2_floor = [](int64_t x) { int64_t p2 = 1; while (p2 * 2 <= x) p2 *= 2; return p2; };
+  int lanes = 1;
+  if (unit && rext >= 16) lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
+  else if (P < 16384 && R >= 256 && rext >= 2) lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
+  if (lanes > 1) { ph.coop_lanes = lanes; ph.coop_scope = found[0]; ph.coop_accum = accum; }
+}
+
 void choose_coop(const Routine& r, Phase& ph, const PlanOptions& opt) {
   ph.coop_lanes = 1;
-  if (!opt.enable_coop || ph.seq_syms.empty()) return;
+  if (!opt.enable_coop) return;
+  if (ph.seq_syms.empty()) { choose_scope_coop(r, ph); return; }
   Binop accum;
   if (!reduction_shape(r, ph, &accum)) return;
   const Stmt& set = *ph.inner[0];
@@ -366,6 +444,17 @@ void account_bytes(const Routine& r, Phase& ph) {
     bytes += n * prec_in_bytes(nd.prec);
   }
   ph.bytes = bytes;
+}
+
+// Does the phase read or write `node`?
+bool phase_touches(const Phase& ph, int node) {
+  if (ph.kind == Phase::Fill) return ph.fill_node == node;
+  if (ph.kind == Phase::Contraction) return ph.gemm.a.node == node || ph.gemm.b.node == node || ph.gemm.c.node == node;
+  std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+  block_accesses(ph.inner, acc, w, f, d);
+  if (w) return true;   // a Zero_out inside the nest: not tracked per node, assume the worst
+  for (auto& a : acc) if (a.node == node) return true;
+  return false;
 }
 
 Block strip_comments(const Block& b, std::string* last_comment) {
@@ -535,9 +624,213 @@ static void devirtualise(Routine& r, const StmtP& sp, const PlanOptions& opt, Pl
   }
 }
 
+// ---- split reductions ---------------------------------------------------------------------------
+// `out[p] := out[p] + e(p, k1..kn)` where the output is small and the reduction runs over the slow
+// axes of its operands (bias / gain gradients: a column sum over all rows).  One thread per output
+// would leave most of the chip idle, and lanes sharing a column read a whole row apart.  Instead
+// the outer part of the reduction range becomes parallel: phase 1 sums slice s into a scratch
+// tensor partial[s, p] (threads adjacent along p: coalesced), phase 2 adds the slices to `out` in
+// index order (deterministic).
+
+static int fresh_symbol(const Routine& r, int* next) {
+  if (*next == 0) {
+    int mx = 0;
+    std::function<void(const Block&)> scan = [&](const Block& b) {
+      for (auto& s : b) {
+        if (s->kind == Stmt::For) { mx = std::max(mx, s->sym); scan(s->body); }
+        std::function<void(const Scalar&)> sc = [&](const Scalar& x) {
+          if (x.kind == Scalar::LocalScope) scan(x.body);
+          if (x.a) sc(*x.a); if (x.b) sc(*x.b); if (x.c) sc(*x.c);
+        };
+        if (s->value) sc(*s->value);
+      }
+    };
+    scan(r.body);
+    for (auto& st : r.statics) mx = std::max(mx, st.sym);
+    *next = mx + 1;
+  }
+  return (*next)++;
+}
+
+// index with `sym` replaced by from + len * hi + lo
+static AxisIndex subst_index(const AxisIndex& a, int sym, int64_t from, int64_t len, int hi, int lo) {
+  if (!a.mentions(sym)) return a;
+  AxisIndex o;
+  o.kind = AxisIndex::Affine;
+  if (a.kind == AxisIndex::Iter) {
+    o.terms = {{len, hi}, {1, lo}};
+    o.offset = from;
+  } else {
+    o.offset = a.offset;
+    for (auto& t : a.terms) {
+      if (t.second != sym) { o.terms.push_back(t); continue; }
+      o.terms.push_back({t.first * len, hi});
+      o.terms.push_back({t.first, lo});
+      o.offset += t.first * from;
+    }
+  }
+  return o;
+}
+
+static ScalarP subst_scalar(const ScalarP& sp, int sym, int64_t from, int64_t len, int hi, int lo, bool* ok) {
+  if (!sp) return sp;
+  if (sp->kind == Scalar::LocalScope) { *ok = false; return sp; }
+  auto o = std::make_shared<Scalar>(*sp);
+  for (auto& ix : o->idcs) ix = subst_index(ix, sym, from, len, hi, lo);
+  if (o->kind == Scalar::Index) o->index = subst_index(o->index, sym, from, len, hi, lo);
+  o->a = subst_scalar(sp->a, sym, from, len, hi, lo, ok);
+  o->b = subst_scalar(sp->b, sym, from, len, hi, lo, ok);
+  o->c = subst_scalar(sp->c, sym, from, len, hi, lo, ok);
+  return o;
+}
+
+static StmtP make_for(int sym, int64_t from, int64_t to, StmtP body) {
+  auto f = std::make_shared<Stmt>();
+  f->kind = Stmt::For; f->sym = sym; f->from = from; f->to = to; f->body = {std::move(body)};
+  return f;
+}
+
+// On success pushes phase 1 onto the plan and rewrites `ph` into phase 2.
+static bool split_reduction(Routine& r, Phase& ph, const PlanOptions& opt, Plan& plan, int* next_sym) {
+  if (!opt.enable_coop || ph.seq_syms.empty()) return false;
+  Binop accum;
+  if (!reduction_shape(r, ph, &accum) || accum != Binop::Add) return false;
+  const Stmt& set = *ph.inner[0];
+  const Node& out = r.node(set.node);
+  if (!(out.prec == Prec::Single || out.prec == Prec::Double || out.prec == Prec::Bfloat16 || out.prec == Prec::Half))
+    return false;
+  int64_t P = 1, R = 1;
+  for (auto e : ph.par_ext) P *= e;
+  for (size_t i = 0; i < ph.seq_syms.size(); ++i) R *= ph.seq_to[i] - ph.seq_from[i] + 1;
+  if (P >= 32768 || R < 128 || P * R < (1 << 20)) return false;
+  for (auto f : ph.par_from) if (f != 0) return false;
+  // lanes sharing the innermost loop already read contiguously: leave those to the lane groups
+  std::vector<Access> acc; bool fl = false; std::set<ScopeId> d;
+  scalar_accesses(*set.value, acc, fl, d);
+  for (auto& a : acc) {
+    if (a.node == set.node) continue;
+    if (get_stride(strides_of(r, a.node, *a.idcs), ph.seq_syms.back()) == 1) return false;
+  }
+  const int64_t s_target = std::min<int64_t>(std::max<int64_t>((131072 + P - 1) / P, 2), R / 8);
+  // whole outer loops first, then a divisor of the next one
+  size_t whole = 0;
+  int64_t S = 1;
+  while (whole < ph.seq_syms.size() && S * (ph.seq_to[whole] - ph.seq_from[whole] + 1) <= s_target) {
+    S *= ph.seq_to[whole] - ph.seq_from[whole] + 1;
+    ++whole;
+  }
+  int64_t hi_ext = 1, lo_ext = 0;
+  if (whole < ph.seq_syms.size()) {
+    const int64_t E = ph.seq_to[whole] - ph.seq_from[whole] + 1;
+    for (int64_t h = std::min(E, s_target / S); h > 1; --h)
+      if (E % h == 0) { hi_ext = h; break; }
+    lo_ext = E / hi_ext;
+  }
+  if (S * hi_ext < 2) return false;
+
+  // value with the split symbol rewritten
+  ScalarP value = set.value;
+  int hi = -1, lo = -1;
+  if (hi_ext > 1) {
+    hi = fresh_symbol(r, next_sym);
+    lo = fresh_symbol(r, next_sym);
+    bool ok = true;
+    value = subst_scalar(value, ph.seq_syms[whole], ph.seq_from[whole], lo_ext, hi, lo, &ok);
+    if (!ok) return false;
+  }
+  // scratch tensor partial[slices.., p..]: output symbols ordered as the output stores them
+  std::vector<size_t> order(ph.par_syms.size());
+  for (size_t i = 0; i < order.size(); ++i) order[i] = i;
+  Strides so = strides_of(r, set.node, set.idcs);
+  std::stable_sort(order.begin(), order.end(), [&](size_t x, size_t y) {
+    return get_stride(so, ph.par_syms[x]) > get_stride(so, ph.par_syms[y]); });
+  int new_id = 1;
+  for (auto& kv : r.nodes) new_id = std::max(new_id, kv.first + 1);
+  Node t;
+  t.id = new_id;
+  t.ident = "part" + std::to_string(new_id) + "_" + out.ident;
+  t.prec = out.prec == Prec::Double ? Prec::Double : Prec::Single;
+  t.mode = Mode::Local;
+  Indices tix;
+  auto iter = [](int sym) { AxisIndex a; a.kind = AxisIndex::Iter; a.sym = sym; return a; };
+  auto shifted = [](int sym, int64_t from) {
+    AxisIndex a;
+    if (from == 0) { a.kind = AxisIndex::Iter; a.sym = sym; }
+    else { a.kind = AxisIndex::Affine; a.terms = {{1, sym}}; a.offset = -from; }
+    return a;
+  };
+  for (size_t i = 0; i < whole; ++i) {
+    t.dims.push_back(ph.seq_to[i] - ph.seq_from[i] + 1);
+    tix.push_back(shifted(ph.seq_syms[i], ph.seq_from[i]));
+  }
+  if (hi_ext > 1) { t.dims.push_back(hi_ext); tix.push_back(iter(hi)); }
+  for (size_t k : order) { t.dims.push_back(ph.par_ext[k]); tix.push_back(iter(ph.par_syms[k])); }
+
+  // the same accumulation with the scratch element in place of the output element
+  auto self = std::make_shared<Scalar>();
+  self->kind = Scalar::Get; self->node = t.id; self->idcs = tix;
+  auto is_self = [&](const Scalar& x) { return x.kind == Scalar::Get && x.node == set.node && same_indices(x.idcs, set.idcs); };
+  auto v1 = std::make_shared<Scalar>(*value);
+  if (v1->kind == Scalar::Tern) v1->c = self;
+  else if (is_self(*set.value->a)) v1->a = self;
+  else v1->b = self;
+  auto set1 = std::make_shared<Stmt>();
+  set1->kind = Stmt::Set; set1->node = t.id; set1->idcs = tix; set1->value = v1;
+  StmtP nest1 = set1;
+  for (size_t i = ph.seq_syms.size(); i-- > whole + (hi_ext > 1 ? 1 : 0);)
+    nest1 = make_for(ph.seq_syms[i], ph.seq_from[i], ph.seq_to[i], nest1);
+  if (hi_ext > 1) {
+    nest1 = make_for(lo, 0, lo_ext - 1, nest1);
+    nest1 = make_for(hi, 0, hi_ext - 1, nest1);
+  }
+  for (size_t i = whole; i-- > 0;) nest1 = make_for(ph.seq_syms[i], ph.seq_from[i], ph.seq_to[i], nest1);
+  for (size_t k = order.size(); k-- > 0;)
+    nest1 = make_for(ph.par_syms[order[k]], 0, ph.par_ext[order[k]] - 1, nest1);
+
+  // phase 2: out[p] := out[p] + partial[s.., p..] over the slices
+  auto get_t = std::make_shared<Scalar>();
+  get_t->kind = Scalar::Get; get_t->node = t.id; get_t->idcs = tix;
+  auto lhs = std::make_shared<Scalar>();
+  lhs->kind = Scalar::Get; lhs->node = set.node; lhs->idcs = set.idcs;
+  auto v2 = std::make_shared<Scalar>();
+  v2->kind = Scalar::Bin; v2->bin = Binop::Add; v2->a = lhs; v2->b = get_t;
+  auto set2 = std::make_shared<Stmt>();
+  set2->kind = Stmt::Set; set2->node = set.node; set2->idcs = set.idcs; set2->value = v2;
+  StmtP nest2 = set2;
+  if (hi_ext > 1) nest2 = make_for(hi, 0, hi_ext - 1, nest2);
+  for (size_t i = whole; i-- > 0;) nest2 = make_for(ph.seq_syms[i], ph.seq_from[i], ph.seq_to[i], nest2);
+  for (size_t k = order.size(); k-- > 0;)
+    nest2 = make_for(ph.par_syms[order[k]], 0, ph.par_ext[order[k]] - 1, nest2);
+
+  r.nodes.emplace(t.id, t);
+  Phase p1;
+  p1.label = ph.label + " (partial sums)";
+  p1.stmt = nest1;
+  p1.fused_zero_init = true;
+  Phase p2;
+  p2.label = ph.label;
+  p2.stmt = nest2;
+  p2.fused_zero_init = ph.fused_zero_init;
+  Binop a1, a2;
+  if (!analyze_nest(r, nest1, p1) || !analyze_nest(r, nest2, p2) || !reduction_shape(r, p1, &a1) ||
+      !reduction_shape(r, p2, &a2) || p1.par_syms.size() != order.size() + whole + (hi_ext > 1 ? 1 : 0) ||
+      p2.par_syms.size() != order.size()) {
+    r.nodes.erase(t.id);
+    return false;
+  }
+  p1.kind = Phase::Generic;
+  choose_coop(r, p1, opt);
+  account_bytes(r, p1);
+  plan.phases.push_back(std::move(p1));
+  plan.scratch.push_back(t);
+  ph = std::move(p2);
+  return true;
+}
+
 Plan make_plan(Routine& r, const PlanOptions& opt) {
   Plan plan;
   std::string label;
+  int next_sym = 0;
   Block top = r.body;
   for (size_t ti = 0; ti < top.size(); ++ti) {
     StmtP sp = top[ti];
@@ -561,11 +854,21 @@ Plan make_plan(Routine& r, const PlanOptions& opt) {
     const bool devirt = plan.phases.size() != before;
     if (!analyze_nest(r, sp, ph)) continue;
 
-    // fold a directly preceding Zero_out of the accumulation target into this phase when the nest
-    // overwrites the whole array: every axis is a full-range parallel iterator or has extent 1.
+    // fold the preceding Zero_out of the accumulation target into this phase (the accumulation then
+    // starts from zero instead of reading the array) when no phase in between touches the array and
+    // the nest overwrites all of it: every axis is a full-range parallel iterator or has extent 1.
     Binop accum;
-    if (!devirt && !plan.phases.empty() && plan.phases.back().kind == Phase::Fill && reduction_shape(r, ph, &accum) &&
-        accum == Binop::Add && plan.phases.back().fill_node == ph.inner[0]->node) {
+    int fill_at = -1;
+    if (!devirt && reduction_shape(r, ph, &accum) && accum == Binop::Add) {
+      // the latest Zero_out of the target with nothing touching the target in between
+      const int target = ph.inner[0]->node;
+      for (int q = (int)plan.phases.size() - 1; q >= 0; --q) {
+        const Phase& prev = plan.phases[q];
+        if (prev.kind == Phase::Fill && prev.fill_node == target) { fill_at = q; break; }
+        if (phase_touches(prev, target)) break;
+      }
+    }
+    if (fill_at >= 0) {
       const Stmt& set = *ph.inner[0];
       const Node& n = r.node(set.node);
       bool full = true;
@@ -578,11 +881,12 @@ Plan make_plan(Routine& r, const PlanOptions& opt) {
             if (ph.par_syms[i] == a.sym) full = ph.par_from[i] == 0 && ph.par_ext[i] == n.dims[p];
         } else full = false;
       }
-      if (full) { ph.fused_zero_init = true; plan.phases.pop_back(); }
+      if (full) { ph.fused_zero_init = true; plan.phases.erase(plan.phases.begin() + fill_at); }
     }
 
     if (!match_contraction(r, ph, opt)) {
       ph.kind = Phase::Generic;
+      split_reduction(r, ph, opt, plan, &next_sym);
       choose_coop(r, ph, opt);
       account_bytes(r, ph);
     } else {

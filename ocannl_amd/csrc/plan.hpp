@@ -53,6 +53,10 @@ struct Phase {
   std::vector<int64_t> seq_from, seq_to;
   Block inner;                // body below the perfect-nest chain
   int coop_lanes = 1;         // >1: that many adjacent lanes share one output (tree-combined)
+  // coop_lanes > 1 with no sequential chain loops: the lanes split the innermost loop of this
+  // inlined scalar reduction `v { v := c; for.. { v := accum(v, e) } }` inside the statement
+  const Scalar* coop_scope = nullptr;
+  Binop coop_accum = Binop::Add;
   bool fused_zero_init = false;  // the preceding Zero_out of the target was folded in (beta = 0)
   // Fill
   int fill_node = -1;

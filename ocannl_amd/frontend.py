@@ -276,10 +276,11 @@ class Graph:
                           lambda g, v, c, x, y: L.Ternop("where", c, L.Const(0.0), g)])
 
     def _union_axes(self, *ts):
+        """Result axes of a broadcasting pointwise operation: those of the operand of highest rank
+        in its own order (so that the result shares its layout), then any the others add."""
         out: List[str] = []
-        for t in ts:
-            if isinstance(t, ConstT):
-                continue
+        ranked = sorted((t for t in ts if not isinstance(t, ConstT)), key=lambda t: -len(t.axes))
+        for t in ranked:
             for a in t.axes:
                 if a not in out:
                     out.append(a)

@@ -399,7 +399,7 @@ def transformer(batch: int = 32, seq: int = 256, d_model: int = 512, heads: int 
 
 
 def _reorder(g: Graph, t: T, axes):
-    """Guarantee the axis order of a tensor (where() orders axes by first appearance)."""
+    """Guarantee the axis order of a tensor (a copy only when it differs)."""
     if tuple(t.axes) == tuple(axes):
         return t
     return g.nary(t.label + "_perm", [t], axes, lambda x: x, [lambda gr, v, x: gr])
