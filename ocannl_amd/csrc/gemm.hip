@@ -64,11 +64,14 @@ constexpr int kPad = 8;        // bf16 elements of row padding (16 bytes)
 constexpr int kBKf = 32;       // K elements per stage (fp32 compute)
 constexpr int kPadf = 4;       // floats of row padding (16 bytes)
 
-__device__ __forceinline__ unsigned f2bf(float f) {   // round to nearest even, as single_to_bfloat16
-  const unsigned w = __float_as_uint(f);
-  return (w + 0x7FFFu + ((w >> 16) & 1u)) >> 16;
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+// fp32 -> bf16, round to nearest even, in hardware (v_cvt_pk_bf16_f32).  Equal to
+// single_to_bfloat16 for every input that is not a NaN.
+__device__ __forceinline__ unsigned f2bf(float f) { return __builtin_bit_cast(unsigned short, (__bf16)f); }
+__device__ __forceinline__ unsigned pack2(float lo, float hi) {
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{lo, hi}, bf16x2_t));
 }
-__device__ __forceinline__ unsigned pack2(float lo, float hi) { return f2bf(lo) | (f2bf(hi) << 16); }
 
 // Raw staging type of 8 consecutive source elements: bf16 sources travel as one 16-byte vector,
 // fp32 sources as two; the fp32 -> bf16 rounding happens when the registers are written to LDS, so
@@ -552,27 +555,35 @@ long batch_count(const GemmDesc& d) {
   return nb;
 }
 
-bool big_tile(const GemmDesc& d) {
-  // 256x256 tiles only when they still fill the chip (>= 256 workgroups)
-  const double tiles = ((d.M + 255) / 256) * (double)((d.N + 255) / 256) * (double)batch_count(d);
-  return tiles >= 256;
+#ifdef OCANNL_GEMM_TIMING
+int g_force_tile = 0, g_force_splits = 0;   // tuning overrides of the probe build
+#endif
+
+// Tile size and split-K factor.  Measured on MI355X: the 256x256 tile (one workgroup per CU) pays
+// off only when every workgroup runs at least ~16 K stages and the launch still has >= 192
+// workgroups, K being split to get there (weight-gradient shapes: small output, K = all rows);
+// otherwise 128x128 tiles, two workgroups per CU, split towards ~512 workgroups.  A split never
+// gets fewer than 8 K stages.  Splits are summed in index order by splitk_reduce_kernel.
+struct TileConfig { bool big; int splits; };
+
+TileConfig tile_config(const GemmDesc& d) {
+  const long nb = batch_count(d);
+  const long t256 = ((d.M + 255) / 256) * ((d.N + 255) / 256) * nb;
+  const long t128 = ((d.M + 127) / 128) * ((d.N + 127) / 128) * nb;
+  auto clampl = [](long v, long lo, long hi) { return v < lo ? lo : (v > hi ? hi : v); };
+  const long s256 = clampl((256 + t256 - 1) / t256, 1, clampl(d.K / 512, 1, 64));
+  TileConfig c;
+  if (t256 * s256 >= 192 && d.K / s256 >= 1024) { c.big = true; c.splits = (int)s256; }
+  else { c.big = false; c.splits = (int)clampl((512 + t128 / 2) / t128, 1, clampl(d.K / 512, 1, 64)); }
+#ifdef OCANNL_GEMM_TIMING
+  if (g_force_tile) c.big = g_force_tile == 256;
+  if (g_force_splits) c.splits = g_force_splits;
+#endif
+  return c;
 }
 
-// Split K when the output has too few tiles to occupy the 256 CUs and K is long enough that every
-// split still runs at least four K stages.
-int split_count(const GemmDesc& d) {
-  const int tile = big_tile(d) ? 256 : 128;
-  const bool f32 = d.a.prec == Prec::Single && d.b.prec == Prec::Single;
-  const long bk = f32 ? kBKf : kBK;
-  const long tiles = ((d.M + tile - 1) / tile) * ((d.N + tile - 1) / tile) * batch_count(d);
-  if (tiles >= 192) return 1;
-  const long ksteps = (d.K + bk - 1) / bk;
-  long want = (256 + tiles - 1) / tiles;
-  long cap = ksteps / 4;
-  long s = want < cap ? want : cap;
-  if (s > 64) s = 64;
-  return s < 2 ? 1 : (int)s;
-}
+bool big_tile(const GemmDesc& d) { return tile_config(d).big; }
+int split_count(const GemmDesc& d) { return tile_config(d).splits; }
 
 template <typename K>
 hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t s) {

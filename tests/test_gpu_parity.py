@@ -147,3 +147,30 @@ def test_split_k_weight_gradient_shape(prec, tol):
     hip2.step()
     assert np.array_equal(hip2.get(w.nodes["dw"]).view(np.uint32), hip.get(w.nodes["dw"]).view(np.uint32))
     hip.close(); hip2.close()
+
+
+def test_single_to_bfloat16_bit_exact_on_all_float_classes():
+    # the device rounds fp32 -> bf16 in hardware; the checker restates the host's integer rounding
+    # (builtins.c:620-627): both must agree on every bit pattern, NaN payloads included
+    rng = np.random.default_rng(7)
+    n = 1 << 22
+    bits = rng.integers(0, 1 << 32, size=n, dtype=np.uint64).astype(np.uint32)
+    special = np.array([0x00000000, 0x80000000, 0x00000001, 0x007FFFFF, 0x00800000, 0x7F7FFFFF, 0xFF7FFFFF,
+                        0x7F800000, 0xFF800000, 0x7FC00000, 0x7FFFFFFF, 0xFFFFFFFF, 0x7F800001, 0x3F808000,
+                        0x3F818000, 0x3F807FFF, 0x3F808001, 0x7F7F8000, 0x00008000, 0x00018000], np.uint32)
+    bits[:special.size] = special
+    # every pattern whose low half sits on a rounding boundary, over a sweep of high halves
+    hi = (np.arange(1 << 16, dtype=np.uint32) << 16)
+    bits[special.size:special.size + (1 << 16)] = hi | 0x8000
+    bits[special.size + (1 << 16):special.size + (2 << 16)] = hi | 0x7FFF
+    L.reset_symbols(0)
+    x = L.Node(1, "x", "single", (n,)); y = L.Node(2, "y", "bfloat16", (n,))
+    i = L.fresh_symbol()
+    r = L.Routine("to_bf16", [L.For(i, 0, n - 1, [L.Set(y, (L.It(i),), L.Get(x, (L.It(i),)))])])
+    init = {1: bits.view(np.float32)}
+    hip, ora = HipRun(r, init), OracleRun(r, init)
+    hip.step(); ora.step()
+    got, want = hip.get(y).view(np.uint16), ora.get(y).view(np.uint16)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, [(hex(bits[k]), hex(got[k]), hex(want[k])) for k in bad[:8]]
+    hip.close()
