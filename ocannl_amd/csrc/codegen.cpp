@@ -291,6 +291,7 @@ struct Printer {
   const Scalar* coop_scope = nullptr;
   int coop_lanes = 1;
   Binop coop_accum = Binop::Add;
+  std::string store_guard;   // prefix of plain stores ("if (lane_ == 0) " when one lane stores for a group)
   // when set, a read of exactly this (node, indices) prints as `self_name`
   const Stmt* self_set = nullptr;
   std::string self_name;
@@ -487,8 +488,7 @@ struct Printer {
         note(c.node, c.idcs);
         std::vector<Def> defs;
         std::string v = scalar(n.prec, *c.value, ind + "  ", defs);
-        with_defs(defs, {std::string(coop_scope ? "if (lane_ == 0) " : "") + n.ident + "[" + offset_str(c.idcs, n.dims) +
-                         "] = " + v + ";"}, ind, out);
+        with_defs(defs, {store_guard + n.ident + "[" + offset_str(c.idcs, n.dims) + "] = " + v + ";"}, ind, out);
         break;
       }
       case Stmt::SetVec: {
@@ -555,6 +555,112 @@ std::string combine_expr(Binop accum, bool dbl, const std::string& a, const std:
 
 }  // namespace
 
+namespace {
+
+// Statements of one phase for a thread whose parallel symbols are already defined.  G > 1: the
+// thread is lane `lane_` of a group of G sharing the point.  `lane0_store`: plain stores are done
+// by lane 0 only (per-row scalars inside a row group).
+void emit_phase_statements(const Routine& r, Printer& pr, const Phase& ph, int G, bool lane0_store,
+                           const std::string& ind, std::vector<std::string>& body) {
+  Binop accum = Binop::Add;
+  bool is_reduction = false;
+  const Stmt* set = nullptr;
+  if ((!ph.seq_syms.empty() || ph.fused_zero_init) && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set) {
+    set = ph.inner[0].get();
+    const Scalar& v = *set->value;
+    auto is_self = [&](const Scalar& s) { return s.kind == Scalar::Get && s.node == set->node && s.idcs == set->idcs; };
+    if (v.kind == Scalar::Tern && v.tern == Ternop::Fma && is_self(*v.c)) { is_reduction = true; accum = Binop::Add; }
+    else if (v.kind == Scalar::Bin && (v.bin == Binop::Add || v.bin == Binop::Max || v.bin == Binop::Min) &&
+             (is_self(*v.a) || is_self(*v.b))) { is_reduction = true; accum = v.bin; }
+  }
+  auto open_seq_loops = [&](std::string& cur_ind, bool coop_last) {
+    for (size_t i = 0; i < ph.seq_syms.size(); ++i) {
+      const std::string s = sym_ident(ph.seq_syms[i]);
+      if (coop_last && i + 1 == ph.seq_syms.size())
+        body.push_back(cur_ind + "for (uint32_t " + s + " = " + std::to_string(ph.seq_from[i]) + " + lane_; " + s +
+                       " <= " + std::to_string(ph.seq_to[i]) + "; " + s + " += " + std::to_string(G) + ") {");
+      else
+        body.push_back(cur_ind + "for (uint32_t " + s + " = " + std::to_string(ph.seq_from[i]) + "; " + s + " <= " +
+                       std::to_string(ph.seq_to[i]) + "; ++" + s + ") {");
+      cur_ind += "  ";
+    }
+  };
+  auto close_seq_loops = [&](std::string& cur_ind) {
+    for (size_t i = 0; i < ph.seq_syms.size(); ++i) { cur_ind.resize(cur_ind.size() - 2); body.push_back(cur_ind + "}"); }
+  };
+  const bool guard = lane0_store || ph.coop_scope;
+  const std::string lane0 = guard && G > 1 ? "if (lane_ == 0) " : "";
+
+  if (is_reduction && G > 1 && !ph.coop_scope && !ph.seq_syms.empty()) {
+    // lanes of a group stride the innermost sequential loop; partials are combined by butterfly
+    // shuffles in a fixed order (deterministic), accumulating in float (double for double).
+    const Node& n = r.node(set->node);
+    pr.note(set->node, set->idcs);
+    const bool dbl = n.prec == Prec::Double;
+    const std::string accT = dbl ? "double" : "float";
+    const Prec accP = dbl ? Prec::Double : Prec::Single;
+    body.push_back(ind + accT + " part_ = " + neutral_literal(accum, dbl) + ";");
+    std::string ci = ind;
+    open_seq_loops(ci, true);
+    const Scalar& v = *set->value;
+    std::vector<Printer::Def> defs;
+    std::vector<std::string> lines;
+    auto widen = [&](const std::string& e) { Pair c = convert_precision(n.prec, accP); return c.first + e + c.second; };
+    if (v.kind == Scalar::Tern) {
+      std::string a = pr.scalar(n.prec, *v.a, ci + "  ", defs), b = pr.scalar(n.prec, *v.b, ci + "  ", defs);
+      lines.push_back(std::string("part_ = ") + (dbl ? "fma(" : "fmaf(") + widen(a) + ", " + widen(b) + ", part_);");
+    } else {
+      auto is_self = [&](const Scalar& s) { return s.kind == Scalar::Get && s.node == set->node && s.idcs == set->idcs; };
+      const Scalar& e = is_self(*v.a) ? *v.b : *v.a;
+      std::string es = pr.scalar(n.prec, e, ci + "  ", defs);
+      lines.push_back("part_ = " + combine_expr(accum, dbl, "part_", widen(es)) + ";");
+    }
+    pr.with_defs(defs, lines, ci, body);
+    close_seq_loops(ci);
+    for (int o = G / 2; o > 0; o >>= 1)
+      body.push_back(ind + "part_ = " + combine_expr(accum, dbl, "part_", "ocn_xshfl(part_, " + std::to_string(o) + ")") + ";");
+    const std::string lhs = n.ident + "[" + offset_str(set->idcs, n.dims) + "]";
+    Pair narrow = convert_precision(accP, n.prec);
+    Pair wide = convert_precision(n.prec, accP);
+    if (ph.fused_zero_init)
+      body.push_back(ind + "if (lane_ == 0) " + lhs + " = " + narrow.first + "part_" + narrow.second + ";");
+    else
+      body.push_back(ind + "if (lane_ == 0) " + lhs + " = " + narrow.first +
+                     combine_expr(accum, dbl, wide.first + lhs + wide.second, "part_") + narrow.second + ";");
+  } else if (is_reduction) {
+    // one thread per output element, sequential loops in the reference's order: for fp32 this is
+    // the same operation sequence as the `cc` backend's serial loop.
+    const Node& n = r.node(set->node);
+    pr.note(set->node, set->idcs);
+    const std::string lhs = n.ident + "[" + offset_str(set->idcs, n.dims) + "]";
+    Pair zero = convert_precision(Prec::Double, n.prec);
+    body.push_back(ind + c_typ(n.prec) + " acc_ = " + (ph.fused_zero_init ? zero.first + "0" + zero.second : lhs) + ";");
+    std::string ci = ind;
+    open_seq_loops(ci, false);
+    pr.self_set = set; pr.self_name = "acc_";
+    if (ph.coop_scope && G > 1) { pr.coop_scope = ph.coop_scope; pr.coop_lanes = G; pr.coop_accum = ph.coop_accum; }
+    std::vector<Printer::Def> defs;
+    std::string v = pr.scalar(n.prec, *set->value, ci + "  ", defs);
+    pr.with_defs(defs, {"acc_ = " + v + ";"}, ci, body);
+    pr.self_set = nullptr;
+    close_seq_loops(ci);
+    body.push_back(ind + lane0 + lhs + " = acc_;");
+    pr.coop_scope = nullptr;
+  } else {
+    if (ph.fused_zero_init) throw InvalidArgument("planner: fused zero-init on a non-reduction phase");
+    std::string ci = ind;
+    open_seq_loops(ci, false);
+    if (ph.coop_scope && G > 1) { pr.coop_scope = ph.coop_scope; pr.coop_lanes = G; pr.coop_accum = ph.coop_accum; }
+    pr.store_guard = lane0;
+    pr.block(ph.inner, ci, body);
+    pr.store_guard.clear();
+    pr.coop_scope = nullptr;
+    close_seq_loops(ci);
+  }
+}
+
+}  // namespace
+
 GeneratedModule generate_module(const Routine& r, const Plan& plan) {
   GeneratedModule mod;
   std::ostringstream src;
@@ -566,38 +672,9 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     Printer pr(r);
     std::vector<std::string> body;
     const std::string ind = "  ";
-
-    // --- thread -> point decode: the symbol with the smallest stride in the first written array
-    //     varies fastest across adjacent threads (coalesced stores)
-    std::vector<size_t> order(ph.par_syms.size());
-    for (size_t i = 0; i < order.size(); ++i) order[i] = i;
-    const Stmt* first_set = nullptr;
-    std::function<void(const Block&)> find_set = [&](const Block& b) {
-      for (auto& s : b) {
-        if (first_set) return;
-        if (s->kind == Stmt::Set || s->kind == Stmt::SetVec) first_set = s.get();
-        else if (s->kind == Stmt::For) find_set(s->body);
-      }
-    };
-    find_set(ph.inner);
-    auto lhs_stride = [&](int sym) -> int64_t {
-      if (!first_set) return 0;
-      const Node& n = r.node(first_set->node);
-      int64_t st = 0, rs = 1;
-      for (int p = (int)first_set->idcs.size() - 1; p >= 0; --p) {
-        const AxisIndex& a = first_set->idcs[p];
-        if (a.kind == AxisIndex::Iter && a.sym == sym) st += rs;
-        if (a.kind == AxisIndex::Affine) for (auto& t : a.terms) if (t.second == sym) st += t.first * rs;
-        rs *= n.dims[p];
-      }
-      return st;
-    };
-    std::stable_sort(order.begin(), order.end(), [&](size_t x, size_t y) {
-      return lhs_stride(ph.par_syms[x]) > lhs_stride(ph.par_syms[y]); });   // slowest first
-
-    uint64_t P = 1;
-    for (auto e : ph.par_ext) P *= (uint64_t)e;
     const int G = ph.coop_lanes;
+    uint64_t P = 1;
+
     body.push_back(ind + "const uint64_t gtid_ = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;");
     if (G > 1) {
       body.push_back(ind + "const uint32_t lane_ = (uint32_t)(gtid_ % " + std::to_string(G) + "u);");
@@ -605,110 +682,55 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     } else {
       body.push_back(ind + "uint64_t pt_ = gtid_;");
     }
-    body.push_back(ind + "if (pt_ >= " + std::to_string(P) + "ull) return;");
-    for (int k = (int)order.size() - 1; k >= 0; --k) {
-      const size_t i = order[k];
-      const std::string s = sym_ident(ph.par_syms[i]);
-      const std::string ext = std::to_string(ph.par_ext[i]) + "ull";
-      std::string line = ind + "const uint32_t " + s + " = (uint32_t)(" + std::to_string(ph.par_from[i]) + " + ";
-      if (k == 0) line += "pt_);";
-      else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
-      body.push_back(line);
-    }
 
-    Binop accum = Binop::Add;
-    bool is_reduction = false;
-    const Stmt* set = nullptr;
-    if ((!ph.seq_syms.empty() || ph.fused_zero_init) && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set) {
-      set = ph.inner[0].get();
-      const Scalar& v = *set->value;
-      auto is_self = [&](const Scalar& s) { return s.kind == Scalar::Get && s.node == set->node && s.idcs == set->idcs; };
-      if (v.kind == Scalar::Tern && v.tern == Ternop::Fma && is_self(*v.c)) { is_reduction = true; accum = Binop::Add; }
-      else if (v.kind == Scalar::Bin && (v.bin == Binop::Add || v.bin == Binop::Max || v.bin == Binop::Min) &&
-               (is_self(*v.a) || is_self(*v.b))) { is_reduction = true; accum = v.bin; }
-      // the lhs indices must not depend on a sequential symbol (they cannot: it would be parallel)
-    }
-
-    auto open_seq_loops = [&](std::string& cur_ind, bool coop_last) {
-      for (size_t i = 0; i < ph.seq_syms.size(); ++i) {
-        const std::string s = sym_ident(ph.seq_syms[i]);
-        if (coop_last && i + 1 == ph.seq_syms.size())
-          body.push_back(cur_ind + "for (uint32_t " + s + " = " + std::to_string(ph.seq_from[i]) + " + lane_; " + s +
-                         " <= " + std::to_string(ph.seq_to[i]) + "; " + s + " += " + std::to_string(G) + ") {");
-        else
-          body.push_back(cur_ind + "for (uint32_t " + s + " = " + std::to_string(ph.seq_from[i]) + "; " + s + " <= " +
-                         std::to_string(ph.seq_to[i]) + "; ++" + s + ") {");
-        cur_ind += "  ";
+    if (!ph.members.empty()) {
+      // ---- row group: a lane group owns one row and runs the member phases in order
+      for (auto e : ph.row_outer_ext) P *= (uint64_t)e;
+      body.push_back(ind + "if (pt_ >= " + std::to_string(P) + "ull) return;");
+      const size_t n = ph.row_outer_ext.size();
+      for (int k = (int)n - 1; k >= 0; --k) {
+        const std::string ext = std::to_string(ph.row_outer_ext[k]) + "ull";
+        std::string line = ind + "const uint32_t row" + std::to_string(k) + "_ = (uint32_t)(";
+        if (k == 0) line += "pt_);";
+        else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
+        body.push_back(line);
       }
-    };
-    auto close_seq_loops = [&](std::string& cur_ind) {
-      for (size_t i = 0; i < ph.seq_syms.size(); ++i) { cur_ind.resize(cur_ind.size() - 2); body.push_back(cur_ind + "}"); }
-    };
-
-    if (is_reduction && G > 1 && !ph.coop_scope) {
-      // lanes of a group stride the innermost sequential loop; partials are combined by butterfly
-      // shuffles in a fixed order (deterministic), accumulating in float (double for double).
-      const Node& n = r.node(set->node);
-      pr.note(set->node, set->idcs);
-      const bool dbl = n.prec == Prec::Double;
-      const std::string accT = dbl ? "double" : "float";
-      const Prec accP = dbl ? Prec::Double : Prec::Single;
-      body.push_back(ind + accT + " part_ = " + neutral_literal(accum, dbl) + ";");
-      std::string ci = ind;
-      open_seq_loops(ci, true);
-      const Scalar& v = *set->value;
-      std::vector<Printer::Def> defs;
-      std::vector<std::string> lines;
-      auto widen = [&](const std::string& e) { Pair c = convert_precision(n.prec, accP); return c.first + e + c.second; };
-      if (v.kind == Scalar::Tern) {
-        std::string a = pr.scalar(n.prec, *v.a, ci + "  ", defs), b = pr.scalar(n.prec, *v.b, ci + "  ", defs);
-        lines.push_back(std::string("part_ = ") + (dbl ? "fma(" : "fmaf(") + widen(a) + ", " + widen(b) + ", part_);");
-      } else {
-        auto is_self = [&](const Scalar& s) { return s.kind == Scalar::Get && s.node == set->node && s.idcs == set->idcs; };
-        const Scalar& e = is_self(*v.a) ? *v.b : *v.a;
-        std::string es = pr.scalar(n.prec, e, ci + "  ", defs);
-        lines.push_back("part_ = " + combine_expr(accum, dbl, "part_", widen(es)) + ";");
+      for (size_t mi = 0; mi < ph.members.size(); ++mi) {
+        const Phase& m = ph.members[mi];
+        if (mi) body.push_back(ind + "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\"); "
+                                     "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
+        body.push_back(ind + "{  /* " + m.label + " */");
+        const std::string mi_ind = ind + "  ";
+        for (size_t k = 0; k < m.row_outer_syms.size(); ++k)
+          body.push_back(mi_ind + "const uint32_t " + sym_ident(m.row_outer_syms[k]) + " = row" + std::to_string(k) + "_;");
+        if (m.row_role == Phase::RowPointwise) {
+          const std::string s = sym_ident(m.row_sym);
+          body.push_back(mi_ind + "for (uint32_t " + s + " = lane_; " + s + " < " + std::to_string(ph.row_len) + "; " + s +
+                         " += " + std::to_string(G) + ") {");
+          emit_phase_statements(r, pr, m, 1, false, mi_ind + "  ", body);
+          body.push_back(mi_ind + "}");
+        } else {
+          emit_phase_statements(r, pr, m, G, true, mi_ind, body);
+        }
+        body.push_back(ind + "}");
       }
-      pr.with_defs(defs, lines, ci, body);
-      close_seq_loops(ci);
-      for (int o = G / 2; o > 0; o >>= 1)
-        body.push_back(ind + "part_ = " + combine_expr(accum, dbl, "part_", "ocn_xshfl(part_, " + std::to_string(o) + ")") + ";");
-      const std::string lhs = n.ident + "[" + offset_str(set->idcs, n.dims) + "]";
-      Pair narrow = convert_precision(accP, n.prec);
-      Pair wide = convert_precision(n.prec, accP);
-      if (ph.fused_zero_init)
-        body.push_back(ind + "if (lane_ == 0) " + lhs + " = " + narrow.first + "part_" + narrow.second + ";");
-      else
-        body.push_back(ind + "if (lane_ == 0) " + lhs + " = " + narrow.first +
-                       combine_expr(accum, dbl, wide.first + lhs + wide.second, "part_") + narrow.second + ";");
-    } else if (is_reduction) {
-      // one thread per output element, sequential loops in the reference's order: for fp32 this is
-      // the same operation sequence as the `cc` backend's serial loop.
-      const Node& n = r.node(set->node);
-      pr.note(set->node, set->idcs);
-      const std::string lhs = n.ident + "[" + offset_str(set->idcs, n.dims) + "]";
-      Pair zero = convert_precision(Prec::Double, n.prec);
-      body.push_back(ind + c_typ(n.prec) + " acc_ = " + (ph.fused_zero_init ? zero.first + "0" + zero.second : lhs) + ";");
-      std::string ci = ind;
-      open_seq_loops(ci, false);
-      pr.self_set = set; pr.self_name = "acc_";
-      if (ph.coop_scope) { pr.coop_scope = ph.coop_scope; pr.coop_lanes = G; pr.coop_accum = ph.coop_accum; }
-      std::vector<Printer::Def> defs;
-      std::string v = pr.scalar(n.prec, *set->value, ci + "  ", defs);
-      pr.with_defs(defs, {"acc_ = " + v + ";"}, ci, body);
-      pr.self_set = nullptr;
-      close_seq_loops(ci);
-      body.push_back(ind + (ph.coop_scope ? "if (lane_ == 0) " : "") + lhs + " = acc_;");
-      pr.coop_scope = nullptr;
     } else {
-      if (ph.fused_zero_init) throw InvalidArgument("planner: fused zero-init on a non-reduction phase");
-      std::string ci = ind;
-      open_seq_loops(ci, false);
-      if (G > 1 && ph.coop_scope) { pr.coop_scope = ph.coop_scope; pr.coop_lanes = G; pr.coop_accum = ph.coop_accum; }
-      else if (G > 1) throw InvalidArgument("planner: lane group without a reduction to share");
-      pr.block(ph.inner, ci, body);
-      pr.coop_scope = nullptr;
-      close_seq_loops(ci);
+      // --- thread -> point decode: the symbol with the smallest stride in the first written array
+      //     varies fastest across adjacent threads (coalesced stores)
+      std::vector<size_t> order = store_order(r, ph);
+      for (auto e : ph.par_ext) P *= (uint64_t)e;
+      body.push_back(ind + "if (pt_ >= " + std::to_string(P) + "ull) return;");
+      for (int k = (int)order.size() - 1; k >= 0; --k) {
+        const size_t i = order[k];
+        const std::string s = sym_ident(ph.par_syms[i]);
+        const std::string ext = std::to_string(ph.par_ext[i]) + "ull";
+        std::string line = ind + "const uint32_t " + s + " = (uint32_t)(" + std::to_string(ph.par_from[i]) + " + ";
+        if (k == 0) line += "pt_);";
+        else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
+        body.push_back(line);
+      }
+      if (G > 1 && !ph.coop_scope && ph.seq_syms.empty()) throw InvalidArgument("planner: lane group without a reduction to share");
+      emit_phase_statements(r, pr, ph, G, false, ind, body);
     }
 
     GeneratedKernel gk;

@@ -827,6 +827,204 @@ static bool split_reduction(Routine& r, Phase& ph, const PlanOptions& opt, Plan&
   return true;
 }
 
+std::vector<size_t> store_order(const Routine& r, const Phase& ph) {
+  std::vector<size_t> order(ph.par_syms.size());
+  for (size_t i = 0; i < order.size(); ++i) order[i] = i;
+  const Stmt* first_set = nullptr;
+  std::function<void(const Block&)> find_set = [&](const Block& b) {
+    for (auto& s : b) {
+      if (first_set) return;
+      if (s->kind == Stmt::Set || s->kind == Stmt::SetVec) first_set = s.get();
+      else if (s->kind == Stmt::For) find_set(s->body);
+    }
+  };
+  find_set(ph.inner);
+  auto lhs_stride = [&](int sym) -> int64_t {
+    if (!first_set) return 0;
+    const Node& n = r.node(first_set->node);
+    int64_t st = 0, rs = 1;
+    for (int p = (int)first_set->idcs.size() - 1; p >= 0; --p) {
+      const AxisIndex& a = first_set->idcs[p];
+      if (a.kind == AxisIndex::Iter && a.sym == sym) st += rs;
+      if (a.kind == AxisIndex::Affine) for (auto& t : a.terms) if (t.second == sym) st += t.first * rs;
+      rs *= n.dims[p];
+    }
+    return st;
+  };
+  std::stable_sort(order.begin(), order.end(), [&](size_t x, size_t y) {
+    return lhs_stride(ph.par_syms[x]) > lhs_stride(ph.par_syms[y]); });
+  return order;
+}
+
+// ---- row groups ---------------------------------------------------------------------------------
+
+namespace {
+
+struct RowShape { std::vector<int64_t> outer; int64_t len = -1; };
+
+// Classifies `ph` as a member of a row group over `shape` (filling in what the shape leaves open).
+bool row_member(const Routine& r, Phase& ph, RowShape& shape, bool first) {
+  if (ph.kind != Phase::Generic || !ph.members.empty()) return false;
+  if (ph.inner.size() != 1 || ph.inner[0]->kind != Stmt::Set) return false;
+  for (auto f : ph.par_from) if (f != 0) return false;
+  for (auto f : ph.seq_from) if (f != 0) return false;
+  std::vector<size_t> order = store_order(r, ph);
+  std::vector<int64_t> ext;
+  std::vector<int> syms;
+  for (size_t k : order) { ext.push_back(ph.par_ext[k]); syms.push_back(ph.par_syms[k]); }
+  const size_t n = first ? 0 : shape.outer.size();
+  auto outer_matches = [&](size_t count) {
+    if (first) return true;
+    if (count != n) return false;
+    for (size_t i = 0; i < n; ++i) if (ext[i] != shape.outer[i]) return false;
+    return true;
+  };
+  Binop accum;
+  if (ph.seq_syms.size() == 1 && reduction_shape(r, ph, &accum)) {          // a row reduction
+    const int64_t T = ph.seq_to[0] + 1;
+    if (!outer_matches(ext.size()) || (shape.len >= 0 && shape.len != T) || T < 16) return false;
+    // the reduced operand must be walked contiguously
+    std::vector<Access> acc; bool fl = false; std::set<ScopeId> d;
+    scalar_accesses(*ph.inner[0]->value, acc, fl, d);
+    bool unit = false;
+    for (auto& a : acc) if (a.node != ph.inner[0]->node && get_stride(strides_of(r, a.node, *a.idcs), ph.seq_syms[0]) == 1) unit = true;
+    if (!unit) return false;
+    ph.row_role = Phase::RowReduce; ph.row_outer_syms = syms; ph.row_sym = ph.seq_syms[0];
+    if (first) shape.outer = ext;
+    shape.len = T;
+    return true;
+  }
+  if (!ph.seq_syms.empty()) return false;
+  if (ph.coop_scope) {                                                        // per-row scalar holding a reduction
+    std::vector<const Stmt*> loops; const Stmt* init = nullptr; const Stmt* upd = nullptr;
+    if (!scope_reduction(*ph.coop_scope, loops, init, upd, &accum) || loops.size() != 1 || loops[0]->from != 0) return false;
+    const int64_t T = loops[0]->to + 1;
+    if (!outer_matches(ext.size()) || (shape.len >= 0 && shape.len != T) || T < 16) return false;
+    ph.row_role = Phase::RowScalar; ph.row_outer_syms = syms; ph.row_sym = loops[0]->sym;
+    if (first) shape.outer = ext;
+    shape.len = T;
+    return true;
+  }
+  if (ph.coop_lanes != 1) return false;
+  if (!first && ext.size() == n) {                                            // per-row scalar
+    if (!outer_matches(ext.size())) return false;
+    ph.row_role = Phase::RowScalar; ph.row_outer_syms = syms; ph.row_sym = -1;
+    return true;
+  }
+  if (ext.size() < 2) return false;                                           // pointwise over rows x T
+  const int64_t T = ext.back();
+  if (!outer_matches(ext.size() - 1) || (shape.len >= 0 && shape.len != T) || T < 16) return false;
+  // the row position must be the unit-stride axis of the store
+  if (get_stride(strides_of(r, ph.inner[0]->node, ph.inner[0]->idcs), syms.back()) != 1) return false;
+  ph.row_role = Phase::RowPointwise;
+  ph.row_outer_syms.assign(syms.begin(), syms.end() - 1);
+  ph.row_sym = syms.back();
+  if (first) shape.outer.assign(ext.begin(), ext.end() - 1);
+  shape.len = T;
+  return true;
+}
+
+// Signature of an access relative to the member's row symbols: which outer axis / row position /
+// constant drives each axis.  Empty when an index is of another form.
+std::string row_signature(const Phase& ph, const Indices& idcs) {
+  std::string sig;
+  for (auto& ix : idcs) {
+    if (ix.kind == AxisIndex::Fixed) sig += "f" + std::to_string(ix.fixed);
+    else if (ix.kind == AxisIndex::Iter) {
+      if (ix.sym == ph.row_sym) sig += "r";
+      else {
+        int pos = -1;
+        for (size_t j = 0; j < ph.row_outer_syms.size(); ++j) if (ph.row_outer_syms[j] == ix.sym) pos = (int)j;
+        if (pos < 0) return "";
+        sig += "o" + std::to_string(pos);
+      }
+    } else return "";
+    sig += ",";
+  }
+  return sig.empty() ? "scalar" : sig;
+}
+
+struct RowDeps {
+  std::map<int, std::set<std::string>> sigs;   // node -> signatures seen (empty string: irregular)
+  std::set<int> written;
+  bool add(const Phase& ph) {
+    std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+    block_accesses(ph.inner, acc, w, f, d);
+    if (w || f) return false;
+    for (auto& a : acc) {
+      sigs[a.node].insert(row_signature(ph, *a.idcs));
+      if (a.write) written.insert(a.node);
+    }
+    for (int node : written) {
+      const auto& s = sigs[node];
+      if (s.size() != 1 || s.begin()->empty()) return false;
+    }
+    return true;
+  }
+};
+
+void group_rows(const Routine& r, Plan& plan) {
+  std::vector<Phase> out;
+  size_t i = 0;
+  while (i < plan.phases.size()) {
+    RowShape shape;
+    std::vector<Phase> run;
+    RowDeps deps;
+    size_t j = i;
+    while (j < plan.phases.size()) {
+      Phase cand = plan.phases[j];
+      RowShape trial = shape;
+      if (!row_member(r, cand, trial, run.empty())) break;
+      RowDeps d2 = deps;
+      if (!d2.add(cand)) break;
+      shape = trial; deps = d2;
+      run.push_back(std::move(cand));
+      ++j;
+    }
+    // a group must know its row length and be worth a launch of its own
+    int64_t rows = 1;
+    for (auto e : shape.outer) rows *= e;
+    if (run.size() >= 2 && shape.len >= 16 && rows * shape.len >= (1 << 16)) {
+      Phase g;
+      g.kind = Phase::Generic;
+      g.label = run.front().label + " .. " + run.back().label;
+      g.row_outer_ext = shape.outer;
+      g.row_len = shape.len;
+      int lanes = 1;
+      while (lanes * 2 <= 64 && lanes * 2 <= shape.len) lanes *= 2;
+      g.coop_lanes = lanes;
+      // algorithmic bytes: what the group reads from outside plus everything it writes
+      std::set<int> produced;
+      double bytes = 0;
+      for (auto& m : run) {
+        std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+        block_accesses(m.inner, acc, w, f, d);
+        std::set<int> reads_inside;
+        for (auto& a : acc) if (!a.write && produced.count(a.node)) reads_inside.insert(a.node);
+        double inside = 0;
+        for (int node : reads_inside) {
+          // the member accounted a full pass over what it reads of this node: take it out again
+          double nelem = (double)rows;
+          for (auto& a : acc) if (!a.write && a.node == node && row_signature(m, *a.idcs).find('r') != std::string::npos) { nelem = (double)rows * (double)shape.len; break; }
+          inside += std::min(nelem, (double)r.node(node).num_elems()) * prec_in_bytes(r.node(node).prec);
+        }
+        bytes += std::max(0.0, m.bytes - inside);
+        for (auto& a : acc) if (a.write) produced.insert(a.node);
+      }
+      g.bytes = bytes;
+      g.members = std::move(run);
+      out.push_back(std::move(g));
+      i = j;
+    } else {
+      out.push_back(plan.phases[i]);
+      ++i;
+    }
+  }
+  plan.phases = std::move(out);
+}
+
+}  // namespace
+
 Plan make_plan(Routine& r, const PlanOptions& opt) {
   Plan plan;
   std::string label;
@@ -894,6 +1092,7 @@ Plan make_plan(Routine& r, const PlanOptions& opt) {
     }
     plan.phases.push_back(std::move(ph));
   }
+  if (opt.enable_coop && opt.enable_row_groups) group_rows(r, plan);
   return plan;
 }
 

@@ -58,6 +58,17 @@ struct Phase {
   const Scalar* coop_scope = nullptr;
   Binop coop_accum = Binop::Add;
   bool fused_zero_init = false;  // the preceding Zero_out of the target was folded in (beta = 0)
+  // Row group (kind Generic, `members` non-empty): consecutive phases that all work row by row
+  // over the same rows -- pointwise over (rows x T), reductions of a row of T elements, per-row
+  // scalars -- and whose mutual dependencies stay inside a row.  They run as ONE kernel in which a
+  // group of `coop_lanes` lanes owns a row and executes the members in order (values pass through
+  // memory, with a workgroup fence in between, and are read back from cache).
+  std::vector<Phase> members;
+  std::vector<int64_t> row_outer_ext;   // extents of the row index space, slowest first
+  int64_t row_len = 0;                  // T
+  enum RowRole : uint8_t { RowPointwise, RowReduce, RowScalar } row_role = RowPointwise;   // as a member
+  std::vector<int> row_outer_syms;      // as a member: this phase's symbols for the outer axes, slowest first
+  int row_sym = -1;                     // as a member: its symbol for the position in the row (-1: none)
   // Fill
   int fill_node = -1;
   // Contraction
@@ -70,6 +81,7 @@ struct PlanOptions {
   int64_t min_mfma_flops = 1 << 22;   // below this a contraction stays a generic kernel
   bool enable_mfma = true;
   bool enable_coop = true;
+  bool enable_row_groups = true;
 };
 
 struct Plan {
@@ -78,5 +90,9 @@ struct Plan {
 };
 
 Plan make_plan(Routine& r, const PlanOptions& opt);
+
+// Positions of ph.par_syms ordered by their stride in the first array the phase writes, slowest
+// first: adjacent threads take adjacent values of the last one (coalesced stores).
+std::vector<size_t> store_order(const Routine& r, const Phase& ph);
 
 }  // namespace ocannl

@@ -109,6 +109,7 @@ PlanOptions parse_options(const char* options) {
     const std::string k = kv.substr(0, eq), v = kv.substr(eq + 1);
     if (k == "mfma") o.enable_mfma = v != "0";
     else if (k == "coop") o.enable_coop = v != "0";
+    else if (k == "rows") o.enable_row_groups = v != "0";
     else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
     else throw InvalidArgument("compile options: unknown key '" + k + "'");
   }
