@@ -292,6 +292,28 @@ struct Printer {
   int coop_lanes = 1;
   Binop coop_accum = Binop::Add;
   std::string store_guard;   // prefix of plain stores ("if (lane_ == 0) " when one lane stores for a group)
+  // Row groups with short rows keep what they produce in registers: a node written inside the
+  // group is also kept in `cache_name` (an array indexed by the unrolled row iteration `it_` for
+  // row-position values, a scalar every lane holds for per-row values) and later reads of it
+  // inside the group use that instead of memory.
+  int row_iters = 0;                        // > 0: loops over the row position run `it_` = 0..row_iters-1, unrolled
+  std::map<int, std::string> cache_name;    // node -> register expression
+  std::set<int> cache_defined;              // nodes whose cache holds the current value
+  // `lhs = value;` with the cache kept in step
+  std::string store_line(int node, const std::string& lhs, const std::string& value, const std::string& guard) {
+    auto it = cache_name.find(node);
+    if (it == cache_name.end()) return guard + lhs + " = " + value + ";";
+    cache_defined.insert(node);
+    return it->second + " = " + value + "; " + guard + lhs + " = " + it->second + ";";
+  }
+  // header of a loop over the row position shared by `lanes` lanes
+  std::string row_loop(const std::string& sym, int64_t from, int64_t to, int lanes, const std::string& ind) {
+    if (row_iters > 0 && from == 0)
+      return ind + "_Pragma(\"unroll\") for (uint32_t it_ = 0; it_ < " + std::to_string(row_iters) + "; ++it_) { const uint32_t " +
+             sym + " = lane_ + it_ * " + std::to_string(lanes) + ";";
+    return ind + "for (uint32_t " + sym + " = " + std::to_string(from) + " + lane_; " + sym + " <= " + std::to_string(to) +
+           "; " + sym + " += " + std::to_string(lanes) + ") {";
+  }
   // when set, a read of exactly this (node, indices) prints as `self_name`
   const Stmt* self_set = nullptr;
   std::string self_name;
@@ -341,6 +363,7 @@ struct Printer {
         const Node& n = r.node(s.node);
         Pair c = convert_precision(n.prec, prec);
         if (self_set && s.node == self_set->node && s.idcs == self_set->idcs) return c.first + self_name + c.second;
+        if (cache_defined.count(s.node)) return c.first + cache_name.at(s.node) + c.second;
         note(s.node, s.idcs);
         return c.first + n.ident + "[" + offset_str(s.idcs, n.dims) + "]" + c.second;
       }
@@ -417,8 +440,7 @@ struct Printer {
     for (size_t i = 0; i < loops.size(); ++i) {
       const std::string sy = sym_ident(loops[i]->sym);
       if (i + 1 == loops.size())
-        d.lines.push_back(ci + "for (uint32_t " + sy + " = " + std::to_string(loops[i]->from) + " + lane_; " + sy + " <= " +
-                          std::to_string(loops[i]->to) + "; " + sy + " += " + std::to_string(coop_lanes) + ") {");
+        d.lines.push_back(row_loop(sy, loops[i]->from, loops[i]->to, coop_lanes, ci));
       else
         d.lines.push_back(ci + "for (uint32_t " + sy + " = " + std::to_string(loops[i]->from) + "; " + sy + " <= " +
                           std::to_string(loops[i]->to) + "; ++" + sy + ") {");
@@ -488,7 +510,7 @@ struct Printer {
         note(c.node, c.idcs);
         std::vector<Def> defs;
         std::string v = scalar(n.prec, *c.value, ind + "  ", defs);
-        with_defs(defs, {store_guard + n.ident + "[" + offset_str(c.idcs, n.dims) + "] = " + v + ";"}, ind, out);
+        with_defs(defs, {store_line(c.node, n.ident + "[" + offset_str(c.idcs, n.dims) + "]", v, store_guard)}, ind, out);
         break;
       }
       case Stmt::SetVec: {
@@ -577,8 +599,7 @@ void emit_phase_statements(const Routine& r, Printer& pr, const Phase& ph, int G
     for (size_t i = 0; i < ph.seq_syms.size(); ++i) {
       const std::string s = sym_ident(ph.seq_syms[i]);
       if (coop_last && i + 1 == ph.seq_syms.size())
-        body.push_back(cur_ind + "for (uint32_t " + s + " = " + std::to_string(ph.seq_from[i]) + " + lane_; " + s +
-                       " <= " + std::to_string(ph.seq_to[i]) + "; " + s + " += " + std::to_string(G) + ") {");
+        body.push_back(pr.row_loop(s, ph.seq_from[i], ph.seq_to[i], G, cur_ind));
       else
         body.push_back(cur_ind + "for (uint32_t " + s + " = " + std::to_string(ph.seq_from[i]) + "; " + s + " <= " +
                        std::to_string(ph.seq_to[i]) + "; ++" + s + ") {");
@@ -622,11 +643,14 @@ void emit_phase_statements(const Routine& r, Printer& pr, const Phase& ph, int G
     const std::string lhs = n.ident + "[" + offset_str(set->idcs, n.dims) + "]";
     Pair narrow = convert_precision(accP, n.prec);
     Pair wide = convert_precision(n.prec, accP);
+    // (every lane holds the combined value after the butterfly)
     if (ph.fused_zero_init)
-      body.push_back(ind + "if (lane_ == 0) " + lhs + " = " + narrow.first + "part_" + narrow.second + ";");
-    else
-      body.push_back(ind + "if (lane_ == 0) " + lhs + " = " + narrow.first +
-                     combine_expr(accum, dbl, wide.first + lhs + wide.second, "part_") + narrow.second + ";");
+      body.push_back(ind + pr.store_line(set->node, lhs, narrow.first + "part_" + narrow.second, "if (lane_ == 0) "));
+    else {
+      const std::string old_v = pr.cache_defined.count(set->node) ? pr.cache_name.at(set->node) : lhs;
+      body.push_back(ind + pr.store_line(set->node, lhs, narrow.first +
+                     combine_expr(accum, dbl, wide.first + old_v + wide.second, "part_") + narrow.second, "if (lane_ == 0) "));
+    }
   } else if (is_reduction) {
     // one thread per output element, sequential loops in the reference's order: for fp32 this is
     // the same operation sequence as the `cc` backend's serial loop.
@@ -634,7 +658,8 @@ void emit_phase_statements(const Routine& r, Printer& pr, const Phase& ph, int G
     pr.note(set->node, set->idcs);
     const std::string lhs = n.ident + "[" + offset_str(set->idcs, n.dims) + "]";
     Pair zero = convert_precision(Prec::Double, n.prec);
-    body.push_back(ind + c_typ(n.prec) + " acc_ = " + (ph.fused_zero_init ? zero.first + "0" + zero.second : lhs) + ";");
+    const std::string old_v = pr.cache_defined.count(set->node) ? pr.cache_name.at(set->node) : lhs;
+    body.push_back(ind + c_typ(n.prec) + " acc_ = " + (ph.fused_zero_init ? zero.first + "0" + zero.second : old_v) + ";");
     std::string ci = ind;
     open_seq_loops(ci, false);
     pr.self_set = set; pr.self_name = "acc_";
@@ -644,7 +669,7 @@ void emit_phase_statements(const Routine& r, Printer& pr, const Phase& ph, int G
     pr.with_defs(defs, {"acc_ = " + v + ";"}, ci, body);
     pr.self_set = nullptr;
     close_seq_loops(ci);
-    body.push_back(ind + lane0 + lhs + " = acc_;");
+    body.push_back(ind + pr.store_line(set->node, lhs, "acc_", lane0));
     pr.coop_scope = nullptr;
   } else {
     if (ph.fused_zero_init) throw InvalidArgument("planner: fused zero-init on a non-reduction phase");
@@ -695,18 +720,36 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
         else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
         body.push_back(line);
       }
+      // short rows: everything the group produces stays in registers as well (no read-back)
+      const bool cached = ph.row_len % G == 0 && ph.row_len / G <= 16;
+      if (cached) {
+        pr.row_iters = (int)(ph.row_len / G);
+        for (auto& m : ph.members) {
+          const Stmt& st = *m.inner[0];
+          if (pr.cache_name.count(st.node)) continue;
+          const Node& wn = r.node(st.node);
+          bool per_position = false;
+          for (auto& ix : st.idcs) if (ix.kind == AxisIndex::Iter && ix.sym == m.row_sym && m.row_role == Phase::RowPointwise) per_position = true;
+          const std::string base = "c" + std::to_string(st.node) + "_";
+          if (per_position) {
+            body.push_back(ind + c_typ(wn.prec) + " " + base + "[" + std::to_string(pr.row_iters) + "];");
+            pr.cache_name[st.node] = base + "[it_]";
+          } else {
+            body.push_back(ind + c_typ(wn.prec) + " " + base + ";");
+            pr.cache_name[st.node] = base;
+          }
+        }
+      }
       for (size_t mi = 0; mi < ph.members.size(); ++mi) {
         const Phase& m = ph.members[mi];
-        if (mi) body.push_back(ind + "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\"); "
-                                     "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
+        if (mi && !cached) body.push_back(ind + "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\"); "
+                                                "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
         body.push_back(ind + "{  /* " + m.label + " */");
         const std::string mi_ind = ind + "  ";
         for (size_t k = 0; k < m.row_outer_syms.size(); ++k)
           body.push_back(mi_ind + "const uint32_t " + sym_ident(m.row_outer_syms[k]) + " = row" + std::to_string(k) + "_;");
         if (m.row_role == Phase::RowPointwise) {
-          const std::string s = sym_ident(m.row_sym);
-          body.push_back(mi_ind + "for (uint32_t " + s + " = lane_; " + s + " < " + std::to_string(ph.row_len) + "; " + s +
-                         " += " + std::to_string(G) + ") {");
+          body.push_back(pr.row_loop(sym_ident(m.row_sym), 0, ph.row_len - 1, G, mi_ind));
           emit_phase_statements(r, pr, m, 1, false, mi_ind + "  ", body);
           body.push_back(mi_ind + "}");
         } else {
