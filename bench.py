@@ -8,7 +8,8 @@ A "step" is one run of the compiled routine (for the training configurations: fo
 are resident in device memory before the timed region starts.  Prints one JSON line.
 
 workloads: transformer (BASELINE config 4, default), dense_bf16 / dense_f32 (config 3),
-attention (config 5), char_mlp (config 2), moons (config 1).
+attention (config 5), char_mlp (config 2), moons (config 1), copy (a 2 x 256 MiB plain copy: the
+yardstick that memory-traffic counters are scaled by).
 """
 from __future__ import annotations
 
@@ -41,7 +42,24 @@ def build_workload(name: str):
         return W.char_mlp(), "train_steps_per_sec", "steps/s", "f32"
     if name == "moons":
         return W.moons_mlp(), "train_steps_per_sec", "steps/s", "f32"
+    if name == "copy":
+        return W.plain_copy(), "train_steps_per_sec", "steps/s", "f32"
     raise SystemExit(f"unknown workload {name}")
+
+
+def measured_traffic(workload: str, kernel: str):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 counter summary of this
+    workload (profiles/<workload>_step_hbm_traffic.txt), or None when there is none."""
+    path = os.path.join(ROOT, "profiles", f"{workload}_step_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        for line in f:
+            if line.startswith("TRAFFIC "):
+                parts = [p.strip() for p in line[len("TRAFFIC "):].split("|")]
+                if parts[0] == kernel:
+                    return float(parts[-1].split()[-1])
+    return None
 
 
 def cpu_baseline(name: str):
@@ -81,6 +99,9 @@ def cpu_baseline(name: str):
         w = W.char_mlp()
         t = time_steps(w, 2000, {w.statics["batch_n"].sym: 0})
         return {"value": 1.0 / t, "unit": "steps/s", "cores": 1, "kind": "port", "sample": "2000 full steps"}
+    if name == "copy":
+        t = time_steps(W.plain_copy(), 5)
+        return {"value": 1.0 / t, "unit": "steps/s", "cores": 1, "kind": "port", "sample": "5 full steps"}
     w = W.moons_mlp()
     t = time_steps(w, 20000, {w.statics["batch_n"].sym: 0})
     return {"value": 1.0 / t, "unit": "steps/s", "cores": 1, "kind": "port", "sample": "20000 full steps"}
@@ -174,13 +195,15 @@ def main():
         f32 = "gemm_f32" in dom_name
         peak = PEAKS["mfma_f32"] if f32 else PEAKS["mfma_bf16"]
         roof = {"bound": "mfma", "kernel": dom_name, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                "frac": achieved / peak, "traffic": None, "launches_per_step": len(dom_idx),
+                "frac": achieved / peak, "traffic": measured_traffic(args.workload, dom_name),
+                "launches_per_step": len(dom_idx),
                 "avg_launch_ms": avg_ms, "flops_per_launch": per_launch}
     else:
         per_launch = kernels[dom_idx[0]]["bytes"]
         achieved = per_launch / (avg_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": PEAKS["hbm"], "unit": "GB/s",
-                "frac": achieved / PEAKS["hbm"], "traffic": None, "launches_per_step": 1, "avg_launch_ms": avg_ms,
+                "frac": achieved / PEAKS["hbm"], "traffic": measured_traffic(args.workload, dom_name),
+                "launches_per_step": 1, "avg_launch_ms": avg_ms,
                 "bytes_per_launch": per_launch}
 
     out = {

@@ -104,21 +104,28 @@ __device__ __forceinline__ void decode_batch(const GemmArgs& g, long z, long& ao
   if (g.nbatch > 0) { const long e = g.batch_ext[0], q = z % e; ao += q * g.a_batch[0]; bo += q * g.b_batch[0]; co += q * g.c_batch[0]; }
 }
 
-// XCD-aware tile order: consecutive hardware workgroup ids land on different XCDs; give XCD x the
-// x-th contiguous slice of the tile sequence, and walk tiles in column-bands of 8 row-tiles so that
-// a slice re-uses the same B panels.
-__device__ __forceinline__ void tile_of_block(long wg, long tiles_m, long tiles_n, long& tm, long& tn) {
-  const long total = tiles_m * tiles_n;
-  long t = wg;
-  if (total % 8 == 0) t = (wg % 8) * (total / 8) + wg / 8;
+// XCD-aware tile order.  Consecutive hardware workgroup ids land on different XCDs (id % 8), each
+// with its own L2.  The tile grid is cut into xcd_m x (8 / xcd_m) rectangles, one per XCD, chosen
+// on the host so that the operand panels shared inside a rectangle are the expensive ones
+// (fewest bytes re-read across XCDs).  Inside its rectangle an XCD walks column-bands of 8
+// row-tiles, so that tiles running at the same time share B panels.
+__device__ __forceinline__ void tile_of_block(long wg, long tiles_m, long tiles_n, int xcd_m, long& tm, long& tn) {
+  long t = wg, rm = tiles_m, rn = tiles_n, m_off = 0, n_off = 0;
+  if (xcd_m > 0) {
+    const int xcd_n = 8 / xcd_m;
+    const long x = wg % 8;
+    rm = tiles_m / xcd_m; rn = tiles_n / xcd_n;
+    m_off = (x / xcd_n) * rm; n_off = (x % xcd_n) * rn;
+    t = wg / 8;
+  }
   constexpr long kGroup = 8;
-  const long band = kGroup * tiles_n;
+  const long band = kGroup * rn;
   const long g = t / band;
   const long first_m = g * kGroup;
-  const long gm = (tiles_m - first_m) < kGroup ? (tiles_m - first_m) : kGroup;
+  const long gm = (rm - first_m) < kGroup ? (rm - first_m) : kGroup;
   const long r = t % band;
-  tm = first_m + r % gm;
-  tn = r / gm;
+  tm = m_off + first_m + r % gm;
+  tn = n_off + r / gm;
 }
 
 // ---- staging one operand tile: global -> registers -> LDS --------------------------------------
@@ -292,7 +299,7 @@ gemm_bf16_kernel(const GemmArgs g) {
   const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
   const long tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
   long tmi, tni;
-  tile_of_block(blockIdx.x, tiles_m, tiles_n, tmi, tni);
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, g.xcd_m, tmi, tni);
   const long m0 = tmi * BM, n0 = tni * BN;
   long ao, bo, co;
   decode_batch(g, blockIdx.z, ao, bo, co);
@@ -453,7 +460,7 @@ gemm_f32_kernel(const GemmArgs g) {
   const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
   const long tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
   long tmi, tni;
-  tile_of_block(blockIdx.x, tiles_m, tiles_n, tmi, tni);
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, g.xcd_m, tmi, tni);
   const long m0 = tmi * BM, n0 = tni * BN;
   long ao, bo, co;
   decode_batch(g, blockIdx.z, ao, bo, co);
@@ -586,7 +593,7 @@ bool big_tile(const GemmDesc& d) { return tile_config(d).big; }
 int split_count(const GemmDesc& d) { return tile_config(d).splits; }
 
 template <typename K>
-hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t s) {
+hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t s, hipEvent_t after_main) {
   static thread_local const void* configured[64];
   static thread_local int n_configured = 0;
   bool done = false;
@@ -603,6 +610,7 @@ hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t
   if (a.splits > 1 && !a.ws) return hipErrorInvalidValue;
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)a.splits, (unsigned)nb), dim3(kThreads), smem, s, a);
   hipError_t e = hipGetLastError();
+  if (e == hipSuccess && after_main) e = hipEventRecord(after_main, s);
   if (e != hipSuccess || a.splits <= 1) return e;
   const long groups = a.M * (a.N / 4);
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((groups + 255) / 256), 1, (unsigned)nb), dim3(256), 0, s, a);
@@ -610,21 +618,21 @@ hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t
 }
 
 template <int BM, int BN, typename AT, typename BT>
-hipError_t launch_bf16_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t s) {
+hipError_t launch_bf16_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t s, hipEvent_t ev) {
   constexpr size_t sm = bf16_smem<BM, BN>();
-  if (akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, true>, sm, BM, BN, a, s);
-  if (akc && !bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, false>, sm, BM, BN, a, s);
-  if (!akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, true>, sm, BM, BN, a, s);
-  return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, false>, sm, BM, BN, a, s);
+  if (akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, true>, sm, BM, BN, a, s, ev);
+  if (akc && !bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, false>, sm, BM, BN, a, s, ev);
+  if (!akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, true>, sm, BM, BN, a, s, ev);
+  return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, false>, sm, BM, BN, a, s, ev);
 }
 
 template <int BM, int BN>
-hipError_t launch_f32_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t s) {
+hipError_t launch_f32_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t s, hipEvent_t ev) {
   constexpr size_t sm = f32_smem<BM, BN>();
-  if (akc && bkc) return launch(gemm_f32_kernel<BM, BN, true, true>, sm, BM, BN, a, s);
-  if (akc && !bkc) return launch(gemm_f32_kernel<BM, BN, true, false>, sm, BM, BN, a, s);
-  if (!akc && bkc) return launch(gemm_f32_kernel<BM, BN, false, true>, sm, BM, BN, a, s);
-  return launch(gemm_f32_kernel<BM, BN, false, false>, sm, BM, BN, a, s);
+  if (akc && bkc) return launch(gemm_f32_kernel<BM, BN, true, true>, sm, BM, BN, a, s, ev);
+  if (akc && !bkc) return launch(gemm_f32_kernel<BM, BN, true, false>, sm, BM, BN, a, s, ev);
+  if (!akc && bkc) return launch(gemm_f32_kernel<BM, BN, false, true>, sm, BM, BN, a, s, ev);
+  return launch(gemm_f32_kernel<BM, BN, false, false>, sm, BM, BN, a, s, ev);
 }
 
 bool a_kcontig(const GemmDesc& d) { return d.a.s_k == 1 || d.K == 1; }
@@ -651,22 +659,37 @@ size_t gemm_workspace_bytes(const GemmDesc& d) {
   return sp > 1 ? (size_t)sp * (size_t)batch_count(d) * (size_t)d.M * (size_t)d.N * sizeof(float) : 0;
 }
 
-hipError_t launch_gemm(const GemmDesc& d, const GemmArgs& a_in, void* workspace, hipStream_t s) {
+hipError_t launch_gemm(const GemmDesc& d, const GemmArgs& a_in, void* workspace, hipStream_t s, hipEvent_t ev) {
   GemmArgs a = a_in;
   a.splits = split_count(d);
   a.ws = static_cast<float*>(workspace);
   const bool akc = a_kcontig(d), bkc = b_kcontig(d);
   const bool big = big_tile(d);
+  {
+    // XCD partition: every A panel is read by each of the xcd_n rectangle columns, every B panel
+    // by each of the xcd_m rows
+    const long tile = big ? 256 : 128;
+    const long tiles_m = (d.M + tile - 1) / tile, tiles_n = (d.N + tile - 1) / tile;
+    const double a_bytes = (double)d.M * prec_in_bytes(d.a.prec), b_bytes = (double)d.N * prec_in_bytes(d.b.prec);
+    a.xcd_m = 0;
+    double best = 0;
+    for (int xm = 1; xm <= 8; xm *= 2) {
+      const int xn = 8 / xm;
+      if (tiles_m % xm || tiles_n % xn) continue;
+      const double cost = a_bytes * xn + b_bytes * xm;
+      if (a.xcd_m == 0 || cost < best) { a.xcd_m = xm; best = cost; }
+    }
+  }
   const bool af = d.a.prec == Prec::Single, bf = d.b.prec == Prec::Single;
-  if (af && bf) return big ? launch_f32_layout<256, 256>(akc, bkc, a, s) : launch_f32_layout<128, 128>(akc, bkc, a, s);
+  if (af && bf) return big ? launch_f32_layout<256, 256>(akc, bkc, a, s, ev) : launch_f32_layout<128, 128>(akc, bkc, a, s, ev);
   if (!af && !bf)
-    return big ? launch_bf16_layout<256, 256, unsigned short, unsigned short>(akc, bkc, a, s)
-               : launch_bf16_layout<128, 128, unsigned short, unsigned short>(akc, bkc, a, s);
+    return big ? launch_bf16_layout<256, 256, unsigned short, unsigned short>(akc, bkc, a, s, ev)
+               : launch_bf16_layout<128, 128, unsigned short, unsigned short>(akc, bkc, a, s, ev);
   if (af && !bf)
-    return big ? launch_bf16_layout<256, 256, float, unsigned short>(akc, bkc, a, s)
-               : launch_bf16_layout<128, 128, float, unsigned short>(akc, bkc, a, s);
-  return big ? launch_bf16_layout<256, 256, unsigned short, float>(akc, bkc, a, s)
-             : launch_bf16_layout<128, 128, unsigned short, float>(akc, bkc, a, s);
+    return big ? launch_bf16_layout<256, 256, float, unsigned short>(akc, bkc, a, s, ev)
+               : launch_bf16_layout<128, 128, float, unsigned short>(akc, bkc, a, s, ev);
+  return big ? launch_bf16_layout<256, 256, unsigned short, float>(akc, bkc, a, s, ev)
+             : launch_bf16_layout<128, 128, unsigned short, float>(akc, bkc, a, s, ev);
 }
 
 }  // namespace ocannl

@@ -18,6 +18,7 @@ struct GemmArgs {
   int64_t a_batch[3], b_batch[3], c_batch[3];
   int accumulate;    // beta = 1
   int c_is_bf16;
+  int xcd_m;         // tile-grid rows of the XCD partition (set by launch_gemm; 0: none)
   int splits;        // split-K factor (set by launch_gemm)
   float* ws;         // split-K workspace [batch][split][M][N] (set by launch_gemm)
 };
@@ -25,7 +26,10 @@ struct GemmArgs {
 // Picks the kernel instance for the operand precisions / layouts and launches it on `stream`.
 // Returns hipErrorInvalidValue for a combination the planner should not have produced.
 // `workspace` must hold gemm_workspace_bytes(desc) bytes (may be null when that is 0).
-hipError_t launch_gemm(const GemmDesc& desc, const GemmArgs& args, void* workspace, hipStream_t stream);
+// `after_main`, when not null, is recorded on the stream right after the contraction kernel itself
+// (before the split-K reduction, if one follows), for per-kernel timing.
+hipError_t launch_gemm(const GemmDesc& desc, const GemmArgs& args, void* workspace, hipStream_t stream,
+                       hipEvent_t after_main = nullptr);
 
 // Bytes of split-K workspace this contraction needs (0 when K is not split).
 size_t gemm_workspace_bytes(const GemmDesc& desc);

@@ -227,11 +227,14 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
       }
       a.accumulate = g.accumulate ? 1 : 0;
       a.c_is_bf16 = g.c.prec == Prec::Bfloat16;
-      hip_check(launch_gemm(g, a, rt.gemm_ws, dev.stream), "launch_gemm");
+      // a bracketed contraction is timed without its split-K reduction (a kernel of its own)
+      hip_check(launch_gemm(g, a, rt.gemm_ws, dev.stream, bracket ? rt.profile_events[rt.profile_used + 1] : nullptr),
+                "launch_gemm");
     }
     if (timed) hip_check(hipEventRecord(rt.timing_events[li + 1], dev.stream), "hipEventRecord");
     if (bracket) {
-      hip_check(hipEventRecord(rt.profile_events[rt.profile_used + 1], dev.stream), "hipEventRecord");
+      if (ph.kind != Phase::Contraction)
+        hip_check(hipEventRecord(rt.profile_events[rt.profile_used + 1], dev.stream), "hipEventRecord");
       rt.profile_used += 2;
     }
   }

@@ -171,6 +171,19 @@ def dense_contraction(b: int = 8192, i: int = 4096, o: int = 4096, prec: str = "
                     f"b|i->o contraction b={b} i={i} o={o} {prec} (dest {out_prec}), fwd+dX+dW")
 
 
+def plain_copy(n: int = 1 << 26, prec: str = "single") -> Workload:
+    """``y[i] = x[i]`` over ``n`` elements: one generated kernel that reads and writes a known
+    number of bytes -- the yardstick for memory-traffic counters."""
+    L.reset_symbols(0)
+    x = L.Node(1, "x", prec, (n,)); y = L.Node(2, "y", prec, (n,))
+    i = L.fresh_symbol()
+    routine = L.Routine("plain_copy", [L.For(i, 0, n - 1, [L.Set(y, (L.It(i),), L.Get(x, (L.It(i),)))])])
+    rng = np.random.default_rng(0)
+    init = {1: as_prec(rng.uniform(-1, 1, n).astype(np.float32), prec)}
+    return Workload("plain_copy", routine, init, {"x": x, "y": y}, {}, [y],
+                    f"copy of {n} {prec} elements ({2 * x.size_in_bytes} bytes of traffic)")
+
+
 # ------------------------------------------------------------------------------------------------
 # config 2: character-level MLP language model
 # ------------------------------------------------------------------------------------------------
