@@ -114,6 +114,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="transformer")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--options", default=None, help="compile options for the library, e.g. 'rows=0;bf16_copies=0'")
     ap.add_argument("--kernel-table", action="store_true", help="print per-kernel times to stderr")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -124,7 +125,7 @@ def main():
 
     w, metric, unit, dtype = build_workload(args.workload)
     t_c = time.perf_counter()
-    hip = HipRun(w.routine, w.init)
+    hip = HipRun(w.routine, w.init, args.options)
     compile_s = time.perf_counter() - t_c
     kernels = hip.code.kernels()
     statics = {s.sym: 0 for s in w.statics.values()}

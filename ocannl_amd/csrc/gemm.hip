@@ -51,11 +51,18 @@ __device__ __forceinline__ void static_for(F&& f) {
 // Phase timestamps for kernel tuning (compiled in only with -DOCANNL_GEMM_TIMING): workgroup w
 // writes the 100 MHz wall clock at stamp i to g_gemm_stamps[8 * w + i].
 #ifdef OCANNL_GEMM_TIMING
+__device__ int g_probe_skip;   // bit 0: no global loads / LDS stores in the main loop; bit 1: no LDS fragment reads
+#define OCANNL_PROBE_SKIP(bit) (g_probe_skip & (bit))
 __device__ long long g_gemm_stamps[8 * 4096];
 #define OCANNL_STAMP(i) \
   do { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && blockIdx.x < 4096) g_gemm_stamps[8 * blockIdx.x + (i)] = wall_clock64(); } while (0)
 #else
 #define OCANNL_STAMP(i) do { } while (0)
+#define OCANNL_PROBE_SKIP(bit) 0
+#endif
+
+#ifndef OCANNL_GEMM_DEEP_PREFETCH
+#define OCANNL_GEMM_DEEP_PREFETCH 0   // 1: two global-load register sets for the bf16 256x256 tile (spills next to double-buffered fragments)
 #endif
 
 constexpr int kThreads = 256;
@@ -165,6 +172,52 @@ struct Stager {
     }
   }
 
+  // The same work cut into single instructions for the interleaved main loop of full tiles (no
+  // bounds checks): kOps loads, then kOps LDS writes, in matching order.  An address is a part
+  // that is uniform over the workgroup (tile origin, op number: scalar registers / immediates) plus
+  // one per-thread 32-bit offset computed once by init_ops().  In the row-contiguous case with
+  // fewer than 256 rows the upper threads repeat the lower threads' blocks (identical values to
+  // identical addresses) instead of branching.
+  static constexpr int kOps = KC ? kChunks : kBlocks * 8;
+  static_assert(KC || kBlocks == 1, "one 8x8 block per thread");
+  unsigned goff, loff;
+
+  __device__ __forceinline__ void init_ops(long ld, int tid) {
+    constexpr int kStride = kBK + kPad;
+    if (KC) {
+      goff = (unsigned)((tid / (kBK / 8)) * ld + (tid % (kBK / 8)) * 8);
+      loff = (tid / (kBK / 8)) * kStride + (tid % (kBK / 8)) * 8;
+    } else {
+      const int blk = tid % ROWS;
+      goff = (unsigned)((blk % (kBK / 8)) * 8 * ld + (blk / (kBK / 8)) * 8);
+      loff = (blk / (kBK / 8)) * 8 * kStride + (blk % (kBK / 8)) * 8;
+    }
+  }
+
+  // `origin` points at the tile's first element (row0, k0): uniform.
+  template <int I>
+  __device__ __forceinline__ void load_op(const T* origin, long ld) {
+    if (KC) regs[I].load(origin + (long)(I * (kThreads / (kBK / 8))) * ld + goff);
+    else regs[I].load(origin + (long)I * ld + goff);
+  }
+
+  template <int I>
+  __device__ __forceinline__ void store_op(unsigned short* lds) const {
+    constexpr int kStride = kBK + kPad;
+    if (KC) {
+      *reinterpret_cast<u32x4*>(lds + loff + I * (kThreads / (kBK / 8)) * kStride) = regs[I].bf16();
+    } else {
+      constexpr int m = I;
+      unsigned w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const unsigned lo = regs[2 * j].bf16()[m / 2], hi = regs[2 * j + 1].bf16()[m / 2];
+        w[j] = __builtin_amdgcn_perm(hi, lo, (m & 1) ? 0x07060302u : 0x05040100u);
+      }
+      *reinterpret_cast<u32x4*>(lds + loff + m * kStride) = u32x4{w[0], w[1], w[2], w[3]};
+    }
+  }
+
   __device__ __forceinline__ void store(unsigned short* lds, int tid) const {
     constexpr int kStride = kBK + kPad;
     if (KC) {
@@ -189,7 +242,7 @@ struct Stager {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const unsigned lo = in[2 * j][m / 2], hi = in[2 * j + 1][m / 2];
-            w[j] = (m & 1) ? ((lo >> 16) | (hi & 0xFFFF0000u)) : ((lo & 0xFFFFu) | (hi << 16));
+            w[j] = __builtin_amdgcn_perm(hi, lo, (m & 1) ? 0x07060302u : 0x05040100u);   // one 16-bit half of each
           }
           *reinterpret_cast<u32x4*>(lds + (row + m) * kStride + kg) = u32x4{w[0], w[1], w[2], w[3]};
         }
@@ -286,7 +339,8 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, f32x16 (&acc)[TM][TN
 // One wavefront per SIMD for the 256x256 tile (the 256 accumulator registers live in AGPRs and the
 // whole 512-register budget is available); two for the 128x128 tile.
 template <int BM, int BN, typename AT, typename BT, bool A_KC, bool B_KC>
-__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, BM >= 256 ? 1 : 2)))
+__global__ void __launch_bounds__(kThreads)
+__attribute__((amdgpu_waves_per_eu((BM < 256 && sizeof(AT) == 2 && sizeof(BT) == 2) ? 2 : 1, BM >= 256 ? 1 : 2)))
 gemm_bf16_kernel(const GemmArgs g) {
   constexpr int kStride = kBK + kPad;
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
@@ -324,7 +378,7 @@ gemm_bf16_kernel(const GemmArgs g) {
   // Software pipeline.  LDS is double buffered; global loads run kPF tiles ahead of the tile being
   // multiplied, held in kPF register sets.  One set is what the register file affords next to a
   // 256-register accumulator; the code is written for any depth.
-  constexpr int kPF = (BM >= 256 && sizeof(AT) == 2 && sizeof(BT) == 2) ? 2 : 1;
+  constexpr int kPF = (OCANNL_GEMM_DEEP_PREFETCH && BM >= 256 && sizeof(AT) == 2 && sizeof(BT) == 2) ? 2 : 1;
   Stager<BM, AT, A_KC> sa[kPF];
   Stager<BN, BT, B_KC> sb[kPF];
   sa[0].load(A, lda, m0, kbeg, g.M, kend, tid);
@@ -344,39 +398,120 @@ gemm_bf16_kernel(const GemmArgs g) {
     constexpr int par = decltype(par_c)::value;
     const int cur = ks & 1;
     // register set `par` held tile ks (already in LDS): refill it with tile ks + kPF
-    if (ks + kPF < ksteps) {
+    if (ks + kPF < ksteps && !OCANNL_PROBE_SKIP(1)) {
       sa[par].load(A, lda, m0, kbeg + (ks + kPF) * kBK, g.M, kend, tid);
       sb[par].load(B, ldb, n0, kbeg + (ks + kPF) * kBK, g.N, kend, tid);
     }
     __builtin_amdgcn_sched_barrier(0);   // the loads are issued before the MFMA block, not sunk below it
     const unsigned short* as = As0 + cur * BM * kStride + (wm0 + (lane & 31)) * kStride + (lane >> 5) * 8;
     const unsigned short* bs = Bs0 + cur * BN * kStride + (wn0 + (lane & 31)) * kStride + (lane >> 5) * 8;
-#pragma unroll
-    for (int kk = 0; kk < kBK / 16; ++kk) {
-      bf16x8 af[TM], bf[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(as + i * 32 * kStride + kk * 16);
-#pragma unroll
-      for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const bf16x8*>(bs + j * 32 * kStride + kk * 16);
+    // fragments are double buffered: the LDS reads of sub-step kk + 1 are issued before the MFMAs
+    // of sub-step kk, so that a lone wave per SIMD does not sit out the LDS latency every time
+    bf16x8 af[2][TM], bf[2][TN];
+    auto read_frags = [&](auto kkc) OCN_LAMBDA_INLINE {
+      constexpr int kk = decltype(kkc)::value, fb = kk & 1;
+      static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
+        constexpr int i = decltype(ic)::value;
+        af[fb][i] = *reinterpret_cast<const bf16x8*>(as + i * 32 * kStride + kk * 16);
+      });
+      static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
+        constexpr int j = decltype(jc)::value;
+        bf[fb][j] = *reinterpret_cast<const bf16x8*>(bs + j * 32 * kStride + kk * 16);
+      });
+    };
+    read_frags(std::integral_constant<int, 0>{});
+    static_for<kBK / 16>([&](auto kkc) OCN_LAMBDA_INLINE {
+      constexpr int kk = decltype(kkc)::value, fb = kk & 1;
+      if constexpr (kk + 1 < kBK / 16) {
+        if (!OCANNL_PROBE_SKIP(2)) read_frags(std::integral_constant<int, kk + 1>{});
+        __builtin_amdgcn_sched_barrier(0);
+      }
       static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
         static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
           constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[fb][i], bf[fb][j], acc[i][j], 0, 0, 0);
         });
       });
-    }
+    });
     __builtin_amdgcn_sched_barrier(0);
     // tile ks + 1 sits in the other register set (or, with one set, in the one just refilled)
-    if (ks + 1 < ksteps) {
+    if (ks + 1 < ksteps && !OCANNL_PROBE_SKIP(1)) {
       constexpr int nxt = (par + 1) % kPF;
       sa[nxt].store(As0 + (cur ^ 1) * BM * kStride, tid);
       sb[nxt].store(Bs0 + (cur ^ 1) * BN * kStride, tid);
     }
     __syncthreads();
   };
-  long ks = 0;
-  for (; ks + kPF <= ksteps; ks += kPF) static_for<kPF>([&](auto p) OCN_LAMBDA_INLINE { step(ks + decltype(p)::value, p); });
-  static_for<kPF>([&](auto p) OCN_LAMBDA_INLINE { if (ks + decltype(p)::value < ksteps) step(ks + decltype(p)::value, p); });
+  // Interleaved K step for full tiles: one basic block in which the other instructions are placed
+  // between the MFMAs by hand (and pinned there), so that they issue while the matrix pipe is busy
+  // -- with one wave per SIMD nothing else would hide them.  Global loads of tile ks + 1 go with
+  // the first half of the MFMAs, its LDS writes with the second half, the LDS reads of the next
+  // sub-step's fragments with the current sub-step.
+  auto fast_step = [&](long ks, auto loads_c) __attribute__((always_inline)) {
+    constexpr bool kLoads = decltype(loads_c)::value;
+    constexpr int kSub = kBK / 16, kPer = TM * TN, kAll = kSub * kPer, kHalf = kAll / 2;
+    constexpr int kA = Stager<BM, AT, A_KC>::kOps, kL = kA + Stager<BN, BT, B_KC>::kOps, kR = TM + TN;
+    const int cur = ks & 1;
+    const long kn = kbeg + (ks + 1) * kBK;
+    const AT* const a_next = A_KC ? A + m0 * lda + kn : A + kn * lda + m0;
+    const BT* const b_next = B_KC ? B + n0 * ldb + kn : B + kn * ldb + n0;
+    unsigned short* const an = As0 + (cur ^ 1) * BM * kStride;
+    unsigned short* const bn = Bs0 + (cur ^ 1) * BN * kStride;
+    const unsigned short* as = As0 + cur * BM * kStride + (wm0 + (lane & 31)) * kStride + (lane >> 5) * 8;
+    const unsigned short* bs = Bs0 + cur * BN * kStride + (wn0 + (lane & 31)) * kStride + (lane >> 5) * 8;
+    bf16x8 af[2][TM], bf[2][TN];
+    auto read_frag = [&](auto kkc, auto rc) OCN_LAMBDA_INLINE {
+      constexpr int kk = decltype(kkc)::value, r = decltype(rc)::value, fb = kk & 1;
+      if constexpr (r < TM) af[fb][r] = *reinterpret_cast<const bf16x8*>(as + r * 32 * kStride + kk * 16);
+      else bf[fb][r - TM] = *reinterpret_cast<const bf16x8*>(bs + (r - TM) * 32 * kStride + kk * 16);
+    };
+    static_for<kR>([&](auto rc) OCN_LAMBDA_INLINE { read_frag(std::integral_constant<int, 0>{}, rc); });
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<kAll>([&](auto mc) OCN_LAMBDA_INLINE {
+      constexpr int m = decltype(mc)::value, kk = m / kPer, idx = m % kPer, i = idx / TN, j = idx % TN, fb = kk & 1;
+      if constexpr (kk + 1 < kSub) {
+        static_for<(idx + 1) * kR / kPer - idx * kR / kPer>([&](auto rc) OCN_LAMBDA_INLINE {
+          read_frag(std::integral_constant<int, kk + 1>{}, std::integral_constant<int, idx * kR / kPer + decltype(rc)::value>{});
+        });
+      }
+      if constexpr (kLoads && m < kHalf) {
+        static_for<(m + 1) * kL / kHalf - m * kL / kHalf>([&](auto oc) OCN_LAMBDA_INLINE {
+          constexpr int o = m * kL / kHalf + decltype(oc)::value;
+          if constexpr (o < kA) sa[0].template load_op<o>(a_next, lda);
+          else sb[0].template load_op<o - kA>(b_next, ldb);
+        });
+      }
+      if constexpr (kLoads && m >= kHalf) {
+        static_for<(m - kHalf + 1) * kL / kHalf - (m - kHalf) * kL / kHalf>([&](auto oc) OCN_LAMBDA_INLINE {
+          constexpr int o = (m - kHalf) * kL / kHalf + decltype(oc)::value;
+          if constexpr (o < kA) sa[0].template store_op<o>(an);
+          else sb[0].template store_op<o - kA>(bn);
+        });
+      }
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[fb][i], bf[fb][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    __syncthreads();
+  };
+
+  sa[0].init_ops(lda, tid);
+  sb[0].init_ops(ldb, tid);
+  // (fp32 sources stage twice the registers: with double-buffered fragments on top the loop
+  // spills; transposing operands bring enough VALU work that pinning it between the MFMAs of one
+  // wave is slower than letting two waves overlap: both keep the plain loop)
+  constexpr bool kInterleave = kPF == 1 && sizeof(AT) == 2 && sizeof(BT) == 2 && A_KC && B_KC;
+  const bool full_tile = kInterleave && m0 + BM <= g.M && n0 + BN <= g.N && ksteps > 0 && kbeg + ksteps * kBK <= kend;
+  if constexpr (kInterleave) {
+    if (full_tile) {
+      for (long ks = 0; ks + 1 < ksteps; ++ks) fast_step(ks, std::true_type{});
+      fast_step(ksteps - 1, std::false_type{});
+    }
+  }
+  if (!full_tile) {
+    long ks = 0;
+    for (; ks + kPF <= ksteps; ks += kPF) static_for<kPF>([&](auto p) OCN_LAMBDA_INLINE { step(ks + decltype(p)::value, p); });
+    static_for<kPF>([&](auto p) OCN_LAMBDA_INLINE { if (ks + decltype(p)::value < ksteps) step(ks + decltype(p)::value, p); });
+  }
   OCANNL_STAMP(2);
 
   epilogue<TM, TN>(g, acc, m0 + wm0, n0 + wn0, co, lane);

@@ -1025,10 +1025,92 @@ void group_rows(const Routine& r, Plan& plan) {
 
 }  // namespace
 
+// ---- bf16 copies of fp32 contraction operands -----------------------------------------------------
+// A contraction with one fp32 and one bf16 operand runs on the bf16 matrix cores: the fp32
+// operand is rounded to bf16 on the way in.  Doing that rounding once, in a pass of its own into a
+// scratch tensor, gives the same bits, lets every contraction that reads the tensor (a gradient
+// feeds both the input-gradient and the weight-gradient contraction) take the all-bf16 kernel, and
+// halves what they read.
+
+namespace {
+
+bool phase_writes(const Phase& ph, int node) {
+  if (ph.kind == Phase::Fill) return ph.fill_node == node;
+  if (ph.kind == Phase::Contraction) return ph.gemm.c.node == node;
+  auto writes = [&](const Phase& q) {
+    std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+    block_accesses(q.inner, acc, w, f, d);
+    if (w) return true;
+    for (auto& a : acc) if (a.write && a.node == node) return true;
+    return false;
+  };
+  if (!ph.members.empty()) { for (auto& m : ph.members) if (writes(m)) return true; return false; }
+  return writes(ph);
+}
+
+struct Bf16Copies {
+  std::map<int, int> copy_of;       // fp32 node -> its bf16 scratch copy
+  std::map<int, size_t> made_at;    // fp32 node -> plan.phases.size() when the copy was planned
+};
+
+void use_bf16_copies(Routine& r, Plan& plan, Phase& ph, Bf16Copies& copies, int* next_sym) {
+  GemmDesc& g = ph.gemm;
+  if ((g.a.prec == Prec::Single) == (g.b.prec == Prec::Single)) return;   // all-fp32 stays exact fp32
+  GemmOperand& op = g.a.prec == Prec::Single ? g.a : g.b;
+  const Node src = r.node(op.node);
+  int copy = -1;
+  auto it = copies.copy_of.find(src.id);
+  if (it != copies.copy_of.end()) {
+    bool stale = false;
+    for (size_t q = copies.made_at[src.id]; q < plan.phases.size(); ++q) stale |= phase_writes(plan.phases[q], src.id);
+    if (!stale) copy = it->second;
+  }
+  if (copy < 0) {
+    int new_id = 1;
+    for (auto& kv : r.nodes) new_id = std::max(new_id, kv.first + 1);
+    Node t;
+    t.id = new_id;
+    t.ident = "bf" + std::to_string(new_id) + "_" + src.ident;
+    t.prec = Prec::Bfloat16;
+    t.mode = Mode::Local;
+    t.dims = src.dims;
+    Indices ix;
+    std::vector<int> syms;
+    for (size_t p = 0; p < src.dims.size(); ++p) {
+      AxisIndex a; a.kind = AxisIndex::Iter; a.sym = fresh_symbol(r, next_sym);
+      syms.push_back(a.sym); ix.push_back(a);
+    }
+    auto get = std::make_shared<Scalar>();
+    get->kind = Scalar::Get; get->node = src.id; get->idcs = ix;
+    auto set = std::make_shared<Stmt>();
+    set->kind = Stmt::Set; set->node = t.id; set->idcs = ix; set->value = get;
+    StmtP nest = set;
+    for (size_t p = src.dims.size(); p-- > 0;) nest = make_for(syms[p], 0, src.dims[p] - 1, nest);
+    r.nodes.emplace(t.id, t);
+    Phase cv;
+    cv.label = "bf16 copy of " + src.ident;
+    cv.stmt = nest;
+    if (!analyze_nest(r, nest, cv)) { r.nodes.erase(t.id); return; }
+    cv.kind = Phase::Generic;
+    account_bytes(r, cv);
+    plan.phases.push_back(std::move(cv));
+    plan.scratch.push_back(t);
+    copies.copy_of[src.id] = t.id;
+    copies.made_at[src.id] = plan.phases.size();
+    copy = t.id;
+  }
+  op.node = copy;
+  op.prec = Prec::Bfloat16;
+  set_contraction_bytes(ph);
+}
+
+}  // namespace
+
 Plan make_plan(Routine& r, const PlanOptions& opt) {
   Plan plan;
   std::string label;
   int next_sym = 0;
+  Bf16Copies copies;
   Block top = r.body;
   for (size_t ti = 0; ti < top.size(); ++ti) {
     StmtP sp = top[ti];
@@ -1089,6 +1171,7 @@ Plan make_plan(Routine& r, const PlanOptions& opt) {
       account_bytes(r, ph);
     } else {
       set_contraction_bytes(ph);
+      if (opt.enable_bf16_copies) use_bf16_copies(r, plan, ph, copies, &next_sym);
     }
     plan.phases.push_back(std::move(ph));
   }

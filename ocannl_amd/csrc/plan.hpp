@@ -82,6 +82,7 @@ struct PlanOptions {
   bool enable_mfma = true;
   bool enable_coop = true;
   bool enable_row_groups = true;
+  bool enable_bf16_copies = false;  // round fp32 operands of mixed contractions to bf16 once, in scratch (measured: the extra pass costs what the contractions gain)
 };
 
 struct Plan {

@@ -110,6 +110,7 @@ PlanOptions parse_options(const char* options) {
     if (k == "mfma") o.enable_mfma = v != "0";
     else if (k == "coop") o.enable_coop = v != "0";
     else if (k == "rows") o.enable_row_groups = v != "0";
+    else if (k == "bf16_copies") o.enable_bf16_copies = v != "0";
     else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
     else throw InvalidArgument("compile options: unknown key '" + k + "'");
   }
