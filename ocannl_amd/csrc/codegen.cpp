@@ -697,89 +697,119 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     Printer pr(r);
     std::vector<std::string> body;
     const std::string ind = "  ";
-    const int G = ph.coop_lanes;
-    uint64_t P = 1;
 
-    body.push_back(ind + "const uint64_t gtid_ = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;");
-    if (G > 1) {
-      body.push_back(ind + "const uint32_t lane_ = (uint32_t)(gtid_ % " + std::to_string(G) + "u);");
-      body.push_back(ind + "uint64_t pt_ = gtid_ / " + std::to_string(G) + "u;");
-    } else {
-      body.push_back(ind + "uint64_t pt_ = gtid_;");
-    }
-
-    if (!ph.members.empty()) {
-      // ---- row group: a lane group owns one row and runs the member phases in order
-      for (auto e : ph.row_outer_ext) P *= (uint64_t)e;
-      body.push_back(ind + "if (pt_ >= " + std::to_string(P) + "ull) return;");
-      const size_t n = ph.row_outer_ext.size();
-      for (int k = (int)n - 1; k >= 0; --k) {
-        const std::string ext = std::to_string(ph.row_outer_ext[k]) + "ull";
-        std::string line = ind + "const uint32_t row" + std::to_string(k) + "_ = (uint32_t)(";
-        if (k == 0) line += "pt_);";
-        else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
-        body.push_back(line);
+    // one phase for the thread (or loop iteration) identified by gtid_; `skip` leaves it
+    auto emit_points = [&](const Phase& q, const std::string& pind, const std::string& skip) {
+      const int QG = q.coop_lanes;
+      uint64_t QP = 1;
+      if (QG > 1) {
+        body.push_back(pind + "const uint32_t lane_ = (uint32_t)(gtid_ % " + std::to_string(QG) + "u);");
+        body.push_back(pind + "uint64_t pt_ = gtid_ / " + std::to_string(QG) + "u;");
+      } else {
+        body.push_back(pind + "uint64_t pt_ = gtid_;");
       }
-      // short rows: everything the group produces stays in registers as well (no read-back)
-      const bool cached = ph.row_len % G == 0 && ph.row_len / G <= 16;
-      if (cached) {
-        pr.row_iters = (int)(ph.row_len / G);
-        for (auto& m : ph.members) {
-          const Stmt& st = *m.inner[0];
-          if (pr.cache_name.count(st.node)) continue;
-          const Node& wn = r.node(st.node);
-          bool per_position = false;
-          for (auto& ix : st.idcs) if (ix.kind == AxisIndex::Iter && ix.sym == m.row_sym && m.row_role == Phase::RowPointwise) per_position = true;
-          const std::string base = "c" + std::to_string(st.node) + "_";
-          if (per_position) {
-            body.push_back(ind + c_typ(wn.prec) + " " + base + "[" + std::to_string(pr.row_iters) + "];");
-            pr.cache_name[st.node] = base + "[it_]";
-          } else {
-            body.push_back(ind + c_typ(wn.prec) + " " + base + ";");
-            pr.cache_name[st.node] = base;
+      if (!q.members.empty()) {
+        // ---- row group: a lane group owns one row and runs the member phases in order
+        for (auto e : q.row_outer_ext) QP *= (uint64_t)e;
+        body.push_back(pind + "if (pt_ >= " + std::to_string(QP) + "ull) " + skip + ";");
+        const size_t n = q.row_outer_ext.size();
+        for (int k = (int)n - 1; k >= 0; --k) {
+          const std::string ext = std::to_string(q.row_outer_ext[k]) + "ull";
+          std::string line = pind + "const uint32_t row" + std::to_string(k) + "_ = (uint32_t)(";
+          if (k == 0) line += "pt_);";
+          else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
+          body.push_back(line);
+        }
+        // short rows: everything the group produces stays in registers as well (no read-back)
+        const bool cached = q.row_len % QG == 0 && q.row_len / QG <= 16;
+        if (cached) {
+          pr.row_iters = (int)(q.row_len / QG);
+          for (auto& m : q.members) {
+            const Stmt& st = *m.inner[0];
+            if (pr.cache_name.count(st.node)) continue;
+            const Node& wn = r.node(st.node);
+            bool per_position = false;
+            for (auto& ix : st.idcs) if (ix.kind == AxisIndex::Iter && ix.sym == m.row_sym && m.row_role == Phase::RowPointwise) per_position = true;
+            const std::string base = "c" + std::to_string(st.node) + "_";
+            if (per_position) {
+              body.push_back(pind + c_typ(wn.prec) + " " + base + "[" + std::to_string(pr.row_iters) + "];");
+              pr.cache_name[st.node] = base + "[it_]";
+            } else {
+              body.push_back(pind + c_typ(wn.prec) + " " + base + ";");
+              pr.cache_name[st.node] = base;
+            }
           }
         }
-      }
-      for (size_t mi = 0; mi < ph.members.size(); ++mi) {
-        const Phase& m = ph.members[mi];
-        if (mi && !cached) body.push_back(ind + "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\"); "
-                                                "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
-        body.push_back(ind + "{  /* " + m.label + " */");
-        const std::string mi_ind = ind + "  ";
-        for (size_t k = 0; k < m.row_outer_syms.size(); ++k)
-          body.push_back(mi_ind + "const uint32_t " + sym_ident(m.row_outer_syms[k]) + " = row" + std::to_string(k) + "_;");
-        if (m.row_role == Phase::RowPointwise) {
-          body.push_back(pr.row_loop(sym_ident(m.row_sym), 0, ph.row_len - 1, G, mi_ind));
-          emit_phase_statements(r, pr, m, 1, false, mi_ind + "  ", body);
-          body.push_back(mi_ind + "}");
-        } else {
-          emit_phase_statements(r, pr, m, G, true, mi_ind, body);
+        for (size_t mi = 0; mi < q.members.size(); ++mi) {
+          const Phase& m = q.members[mi];
+          if (mi && !cached) body.push_back(pind + "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\"); "
+                                                   "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
+          body.push_back(pind + "{  /* " + m.label + " */");
+          const std::string mi_ind = pind + "  ";
+          for (size_t k = 0; k < m.row_outer_syms.size(); ++k)
+            body.push_back(mi_ind + "const uint32_t " + sym_ident(m.row_outer_syms[k]) + " = row" + std::to_string(k) + "_;");
+          if (m.row_role == Phase::RowPointwise) {
+            body.push_back(pr.row_loop(sym_ident(m.row_sym), 0, q.row_len - 1, QG, mi_ind));
+            emit_phase_statements(r, pr, m, 1, false, mi_ind + "  ", body);
+            body.push_back(mi_ind + "}");
+          } else {
+            emit_phase_statements(r, pr, m, QG, true, mi_ind, body);
+          }
+          body.push_back(pind + "}");
         }
-        body.push_back(ind + "}");
+        pr.row_iters = 0; pr.cache_name.clear(); pr.cache_defined.clear();
+      } else {
+        // --- point decode: the symbol with the smallest stride in the first written array varies
+        //     fastest across adjacent threads (coalesced stores)
+        std::vector<size_t> order = store_order(r, q);
+        for (auto e : q.par_ext) QP *= (uint64_t)e;
+        body.push_back(pind + "if (pt_ >= " + std::to_string(QP) + "ull) " + skip + ";");
+        for (int k = (int)order.size() - 1; k >= 0; --k) {
+          const size_t i = order[k];
+          const std::string sy = sym_ident(q.par_syms[i]);
+          const std::string ext = std::to_string(q.par_ext[i]) + "ull";
+          std::string line = pind + "const uint32_t " + sy + " = (uint32_t)(" + std::to_string(q.par_from[i]) + " + ";
+          if (k == 0) line += "pt_);";
+          else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
+          body.push_back(line);
+        }
+        if (QG > 1 && !q.coop_scope && q.seq_syms.empty()) throw InvalidArgument("planner: lane group without a reduction to share");
+        emit_phase_statements(r, pr, q, QG, false, pind, body);
       }
+      return QP * (uint64_t)QG;
+    };
+
+    uint64_t total_threads = 0;
+    if (!ph.serial_members.empty()) {
+      // ---- the whole routine in one workgroup: phases in order, a barrier after each
+      for (auto& q : ph.serial_members) {
+        body.push_back(ind + "/* " + q.label + " */");
+        if (q.kind == Phase::Fill) {
+          const Node& fn = r.node(q.fill_node);
+          pr.used_nodes.insert(q.fill_node);
+          Pair cv = convert_precision(Prec::Double, fn.prec);
+          body.push_back(ind + "for (uint32_t z_ = threadIdx.x; z_ < " + std::to_string(fn.num_elems()) + "u; z_ += 256u) " +
+                         fn.ident + "[z_] = " + cv.first + "0" + cv.second + ";");
+        } else {
+          uint64_t qt = (uint64_t)q.coop_lanes;
+          for (auto e : (q.members.empty() ? q.par_ext : q.row_outer_ext)) qt *= (uint64_t)e;
+          const uint64_t rounded = (qt + 255) / 256 * 256;
+          body.push_back(ind + "for (uint64_t gtid_ = threadIdx.x; gtid_ < " + std::to_string(rounded) + "ull; gtid_ += 256u) {");
+          emit_points(q, ind + "  ", "continue");
+          body.push_back(ind + "}");
+        }
+        body.push_back(ind + "__syncthreads();");
+      }
+      total_threads = 256;
     } else {
-      // --- thread -> point decode: the symbol with the smallest stride in the first written array
-      //     varies fastest across adjacent threads (coalesced stores)
-      std::vector<size_t> order = store_order(r, ph);
-      for (auto e : ph.par_ext) P *= (uint64_t)e;
-      body.push_back(ind + "if (pt_ >= " + std::to_string(P) + "ull) return;");
-      for (int k = (int)order.size() - 1; k >= 0; --k) {
-        const size_t i = order[k];
-        const std::string s = sym_ident(ph.par_syms[i]);
-        const std::string ext = std::to_string(ph.par_ext[i]) + "ull";
-        std::string line = ind + "const uint32_t " + s + " = (uint32_t)(" + std::to_string(ph.par_from[i]) + " + ";
-        if (k == 0) line += "pt_);";
-        else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
-        body.push_back(line);
-      }
-      if (G > 1 && !ph.coop_scope && ph.seq_syms.empty()) throw InvalidArgument("planner: lane group without a reduction to share");
-      emit_phase_statements(r, pr, ph, G, false, ind, body);
+      body.push_back(ind + "const uint64_t gtid_ = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;");
+      total_threads = emit_points(ph, ind, "return");
     }
 
     GeneratedKernel gk;
     gk.name = r.name + "_k" + std::to_string(kidx++);
     gk.phase_index = (int)pi;
-    gk.threads = P * (uint64_t)G;
+    gk.threads = total_threads;
     gk.block = 256;
     std::vector<std::string> decls;
     for (int id : r.node_order) {

@@ -715,7 +715,8 @@ TileConfig tile_config(const GemmDesc& d) {
   auto clampl = [](long v, long lo, long hi) { return v < lo ? lo : (v > hi ? hi : v); };
   const long s256 = clampl((256 + t256 - 1) / t256, 1, clampl(d.K / 512, 1, 64));
   TileConfig c;
-  if (t256 * s256 >= 192 && d.K / s256 >= 1024) { c.big = true; c.splits = (int)s256; }
+  // (an output narrower than 256 would waste most of a 256-wide tile)
+  if (t256 * s256 >= 192 && d.K / s256 >= 1024 && d.M > 128 && d.N > 128) { c.big = true; c.splits = (int)s256; }
   else { c.big = false; c.splits = (int)clampl((512 + t128 / 2) / t128, 1, clampl(d.K / 512, 1, 64)); }
 #ifdef OCANNL_GEMM_TIMING
   if (g_force_tile) c.big = g_force_tile == 256;

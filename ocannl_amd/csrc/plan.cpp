@@ -993,23 +993,25 @@ void group_rows(const Routine& r, Plan& plan) {
       int lanes = 1;
       while (lanes * 2 <= 64 && lanes * 2 <= shape.len) lanes *= 2;
       g.coop_lanes = lanes;
-      // algorithmic bytes: what the group reads from outside plus everything it writes
-      std::set<int> produced;
+      // algorithmic bytes: every array the group writes, once, plus every array it reads without
+      // having produced it, once; an array indexed by the row position counts rows x T elements,
+      // a per-row one counts rows, anything else (broadcast operands) its own size at most
+      std::set<int> produced, counted_r, counted_w;
       double bytes = 0;
+      auto touched = [&](const Phase& m, const Access& a) {
+        const Node& nd = r.node(a.node);
+        const std::string sig = row_signature(m, *a.idcs);
+        double n = sig.empty() ? (double)nd.num_elems()
+                               : (double)rows * (sig.find('r') != std::string::npos ? (double)shape.len : 1.0);
+        return std::min(n, (double)nd.num_elems()) * prec_in_bytes(nd.prec);
+      };
       for (auto& m : run) {
         std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
         block_accesses(m.inner, acc, w, f, d);
-        std::set<int> reads_inside;
-        for (auto& a : acc) if (!a.write && produced.count(a.node)) reads_inside.insert(a.node);
-        double inside = 0;
-        for (int node : reads_inside) {
-          // the member accounted a full pass over what it reads of this node: take it out again
-          double nelem = (double)rows;
-          for (auto& a : acc) if (!a.write && a.node == node && row_signature(m, *a.idcs).find('r') != std::string::npos) { nelem = (double)rows * (double)shape.len; break; }
-          inside += std::min(nelem, (double)r.node(node).num_elems()) * prec_in_bytes(r.node(node).prec);
-        }
-        bytes += std::max(0.0, m.bytes - inside);
-        for (auto& a : acc) if (a.write) produced.insert(a.node);
+        for (auto& a : acc)
+          if (!a.write && !produced.count(a.node) && counted_r.insert(a.node).second) bytes += touched(m, a);
+        for (auto& a : acc)
+          if (a.write) { produced.insert(a.node); if (counted_w.insert(a.node).second) bytes += touched(m, a); }
       }
       g.bytes = bytes;
       g.members = std::move(run);
@@ -1021,6 +1023,46 @@ void group_rows(const Routine& r, Plan& plan) {
     }
   }
   plan.phases = std::move(out);
+}
+
+}  // namespace
+
+// ---- tiny routines ---------------------------------------------------------------------------------
+namespace {
+
+void serialise_tiny(const Routine& r, Plan& plan) {
+  if (plan.phases.size() < 4) return;
+  double bytes = 0;
+  // the workgroup's 256 threads loop over each phase's points, and with four waves nothing hides
+  // the memory latency of a trip (about a microsecond each, measured): worth it only while the
+  // trips per phase stay below what a launch costs
+  int64_t iterations = 0;
+  for (auto& ph : plan.phases) {
+    if (ph.kind == Phase::Fill) {
+      iterations += r.node(ph.fill_node).num_elems() / 256 + 1;
+    } else if (ph.kind == Phase::Generic && !ph.members.empty()) {
+      int64_t threads = ph.coop_lanes;
+      for (auto e : ph.row_outer_ext) threads *= e;
+      if (threads > 131072) return;
+      iterations += (threads / 256 + 1) * (int64_t)ph.members.size();
+    } else if (ph.kind == Phase::Generic) {
+      int64_t threads = ph.coop_lanes;
+      for (auto e : ph.par_ext) threads *= e;
+      int64_t work = 1;
+      for (size_t i = 0; i < ph.seq_syms.size(); ++i) work *= ph.seq_to[i] - ph.seq_from[i] + 1;
+      if (threads > 131072 || work > 4096) return;
+      iterations += threads / 256 + 1;
+    } else return;
+    bytes += ph.bytes;
+  }
+  if (iterations > 8 * (int64_t)plan.phases.size()) return;
+  Phase g;
+  g.kind = Phase::Generic;
+  g.label = "whole routine, one workgroup";
+  g.bytes = bytes;
+  g.serial_members = std::move(plan.phases);
+  plan.phases.clear();
+  plan.phases.push_back(std::move(g));
 }
 
 }  // namespace
@@ -1176,6 +1218,7 @@ Plan make_plan(Routine& r, const PlanOptions& opt) {
     plan.phases.push_back(std::move(ph));
   }
   if (opt.enable_coop && opt.enable_row_groups) group_rows(r, plan);
+  if (opt.enable_serial_group) serialise_tiny(r, plan);
   return plan;
 }
 

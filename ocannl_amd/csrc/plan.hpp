@@ -69,6 +69,10 @@ struct Phase {
   enum RowRole : uint8_t { RowPointwise, RowReduce, RowScalar } row_role = RowPointwise;   // as a member
   std::vector<int> row_outer_syms;      // as a member: this phase's symbols for the outer axes, slowest first
   int row_sym = -1;                     // as a member: its symbol for the position in the row (-1: none)
+  // Serial group (kind Generic, `serial_members` non-empty): a routine whose phases are all tiny runs
+  // as ONE kernel of a single workgroup that executes the phases in order with a barrier in between
+  // (dozens of launches of a few microseconds each would otherwise be pure launch latency).
+  std::vector<Phase> serial_members;
   // Fill
   int fill_node = -1;
   // Contraction
@@ -82,6 +86,7 @@ struct PlanOptions {
   bool enable_mfma = true;
   bool enable_coop = true;
   bool enable_row_groups = true;
+  bool enable_serial_group = true;   // tiny routines as one single-workgroup kernel
   bool enable_bf16_copies = false;  // round fp32 operands of mixed contractions to bf16 once, in scratch (measured: the extra pass costs what the contractions gain)
 };
 

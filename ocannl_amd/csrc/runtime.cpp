@@ -111,6 +111,7 @@ PlanOptions parse_options(const char* options) {
     else if (k == "coop") o.enable_coop = v != "0";
     else if (k == "rows") o.enable_row_groups = v != "0";
     else if (k == "bf16_copies") o.enable_bf16_copies = v != "0";
+    else if (k == "serial") o.enable_serial_group = v != "0";
     else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
     else throw InvalidArgument("compile options: unknown key '" + k + "'");
   }
