@@ -136,120 +136,89 @@ __device__ __forceinline__ void tile_of_block(long wg, long tiles_m, long tiles_
 }
 
 // ---- staging one operand tile: global -> registers -> LDS --------------------------------------
-// ROWS x kBK tile starting at (row0, k0).  K-contiguous: a thread owns chunks of 8 k at one row.
-// Row-contiguous: a thread owns 8(k) x 8(row) blocks which it transposes in registers on the way to
-// LDS; adjacent lanes take adjacent k-groups of the same rows, so that both the global loads (eight
-// 128-byte row pieces per instruction) and the LDS writes (eight lanes fill one padded row) are
-// conflict-free.
+// ROWS x kBK tile starting at (row0, k0); a thread owns 16-byte chunks (8 elements, converted to
+// bf16 on the way to LDS).
+//   K-contiguous operand:   chunk = 8 k of one row;  LDS holds [row][k], row stride kBK + kPad.
+//   row-contiguous operand: chunk = 8 rows of one k; LDS holds [k][row], row stride ROWS + kPadT --
+//     the tile is NOT transposed on the way in: the MFMA fragments are read with
+//     ds_read_b64_tr_b16, which hands a lane the four k values of its own row (see tr_fragment).
+// Either way global loads and LDS writes are plain 16-byte accesses, adjacent lanes adjacent.
+constexpr int kPadT = 32;   // bf16 elements of padding per k-row of a [k][row] tile: consecutive k
+                            // rows start 64 bytes apart modulo the 256-byte bank cycle
+
+template <int ROWS, bool KC>
+constexpr int lds_tile_elems() { return KC ? ROWS * (kBK + kPad) : kBK * (ROWS + kPadT); }
+
 template <int ROWS, typename T, bool KC>
 struct Stager {
-  static constexpr int kChunks = ROWS * (kBK / 8) / kThreads;        // 8-element chunks per thread
-  static constexpr int kBlocks = (ROWS + kThreads - 1) / kThreads;   // 8x8 blocks per thread
-  Raw8<T> regs[KC ? kChunks : kBlocks * 8];
+  static constexpr int kChunks = ROWS * (kBK / 8) / kThreads;   // chunks per thread
+  static constexpr int kPerLine = KC ? kBK / 8 : ROWS / 8;       // chunks per contiguous line
+  static constexpr int kLineStride = KC ? kBK + kPad : ROWS + kPadT;   // LDS elements per line
+  static constexpr int kLinesPerOp = kThreads / kPerLine;        // lines covered by one op of the workgroup
+  Raw8<T> regs[kChunks];
 
+  // checked version for ragged tiles: `rows` / `K` are the operand's extents
   __device__ __forceinline__ void load(const T* base, long ld, long row0, long k0, long rows, long K, int tid) {
-    if (KC) {
 #pragma unroll
-      for (int j = 0; j < kChunks; ++j) {
-        const int c = tid + kThreads * j;
-        const long row = row0 + c / (kBK / 8);
-        const long k = k0 + (c % (kBK / 8)) * 8;
-        regs[j].zero();
-        if (row < rows && k < K) regs[j].load(base + row * ld + k);
-      }
-    } else {
+    for (int j = 0; j < kChunks; ++j) {
+      const int c = tid + kThreads * j;
+      const long line = c / kPerLine, pos = (c % kPerLine) * 8;
+      regs[j].zero();
+      if (KC) { if (row0 + line < rows && k0 + pos < K) regs[j].load(base + (row0 + line) * ld + k0 + pos); }
+      else    { if (k0 + line < K && row0 + pos < rows) regs[j].load(base + (k0 + line) * ld + row0 + pos); }
+    }
+  }
+
+  __device__ __forceinline__ void store(unsigned short* lds, int tid) const {
 #pragma unroll
-      for (int jb = 0; jb < kBlocks; ++jb) {
-        const int blk = tid + kThreads * jb;
-        const long kg = k0 + (blk % (kBK / 8)) * 8;
-        const long row = row0 + (blk / (kBK / 8)) * 8;
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) {
-          regs[jb * 8 + kk].zero();
-          if (blk < ROWS && row < rows && kg + kk < K) regs[jb * 8 + kk].load(base + (kg + kk) * ld + row);
-        }
-      }
+    for (int j = 0; j < kChunks; ++j) {
+      const int c = tid + kThreads * j;
+      *reinterpret_cast<u32x4*>(lds + (c / kPerLine) * kLineStride + (c % kPerLine) * 8) = regs[j].bf16();
     }
   }
 
   // The same work cut into single instructions for the interleaved main loop of full tiles (no
   // bounds checks): kOps loads, then kOps LDS writes, in matching order.  An address is a part
   // that is uniform over the workgroup (tile origin, op number: scalar registers / immediates) plus
-  // one per-thread 32-bit offset computed once by init_ops().  In the row-contiguous case with
-  // fewer than 256 rows the upper threads repeat the lower threads' blocks (identical values to
-  // identical addresses) instead of branching.
-  static constexpr int kOps = KC ? kChunks : kBlocks * 8;
-  static_assert(KC || kBlocks == 1, "one 8x8 block per thread");
+  // one per-thread 32-bit offset computed once by init_ops().
+  static constexpr int kOps = kChunks;
   unsigned goff, loff;
 
   __device__ __forceinline__ void init_ops(long ld, int tid) {
-    constexpr int kStride = kBK + kPad;
-    if (KC) {
-      goff = (unsigned)((tid / (kBK / 8)) * ld + (tid % (kBK / 8)) * 8);
-      loff = (tid / (kBK / 8)) * kStride + (tid % (kBK / 8)) * 8;
-    } else {
-      const int blk = tid % ROWS;
-      goff = (unsigned)((blk % (kBK / 8)) * 8 * ld + (blk / (kBK / 8)) * 8);
-      loff = (blk / (kBK / 8)) * 8 * kStride + (blk % (kBK / 8)) * 8;
-    }
+    goff = (unsigned)((tid / kPerLine) * ld + (tid % kPerLine) * 8);
+    loff = (tid / kPerLine) * kLineStride + (tid % kPerLine) * 8;
   }
 
-  // `origin` points at the tile's first element (row0, k0): uniform.
+  // `origin` points at the tile's first element: uniform.
   template <int I>
   __device__ __forceinline__ void load_op(const T* origin, long ld) {
-    if (KC) regs[I].load(origin + (long)(I * (kThreads / (kBK / 8))) * ld + goff);
-    else regs[I].load(origin + (long)I * ld + goff);
+    regs[I].load(origin + (long)(I * kLinesPerOp) * ld + goff);
   }
 
   template <int I>
   __device__ __forceinline__ void store_op(unsigned short* lds) const {
-    constexpr int kStride = kBK + kPad;
-    if (KC) {
-      *reinterpret_cast<u32x4*>(lds + loff + I * (kThreads / (kBK / 8)) * kStride) = regs[I].bf16();
-    } else {
-      constexpr int m = I;
-      unsigned w[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const unsigned lo = regs[2 * j].bf16()[m / 2], hi = regs[2 * j + 1].bf16()[m / 2];
-        w[j] = __builtin_amdgcn_perm(hi, lo, (m & 1) ? 0x07060302u : 0x05040100u);
-      }
-      *reinterpret_cast<u32x4*>(lds + loff + m * kStride) = u32x4{w[0], w[1], w[2], w[3]};
-    }
-  }
-
-  __device__ __forceinline__ void store(unsigned short* lds, int tid) const {
-    constexpr int kStride = kBK + kPad;
-    if (KC) {
-#pragma unroll
-      for (int j = 0; j < kChunks; ++j) {
-        const int c = tid + kThreads * j;
-        *reinterpret_cast<u32x4*>(lds + (c / (kBK / 8)) * kStride + (c % (kBK / 8)) * 8) = regs[j].bf16();
-      }
-    } else {
-#pragma unroll
-      for (int jb = 0; jb < kBlocks; ++jb) {
-        const int blk = tid + kThreads * jb;
-        if (blk >= ROWS) break;
-        const int kg = (blk % (kBK / 8)) * 8, row = (blk / (kBK / 8)) * 8;
-        u32x4 in[8];
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) in[kk] = regs[jb * 8 + kk].bf16();
-        // transpose 8x8 of 16-bit: out[m] holds k = 0..7 for row m
-#pragma unroll
-        for (int m = 0; m < 8; ++m) {
-          unsigned w[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const unsigned lo = in[2 * j][m / 2], hi = in[2 * j + 1][m / 2];
-            w[j] = __builtin_amdgcn_perm(hi, lo, (m & 1) ? 0x07060302u : 0x05040100u);   // one 16-bit half of each
-          }
-          *reinterpret_cast<u32x4*>(lds + (row + m) * kStride + kg) = u32x4{w[0], w[1], w[2], w[3]};
-        }
-      }
-    }
+    *reinterpret_cast<u32x4*>(lds + loff + I * kLinesPerOp * kLineStride) = regs[I].bf16();
   }
 };
+
+// MFMA fragment (row = lane % 32 of a 32-row block, k = 8 * (lane / 32) + 0..7 of a 16-k sub-step)
+// out of a [k][row] tile.  ds_read_b64_tr_b16 works on groups of 16 lanes: lane p of a group
+// supplies the address of four consecutive 16-bit words, and receives word p % 4 of the chunks
+// supplied by lanes p / 4, p / 4 + 4, p / 4 + 8, p / 4 + 12.  With lane 4 j + q pointing at
+// (k = j, rows 4 q .. 4 q + 3), lane p gets row p at k = 0..3: its own row, four consecutive k.
+// `tile` points at (k = 0, row = 0) of the 16-k sub-step and the 32-row block.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ unsigned tr_lane_offset(int lane, int line_stride) {
+  const int p = lane & 15;
+  return (unsigned)(((lane >> 5) * 8 + (p >> 2)) * line_stride + ((lane >> 4) & 1) * 16 + (p & 3) * 4);
+}
+__device__ __forceinline__ bf16x8 tr_fragment(const unsigned short* at_lane, int line_stride) {
+  typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(at_lane));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(at_lane + 4 * line_stride));
+  return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
 
 // ---- epilogue -----------------------------------------------------------------------------------
 // One wave's block of TM x TN accumulator tiles -> memory, one row of tiles (32 x TN*32) at a
@@ -342,11 +311,12 @@ template <int BM, int BN, typename AT, typename BT, bool A_KC, bool B_KC>
 __global__ void __launch_bounds__(kThreads)
 __attribute__((amdgpu_waves_per_eu((BM < 256 && sizeof(AT) == 2 && sizeof(BT) == 2) ? 2 : 1, BM >= 256 ? 1 : 2)))
 gemm_bf16_kernel(const GemmArgs g) {
-  constexpr int kStride = kBK + kPad;
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+  constexpr int kAT = lds_tile_elems<BM, A_KC>(), kBT = lds_tile_elems<BN, B_KC>();   // one stage of each operand
+  constexpr int kAS = Stager<BM, AT, A_KC>::kLineStride, kBS = Stager<BN, BT, B_KC>::kLineStride;
   extern __shared__ __align__(16) unsigned short smem[];
   unsigned short* const As0 = smem;
-  unsigned short* const Bs0 = smem + 2 * BM * kStride;
+  unsigned short* const Bs0 = smem + 2 * kAT;
 
   OCANNL_STAMP(0);
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -360,6 +330,19 @@ gemm_bf16_kernel(const GemmArgs g) {
   const AT* A = static_cast<const AT*>(g.a) + ao;
   const BT* B = static_cast<const BT*>(g.b) + bo;
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
+
+  // per-lane offsets of the MFMA fragments inside a stage of each operand
+  const unsigned a_frag = A_KC ? (unsigned)((wm0 + (lane & 31)) * kAS + (lane >> 5) * 8) : (unsigned)wm0 + tr_lane_offset(lane, kAS);
+  const unsigned b_frag = B_KC ? (unsigned)((wn0 + (lane & 31)) * kBS + (lane >> 5) * 8) : (unsigned)wn0 + tr_lane_offset(lane, kBS);
+  // fragment of 32-row block `blk`, 16-k sub-step `kk`, from the stage starting at `stage`
+  auto a_fragment = [&](const unsigned short* stage, int blk, int kk) OCN_LAMBDA_INLINE -> bf16x8 {
+    if constexpr (A_KC) return *reinterpret_cast<const bf16x8*>(stage + a_frag + blk * 32 * kAS + kk * 16);
+    else return tr_fragment(stage + a_frag + kk * 16 * kAS + blk * 32, kAS);
+  };
+  auto b_fragment = [&](const unsigned short* stage, int blk, int kk) OCN_LAMBDA_INLINE -> bf16x8 {
+    if constexpr (B_KC) return *reinterpret_cast<const bf16x8*>(stage + b_frag + blk * 32 * kBS + kk * 16);
+    else return tr_fragment(stage + b_frag + kk * 16 * kBS + blk * 32, kBS);
+  };
 
   f32x16 acc[TM][TN];
   static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
@@ -403,8 +386,8 @@ gemm_bf16_kernel(const GemmArgs g) {
       sb[par].load(B, ldb, n0, kbeg + (ks + kPF) * kBK, g.N, kend, tid);
     }
     __builtin_amdgcn_sched_barrier(0);   // the loads are issued before the MFMA block, not sunk below it
-    const unsigned short* as = As0 + cur * BM * kStride + (wm0 + (lane & 31)) * kStride + (lane >> 5) * 8;
-    const unsigned short* bs = Bs0 + cur * BN * kStride + (wn0 + (lane & 31)) * kStride + (lane >> 5) * 8;
+    const unsigned short* as = As0 + cur * kAT;
+    const unsigned short* bs = Bs0 + cur * kBT;
     // fragments are double buffered: the LDS reads of sub-step kk + 1 are issued before the MFMAs
     // of sub-step kk, so that a lone wave per SIMD does not sit out the LDS latency every time
     bf16x8 af[2][TM], bf[2][TN];
@@ -412,11 +395,11 @@ gemm_bf16_kernel(const GemmArgs g) {
       constexpr int kk = decltype(kkc)::value, fb = kk & 1;
       static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
         constexpr int i = decltype(ic)::value;
-        af[fb][i] = *reinterpret_cast<const bf16x8*>(as + i * 32 * kStride + kk * 16);
+        af[fb][i] = a_fragment(as, i, kk);
       });
       static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
         constexpr int j = decltype(jc)::value;
-        bf[fb][j] = *reinterpret_cast<const bf16x8*>(bs + j * 32 * kStride + kk * 16);
+        bf[fb][j] = b_fragment(bs, j, kk);
       });
     };
     read_frags(std::integral_constant<int, 0>{});
@@ -437,8 +420,8 @@ gemm_bf16_kernel(const GemmArgs g) {
     // tile ks + 1 sits in the other register set (or, with one set, in the one just refilled)
     if (ks + 1 < ksteps && !OCANNL_PROBE_SKIP(1)) {
       constexpr int nxt = (par + 1) % kPF;
-      sa[nxt].store(As0 + (cur ^ 1) * BM * kStride, tid);
-      sb[nxt].store(Bs0 + (cur ^ 1) * BN * kStride, tid);
+      sa[nxt].store(As0 + (cur ^ 1) * kAT, tid);
+      sb[nxt].store(Bs0 + (cur ^ 1) * kBT, tid);
     }
     __syncthreads();
   };
@@ -455,15 +438,15 @@ gemm_bf16_kernel(const GemmArgs g) {
     const long kn = kbeg + (ks + 1) * kBK;
     const AT* const a_next = A_KC ? A + m0 * lda + kn : A + kn * lda + m0;
     const BT* const b_next = B_KC ? B + n0 * ldb + kn : B + kn * ldb + n0;
-    unsigned short* const an = As0 + (cur ^ 1) * BM * kStride;
-    unsigned short* const bn = Bs0 + (cur ^ 1) * BN * kStride;
-    const unsigned short* as = As0 + cur * BM * kStride + (wm0 + (lane & 31)) * kStride + (lane >> 5) * 8;
-    const unsigned short* bs = Bs0 + cur * BN * kStride + (wn0 + (lane & 31)) * kStride + (lane >> 5) * 8;
+    unsigned short* const an = As0 + (cur ^ 1) * kAT;
+    unsigned short* const bn = Bs0 + (cur ^ 1) * kBT;
+    const unsigned short* as = As0 + cur * kAT;
+    const unsigned short* bs = Bs0 + cur * kBT;
     bf16x8 af[2][TM], bf[2][TN];
     auto read_frag = [&](auto kkc, auto rc) OCN_LAMBDA_INLINE {
       constexpr int kk = decltype(kkc)::value, r = decltype(rc)::value, fb = kk & 1;
-      if constexpr (r < TM) af[fb][r] = *reinterpret_cast<const bf16x8*>(as + r * 32 * kStride + kk * 16);
-      else bf[fb][r - TM] = *reinterpret_cast<const bf16x8*>(bs + (r - TM) * 32 * kStride + kk * 16);
+      if constexpr (r < TM) af[fb][r] = a_fragment(as, r, kk);
+      else bf[fb][r - TM] = b_fragment(bs, r - TM, kk);
     };
     static_for<kR>([&](auto rc) OCN_LAMBDA_INLINE { read_frag(std::integral_constant<int, 0>{}, rc); });
     __builtin_amdgcn_sched_barrier(0);
@@ -497,9 +480,8 @@ gemm_bf16_kernel(const GemmArgs g) {
   sa[0].init_ops(lda, tid);
   sb[0].init_ops(ldb, tid);
   // (fp32 sources stage twice the registers: with double-buffered fragments on top the loop
-  // spills; transposing operands bring enough VALU work that pinning it between the MFMAs of one
-  // wave is slower than letting two waves overlap: both keep the plain loop)
-  constexpr bool kInterleave = kPF == 1 && sizeof(AT) == 2 && sizeof(BT) == 2 && A_KC && B_KC;
+  // spills, so they keep the plain loop)
+  constexpr bool kInterleave = kPF == 1 && sizeof(AT) == 2 && sizeof(BT) == 2;
   const bool full_tile = kInterleave && m0 + BM <= g.M && n0 + BN <= g.N && ksteps > 0 && kbeg + ksteps * kBK <= kend;
   if constexpr (kInterleave) {
     if (full_tile) {
@@ -659,8 +641,8 @@ gemm_f32_kernel(const GemmArgs g) {
   epilogue<TM, TN>(g, acc, m0 + wm0, n0 + wn0, co, lane);
 }
 
-template <int BM, int BN>
-constexpr size_t bf16_smem() { return 2ull * (BM + BN) * (kBK + kPad) * sizeof(unsigned short); }
+template <int BM, int BN, bool A_KC, bool B_KC>
+constexpr size_t bf16_smem() { return 2ull * (lds_tile_elems<BM, A_KC>() + lds_tile_elems<BN, B_KC>()) * sizeof(unsigned short); }
 template <int BM, int BN>
 constexpr size_t f32_smem() { return 2ull * (BM + BN) * (kBKf + kPadf) * sizeof(float); }
 
@@ -755,11 +737,10 @@ hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t
 
 template <int BM, int BN, typename AT, typename BT>
 hipError_t launch_bf16_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t s, hipEvent_t ev) {
-  constexpr size_t sm = bf16_smem<BM, BN>();
-  if (akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, true>, sm, BM, BN, a, s, ev);
-  if (akc && !bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, false>, sm, BM, BN, a, s, ev);
-  if (!akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, true>, sm, BM, BN, a, s, ev);
-  return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, false>, sm, BM, BN, a, s, ev);
+  if (akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, true>, bf16_smem<BM, BN, true, true>(), BM, BN, a, s, ev);
+  if (akc && !bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, false>, bf16_smem<BM, BN, true, false>(), BM, BN, a, s, ev);
+  if (!akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, true>, bf16_smem<BM, BN, false, true>(), BM, BN, a, s, ev);
+  return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, false>, bf16_smem<BM, BN, false, false>(), BM, BN, a, s, ev);
 }
 
 template <int BM, int BN>
