@@ -300,11 +300,27 @@ struct Printer {
   std::map<int, std::string> cache_name;    // node -> register expression
   std::set<int> cache_defined;              // nodes whose cache holds the current value
   // `lhs = value;` with the cache kept in step
+  const std::map<int, int>* mirrors = nullptr;   // fp32 node -> bf16 copy stored alongside (Plan::mirrors)
   std::string store_line(int node, const std::string& lhs, const std::string& value, const std::string& guard) {
+    std::string mirror_lhs;
+    if (mirrors) {
+      auto m = mirrors->find(node);
+      if (m != mirrors->end()) {
+        used_nodes.insert(m->second);
+        mirror_lhs = r.node(m->second).ident + lhs.substr(lhs.find('['));   // same dims: same offset
+      }
+    }
     auto it = cache_name.find(node);
-    if (it == cache_name.end()) return guard + lhs + " = " + value + ";";
+    if (it == cache_name.end()) {
+      if (mirror_lhs.empty()) return guard + lhs + " = " + value + ";";
+      const std::string t = "m" + std::to_string(fresh++) + "_";
+      return "{ const " + std::string(c_typ(r.node(node).prec)) + " " + t + " = " + value + "; " + guard + "{ " + lhs + " = " + t +
+             "; " + mirror_lhs + " = single_to_bfloat16(" + t + "); } }";
+    }
     cache_defined.insert(node);
-    return it->second + " = " + value + "; " + guard + lhs + " = " + it->second + ";";
+    std::string line = it->second + " = " + value + "; " + guard + "{ " + lhs + " = " + it->second + ";";
+    if (!mirror_lhs.empty()) line += " " + mirror_lhs + " = single_to_bfloat16(" + it->second + ");";
+    return line + " }";
   }
   // header of a loop over the row position shared by `lanes` lanes
   std::string row_loop(const std::string& sym, int64_t from, int64_t to, int lanes, const std::string& ind) {
@@ -695,6 +711,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     const Phase& ph = plan.phases[pi];
     if (ph.kind != Phase::Generic) continue;
     Printer pr(r);
+    pr.mirrors = &plan.mirrors;
     std::vector<std::string> body;
     const std::string ind = "  ";
 

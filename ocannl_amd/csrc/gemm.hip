@@ -683,23 +683,27 @@ long batch_count(const GemmDesc& d) {
 int g_force_tile = 0, g_force_splits = 0;   // tuning overrides of the probe build
 #endif
 
-// Tile size and split-K factor.  Measured on MI355X: the 256x256 tile (one workgroup per CU) pays
-// off only when every workgroup runs at least ~16 K stages and the launch still has >= 192
-// workgroups, K being split to get there (weight-gradient shapes: small output, K = all rows);
-// otherwise 128x128 tiles, two workgroups per CU, split towards ~512 workgroups.  A split never
-// gets fewer than 8 K stages.  Splits are summed in index order by splitk_reduce_kernel.
+// Tile size and split-K factor, from a measured sweep on MI355X (bf16 operands).  256x256 tiles
+// (one workgroup per CU) win only when the output alone gives >= 256 of them; anything smaller
+// runs 128x128 tiles, two workgroups per CU, and when those are fewer than 256 K is split
+// towards ~512 workgroups, never below 8 K stages per split.  Splits are summed in index order by
+// splitk_reduce_kernel (deterministic).
 struct TileConfig { bool big; int splits; };
 
 TileConfig tile_config(const GemmDesc& d) {
   const long nb = batch_count(d);
   const long t256 = ((d.M + 255) / 256) * ((d.N + 255) / 256) * nb;
   const long t128 = ((d.M + 127) / 128) * ((d.N + 127) / 128) * nb;
-  auto clampl = [](long v, long lo, long hi) { return v < lo ? lo : (v > hi ? hi : v); };
-  const long s256 = clampl((256 + t256 - 1) / t256, 1, clampl(d.K / 512, 1, 64));
   TileConfig c;
-  // (an output narrower than 256 would waste most of a 256-wide tile)
-  if (t256 * s256 >= 192 && d.K / s256 >= 1024 && d.M > 128 && d.N > 128) { c.big = true; c.splits = (int)s256; }
-  else { c.big = false; c.splits = (int)clampl((512 + t128 / 2) / t128, 1, clampl(d.K / 512, 1, 64)); }
+  if (t256 >= 256 && d.M > 128 && d.N > 128) { c.big = true; c.splits = 1; }
+  else {
+    c.big = false;
+    long s = 1;
+    if (t128 < 256) {
+      while (s * 2 * t128 <= 512 && s * 2 <= d.K / 512 && s < 64) s *= 2;
+    }
+    c.splits = (int)s;
+  }
 #ifdef OCANNL_GEMM_TIMING
   if (g_force_tile) c.big = g_force_tile == 256;
   if (g_force_splits) c.splits = g_force_splits;

@@ -1090,6 +1090,25 @@ bool phase_writes(const Phase& ph, int node) {
   return writes(ph);
 }
 
+// Does the generated phase store to every element of `node`?  (Every axis of its store is a
+// full-range parallel iterator or has extent 1.)
+bool writes_whole_node(const Routine& r, const Phase& ph, int node) {
+  if (ph.inner.size() != 1 || ph.inner[0]->kind != Stmt::Set || ph.inner[0]->node != node) return false;
+  const Stmt& set = *ph.inner[0];
+  const Node& n = r.node(node);
+  for (size_t p = 0; p < set.idcs.size(); ++p) {
+    const AxisIndex& a = set.idcs[p];
+    if (a.kind == AxisIndex::Fixed) { if (n.dims[p] != 1) return false; }
+    else if (a.kind == AxisIndex::Iter) {
+      bool ok = false;
+      for (size_t i = 0; i < ph.par_syms.size(); ++i)
+        if (ph.par_syms[i] == a.sym) ok = ph.par_from[i] == 0 && ph.par_ext[i] == n.dims[p];
+      if (!ok) return false;
+    } else return false;
+  }
+  return true;
+}
+
 struct Bf16Copies {
   std::map<int, int> copy_of;       // fp32 node -> its bf16 scratch copy
   std::map<int, size_t> made_at;    // fp32 node -> plan.phases.size() when the copy was planned
@@ -1108,6 +1127,27 @@ void use_bf16_copies(Routine& r, Plan& plan, Phase& ph, Bf16Copies& copies, int*
     if (!stale) copy = it->second;
   }
   if (copy < 0) {
+    auto m = plan.mirrors.find(src.id);
+    if (m != plan.mirrors.end()) copy = m->second;
+  }
+  // Can the kernels that produce the tensor keep the copy themselves?  Yes when everything that
+  // writes it in this routine is a generated kernel (or a zero fill), and some writer covers the
+  // whole tensor before this contraction reads it.
+  bool mirror = false;
+  std::vector<size_t> fills;
+  if (copy < 0) {
+    bool all_generated = true, whole = false, any = false;
+    for (size_t q = 0; q < plan.phases.size(); ++q) {
+      const Phase& w = plan.phases[q];
+      if (!phase_writes(w, src.id)) continue;
+      any = true;
+      if (w.kind == Phase::Fill) { fills.push_back(q); whole = true; }
+      else if (w.kind == Phase::Generic && w.members.empty() && w.serial_members.empty()) whole |= writes_whole_node(r, w, src.id);
+      else all_generated = false;
+    }
+    mirror = any && all_generated && whole && src.mode != Mode::Virtual && !src.read_only;
+  }
+  if (copy < 0) {
     int new_id = 1;
     for (auto& kv : r.nodes) new_id = std::max(new_id, kv.first + 1);
     Node t;
@@ -1116,6 +1156,22 @@ void use_bf16_copies(Routine& r, Plan& plan, Phase& ph, Bf16Copies& copies, int*
     t.prec = Prec::Bfloat16;
     t.mode = Mode::Local;
     t.dims = src.dims;
+    if (mirror) {
+      r.nodes.emplace(t.id, t);
+      plan.scratch.push_back(t);
+      plan.mirrors[src.id] = t.id;
+      // a remaining zero fill of the tensor zeroes the copy too (bf16 zero is all-zero bits)
+      for (size_t k = fills.size(); k-- > 0;) {
+        Phase f;
+        f.kind = Phase::Fill; f.label = "zero bf16 copy of " + src.ident; f.fill_node = t.id;
+        f.bytes = (double)t.size_in_bytes();
+        plan.phases.insert(plan.phases.begin() + fills[k] + 1, std::move(f));
+      }
+      op.node = t.id;
+      op.prec = Prec::Bfloat16;
+      set_contraction_bytes(ph);
+      return;
+    }
     Indices ix;
     std::vector<int> syms;
     for (size_t p = 0; p < src.dims.size(); ++p) {

@@ -10,6 +10,7 @@
 //   * Generic      -- anything else: a generated kernel with one thread (or one cooperating lane
 //                     group) per point of the nest's parallel index space.
 #pragma once
+#include <map>
 #include <string>
 #include <vector>
 
@@ -87,12 +88,15 @@ struct PlanOptions {
   bool enable_coop = true;
   bool enable_row_groups = true;
   bool enable_serial_group = true;   // tiny routines as one single-workgroup kernel
-  bool enable_bf16_copies = false;  // round fp32 operands of mixed contractions to bf16 once, in scratch (measured: the extra pass costs what the contractions gain)
+  bool enable_bf16_copies = true;   // keep bf16 copies of fp32 operands of mixed contractions (written by the producing kernels)
 };
 
 struct Plan {
   std::vector<Phase> phases;
   std::vector<Node> scratch;   // nodes invented by the planner (de-virtualised contraction results)
+  // fp32 node -> bf16 scratch copy kept in step by every generated store to the node (a store to
+  // the node also stores the rounded value to the copy): the copy feeds bf16 contractions
+  std::map<int, int> mirrors;
 };
 
 Plan make_plan(Routine& r, const PlanOptions& opt);
