@@ -1,0 +1,116 @@
+"""GPU parity of the planner's kernel-fusing rewrites at sizes where they switch on: row groups
+(register-cached and fenced), split column reductions, lane-cooperative scalar reductions, bf16
+operand copies kept by the producing kernels, the single-workgroup kernel for tiny routines."""
+import re
+
+import numpy as np
+import pytest
+
+from ocannl_amd import backend as B
+from ocannl_amd import llir as L
+from ocannl_amd import workloads as W
+from parity import HipRun, OracleRun, rel_err
+from test_gpu_models import _err, _widened_init
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("prec,tol", [("single", 1e-4), ("bfloat16", 2e-2)])
+def test_transformer_with_row_groups_and_operand_copies(prec, tol):
+    # seq 128: soft-max rows of 128 (2 per lane: kept in registers); vocab 2048: rows of 2048 (32 per
+    # lane: through memory with fences); bf16 values with fp32 gradients: mirrored bf16 copies
+    kw = dict(batch=4, seq=128, d_model=128, heads=2, d_ff=256, layers=1, vocab=2048, grad_prec="single", lr=0.05)
+    w = W.transformer(prec=prec, **kw)
+    wr = W.transformer(prec="single", **kw)
+    hip = HipRun(w.routine, w.init)
+    src = hip.code.source()
+    assert "row0_" in src and "it_" in src and "__builtin_amdgcn_fence" in src
+    if prec == "bfloat16":
+        assert re.search(r"bf\d+_\w+\[[^\]]*\] = single_to_bfloat16\(", src)
+    n_default = len(hip.code.kernels())
+    n_plain = len(B.compile(w.routine, "rows=0;bf16_copies=0").kernels())
+    assert n_default < n_plain
+    ora = OracleRun(wr.routine, _widened_init(w, wr))
+    for _ in range(2):
+        hip.step(); ora.step()
+        lh = float(W.to_float(hip.get(w.nodes["loss"]), w.nodes["loss"].prec)[0]); lo = float(ora.get(wr.nodes["loss"])[0])
+        assert abs(lh - lo) <= tol * max(abs(lo), 1.0), (lh, lo)
+    for name in ("w_embed", "w_q_l0", "w_ffn2_l0", "w_out", "gamma_ln1_l0", "beta_ln2_l0", "pos_encoding"):
+        assert _err(W.to_float(hip.get(w.nodes[name]), prec), ora.get(wr.nodes[name]), prec) <= tol, name
+    hip.close()
+
+
+def test_row_groups_equal_separate_kernels_bit_for_bit():
+    # fusing phases into row groups changes where values live, not what is computed
+    kw = dict(batch=4, seq=128, d_model=128, heads=2, d_ff=256, layers=1, vocab=512, prec="single", grad_prec="single")
+    w = W.transformer(**kw)
+    a, b = HipRun(w.routine, w.init), HipRun(w.routine, w.init, "rows=0")
+    assert len(a.code.kernels()) < len(b.code.kernels())
+    a.step(); b.step()
+    for name in ("loss", "w_q_l0", "w_out", "gamma_ln1_l0"):
+        assert np.array_equal(a.get(w.nodes[name]), b.get(w.nodes[name])), name
+    a.close(); b.close()
+
+
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_split_column_reduction(accumulate):
+    # out[j] (+)= sum_i x[i, j] * y[i, j]: small output, reduction over the slow axis
+    rows, cols = 4096, 256
+    L.reset_symbols(0)
+    x = L.Node(1, "x", "single", (rows, cols)); y = L.Node(2, "y", "single", (rows, cols))
+    out = L.Node(3, "out", "single", (cols,))
+    j, i = L.fresh_symbol(), L.fresh_symbol()
+    body = [] if accumulate else [L.ZeroOut(out)]
+    body.append(L.For(j, 0, cols - 1, [L.For(i, 0, rows - 1, [
+        L.Set(out, (L.It(j),), L.Ternop("fma", L.Get(x, (L.It(i), L.It(j))), L.Get(y, (L.It(i), L.It(j))),
+                                         L.Get(out, (L.It(j),))))])]))
+    r = L.Routine("colsum", body)
+    rng = np.random.default_rng(3)
+    init = {1: rng.standard_normal((rows, cols)).astype(np.float32), 2: rng.standard_normal((rows, cols)).astype(np.float32),
+            3: rng.standard_normal(cols).astype(np.float32)}
+    hip, ora = HipRun(r, init), OracleRun(r, init)
+    src = hip.code.source()
+    assert re.search(r"part\d+_out", src), "the reduction was not split"
+    assert len(hip.code.kernels()) == 2
+    hip.step(); ora.step()
+    assert rel_err(hip.get(out), ora.get(out), "single") <= 1e-4
+    # the unsplit, sequential version is bit-identical to the checker
+    seq = HipRun(r, init, "coop=0")
+    seq.step()
+    assert np.array_equal(seq.get(out), ora.get(out))
+    hip.close(); seq.close()
+
+
+def test_scalar_reduction_shared_by_lanes():
+    # loss = (sum_i -log p[i]) / n written as an inlined scalar reduction inside one statement
+    n = 8192
+    L.reset_symbols(0)
+    p = L.Node(1, "p", "single", (n,)); loss = L.Node(2, "loss", "single", (1,))
+    acc = L.Node(3, "acc", "single", (1,), mode="virtual")
+    i = L.fresh_symbol()
+    sc = L.Scope(acc, 1)
+    scope = L.LocalScope(sc, [
+        L.SetLocal(sc, L.Const(0.0)),
+        L.For(i, 0, n - 1, [L.SetLocal(sc, L.Binop("add", L.GetLocal(sc), L.Unop("neg", L.Unop("log", L.Get(p, (L.It(i),))))))])])
+    r = L.Routine("nll", [L.Set(loss, (L.Fixed(0),), L.Binop("div", scope, L.Const(float(n))))])
+    init = {1: np.random.default_rng(5).uniform(0.05, 1.0, n).astype(np.float32)}
+    hip, ora = HipRun(r, init), OracleRun(r, init)
+    assert "ocn_xshfl" in hip.code.source()
+    hip.step(); ora.step()
+    assert rel_err(hip.get(loss), ora.get(loss), "single") <= 1e-4
+    hip.close()
+
+
+def test_tiny_routine_is_one_workgroup_with_identical_results():
+    w = W.moons_mlp()
+    sym = w.statics["batch_n"].sym
+    one, many = HipRun(w.routine, w.init, "coop=0"), HipRun(w.routine, w.init, "coop=0;serial=0")
+    assert len(one.code.kernels()) == 1 and len(many.code.kernels()) > 10
+    ora = OracleRun(w.routine, w.init)
+    for step in range(10):
+        st = {sym: step}
+        one.step(st); many.step(st); ora.step(st)
+    for name in ("w1", "w2", "w3", "b1"):
+        assert np.array_equal(one.get(w.nodes[name]), many.get(w.nodes[name])), name
+        assert rel_err(one.get(w.nodes[name]), ora.get(w.nodes[name]), "single") <= 1e-5, name
+    one.close(); many.close()
