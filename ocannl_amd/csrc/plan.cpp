@@ -1204,11 +1204,79 @@ void use_bf16_copies(Routine& r, Plan& plan, Phase& ph, Bf16Copies& copies, int*
 
 }  // namespace
 
+// ---- scalar locals at routine scope ------------------------------------------------------------
+// `Declare_local` / `Set_local` outside any `Local_scope` (low_level.mli:22-51) declare a scalar
+// that lives across top-level statements.  The serial C code keeps it in a variable; here the
+// statements become different kernels, so the scalar gets a one-element scratch tensor: the
+// declaration disappears (a zero fill if it asked for initialisation), `Set_local` becomes a store
+// and every read of the scalar a load.
+namespace {
+
+void lift_routine_locals(Routine& r, Plan& plan) {
+  std::map<ScopeId, int> lifted;
+  for (auto& sp : r.body)
+    if (sp->kind == Stmt::DeclareLocal) lifted[sp->scope] = -1;
+  if (lifted.empty()) return;
+  int new_id = 1;
+  for (auto& kv : r.nodes) new_id = std::max(new_id, kv.first + 1);
+  for (auto& kv : lifted) {
+    Node t;
+    t.id = new_id++;
+    t.ident = "v" + std::to_string(kv.first.scope) + "_" + r.node(kv.first.node).ident;
+    t.prec = r.node(kv.first.node).prec;
+    t.mode = Mode::Local;
+    t.dims = {1};
+    r.nodes.emplace(t.id, t);
+    plan.scratch.push_back(t);
+    kv.second = t.id;
+  }
+  Indices zero(1);
+  zero[0].kind = AxisIndex::Fixed; zero[0].fixed = 0;
+  std::function<ScalarP(const ScalarP&)> sc;
+  std::function<Block(const Block&)> blk;
+  sc = [&](const ScalarP& s) -> ScalarP {
+    if (!s) return s;
+    if (s->kind == Scalar::GetLocal) {
+      auto it = lifted.find(s->scope);
+      if (it == lifted.end()) return s;
+      auto g = std::make_shared<Scalar>();
+      g->kind = Scalar::Get; g->node = it->second; g->idcs = zero;
+      return g;
+    }
+    auto o = std::make_shared<Scalar>(*s);
+    if (s->kind == Scalar::LocalScope) o->body = blk(s->body);
+    o->a = sc(s->a); o->b = sc(s->b); o->c = sc(s->c);
+    return o;
+  };
+  blk = [&](const Block& b) -> Block {
+    Block out;
+    for (auto& sp : b) {
+      auto o = std::make_shared<Stmt>(*sp);
+      if (sp->kind == Stmt::For) o->body = blk(sp->body);
+      if (sp->value) o->value = sc(sp->value);
+      if (sp->kind == Stmt::SetLocal) {
+        auto it = lifted.find(sp->scope);
+        if (it != lifted.end()) { o->kind = Stmt::Set; o->node = it->second; o->idcs = zero; }
+      }
+      if (sp->kind == Stmt::DeclareLocal && lifted.count(sp->scope)) {
+        if (!sp->needs_init) continue;
+        o->kind = Stmt::ZeroOut; o->node = lifted.at(sp->scope);
+      }
+      out.push_back(o);
+    }
+    return out;
+  };
+  r.body = blk(r.body);
+}
+
+}  // namespace
+
 Plan make_plan(Routine& r, const PlanOptions& opt) {
   Plan plan;
   std::string label;
   int next_sym = 0;
   Bf16Copies copies;
+  lift_routine_locals(r, plan);
   Block top = r.body;
   for (size_t ti = 0; ti < top.size(); ++ti) {
     StmtP sp = top[ti];
@@ -1226,7 +1294,7 @@ Plan make_plan(Routine& r, const PlanOptions& opt) {
       continue;
     }
     if (sp->kind == Stmt::DeclareLocal || sp->kind == Stmt::SetLocal)
-      throw InvalidArgument("hip backend: scalar locals at routine scope are not supported (routine " + r.name + ")");
+      throw InvalidArgument("hip backend: Set_local of an undeclared scalar at routine scope (routine " + r.name + ")");
     const size_t before = plan.phases.size();
     devirtualise(r, sp, opt, plan, label);
     const bool devirt = plan.phases.size() != before;

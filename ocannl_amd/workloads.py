@@ -193,7 +193,6 @@ def char_mlp(batch: int = 32, vocab: int = 27, context: int = 3, embed: int = 10
     """test/training/mlp_names.ml:145-168 with synthetic tokens: ids -> embedding gather ->
     ``tanh(emb +* w1 + b1)`` -> logits -> stable log-softmax cross entropy; Adam update.  A fresh
     batch is a slice of a resident id/target set selected by the static index ``batch_n``."""
-    from .frontend import gather_rows
     L.reset_symbols(0)
     g = Graph("single", "single")
     batch_n = L.StaticSymbol(L.fresh_symbol(), n_batches)
@@ -207,11 +206,8 @@ def char_mlp(batch: int = 32, vocab: int = 27, context: int = 3, embed: int = 10
     c = g.param("c", ("e", "v"), (embed, vocab))
     w1 = g.param("w1", ("h", "s", "e"), (hidden, context, embed)); b1 = g.param("b1", ("h",), (hidden,))
     w2 = g.param("w2", ("v", "h"), (vocab, hidden)); b2 = g.param("b2", ("v",), (vocab,))
-    # the gather reads the id through the slice
-    ids_view = T(ids_all.value, ("b", "s"), None)
-    ids_view._getter = ids._getter
-    ids_view._dims = (batch, context)
-    emb = _gather_slice(g, c, ids, "v", batch, context)
+    # the gather reads the ids through the slice's getter
+    emb = _gather_rows_with_getter(g, c, ids, (batch, context), "v")
     hid = g.unary("tanh", g.add(g.einsum(emb, w1, ("b", "h"), ident="emb_w1"), b1, ("b", "h")), ident="hidden")
     logits = g.add(g.einsum(w2, hid, ("b", "v"), ident="w2h"), b2, ("b", "v"), ident="logits")
     max_l = g.reduce(logits, ("b",), accum="max", ident="max_l")
@@ -239,17 +235,6 @@ def char_mlp(batch: int = 32, vocab: int = 27, context: int = 3, embed: int = 10
         nodes["v_" + p.label] = p.adam_v
     return Workload("char_mlp", routine, init, nodes, {"batch_n": batch_n}, [loss.value],
                     f"char MLP LM vocab {vocab} ctx {context} emb {embed} hid {hidden} batch {batch}, Adam lr {lr}")
-
-
-def _gather_slice(g, table, ids_slice, table_axis, batch, context):
-    from .frontend import gather_rows
-    # gather_rows reads ids through `ids.value` with its axes; give it a view whose element read
-    # goes through the slice getter
-    class _IdsView:
-        pass
-    view = T(ids_slice.value, ids_slice.axes, None)
-    view._getter = ids_slice._getter
-    return _gather_rows_with_getter(g, table, view, (batch, context), table_axis)
 
 
 def _gather_rows_with_getter(g, table, ids, ids_dims, table_axis, ident="embed"):

@@ -174,3 +174,27 @@ def test_single_to_bfloat16_bit_exact_on_all_float_classes():
     bad = np.nonzero(got != want)[0]
     assert bad.size == 0, [(hex(bits[k]), hex(got[k]), hex(want[k])) for k in bad[:8]]
     hip.close()
+
+
+def test_routine_scope_scalar_locals():
+    # arrayjit/test/test_local_scope_init.expected, cases 5 and 6: a Declare_local hoisted to routine
+    # scope is written by one statement and read by later ones (kernels of their own here)
+    L.reset_symbols(10)
+    z = (L.Fixed(0),)
+    s3 = L.Node(9, "src3", "single", (1,)); o3 = L.Node(10, "out3", "single", (1,)); o4 = L.Node(11, "out4", "single", (1,))
+    s4 = L.Node(12, "src4", "single", (4,)); o5 = L.Node(13, "out5", "single", (1,)); o6 = L.Node(14, "out6", "single", (1,))
+    a, b = L.Scope(s3, 30), L.Scope(s4, 40)
+    body = [L.DeclareLocal(a, False), L.SetLocal(a, L.Get(s3, z)),
+            L.Set(o3, z, L.GetLocal(a)), L.Set(o4, z, L.Binop("mul", L.GetLocal(a), L.Const(2.0))),
+            L.DeclareLocal(b, True),
+            L.For(4, 0, 3, [L.SetLocal(b, L.Binop("add", L.GetLocal(b), L.Get(s4, (L.It(4),))))]),
+            L.Set(o5, z, L.GetLocal(b)), L.Set(o6, z, L.Binop("add", L.GetLocal(b), L.GetLocal(a)))]
+    r = L.Routine("hoisted_locals", body)
+    init = {9: np.array([1.5], np.float32), 12: np.array([1, 2, 3, 4.25], np.float32)}
+    for opts in (None, "serial=0"):
+        hip, ora = HipRun(r, init, opts), OracleRun(r, init)
+        hip.step(); ora.step()
+        for n in (o3, o4, o5, o6):
+            assert np.array_equal(hip.get(n), ora.get(n)), n.ident
+        assert hip.get(o5)[0] == 10.25 and hip.get(o6)[0] == 11.75
+        hip.close()
