@@ -684,7 +684,8 @@ int g_force_tile = 0, g_force_splits = 0;   // tuning overrides of the probe bui
 #endif
 
 // Tile size and split-K factor, from a measured sweep on MI355X (bf16 operands).  256x256 tiles
-// (one workgroup per CU) win only when the output alone gives >= 256 of them; anything smaller
+// (one workgroup per CU) win only when the output alone gives >= 256 of them and K runs at least
+// 8 stages (below that a launch is all prologue and epilogue); anything else
 // runs 128x128 tiles, two workgroups per CU, and when those are fewer than 256 K is split
 // towards ~512 workgroups, never below 8 K stages per split.  Splits are summed in index order by
 // splitk_reduce_kernel (deterministic).
@@ -695,7 +696,7 @@ TileConfig tile_config(const GemmDesc& d) {
   const long t256 = ((d.M + 255) / 256) * ((d.N + 255) / 256) * nb;
   const long t128 = ((d.M + 127) / 128) * ((d.N + 127) / 128) * nb;
   TileConfig c;
-  if (t256 >= 256 && d.M > 128 && d.N > 128) { c.big = true; c.splits = 1; }
+  if (t256 >= 256 && d.M > 128 && d.N > 128 && d.K >= 512) { c.big = true; c.splits = 1; }
   else {
     c.big = false;
     long s = 1;
