@@ -62,7 +62,7 @@ __device__ long long g_gemm_stamps[8 * 4096];
 #endif
 
 #ifndef OCANNL_GEMM_DEEP_PREFETCH
-#define OCANNL_GEMM_DEEP_PREFETCH 0   // 1: two global-load register sets for the bf16 256x256 tile (spills next to double-buffered fragments)
+#define OCANNL_GEMM_DEEP_PREFETCH 0   // 1: two global-load register sets for bf16 sources
 #endif
 
 constexpr int kThreads = 256;
@@ -359,9 +359,10 @@ gemm_bf16_kernel(const GemmArgs g) {
   const long ksteps = kend > kbeg ? (kend - kbeg + kBK - 1) / kBK : 0;
 
   // Software pipeline.  LDS is double buffered; global loads run kPF tiles ahead of the tile being
-  // multiplied, held in kPF register sets.  One set is what the register file affords next to a
-  // 256-register accumulator; the code is written for any depth.
-  constexpr int kPF = (OCANNL_GEMM_DEEP_PREFETCH && BM >= 256 && sizeof(AT) == 2 && sizeof(BT) == 2) ? 2 : 1;
+  // multiplied, held in kPF register sets.  The code is written for one or two sets; two were
+  // measured slower for both tile sizes (the second set spills next to the double-buffered
+  // fragments), so one it is unless OCANNL_GEMM_DEEP_PREFETCH is defined.
+  constexpr int kPF = (OCANNL_GEMM_DEEP_PREFETCH && sizeof(AT) == 2 && sizeof(BT) == 2) ? 2 : 1;
   Stager<BM, AT, A_KC> sa[kPF];
   Stager<BN, BT, B_KC> sb[kPF];
   sa[0].load(A, lda, m0, kbeg, g.M, kend, tid);
@@ -430,12 +431,13 @@ gemm_bf16_kernel(const GemmArgs g) {
   // -- with one wave per SIMD nothing else would hide them.  Global loads of tile ks + 1 go with
   // the first half of the MFMAs, its LDS writes with the second half, the LDS reads of the next
   // sub-step's fragments with the current sub-step.
-  auto fast_step = [&](long ks, auto loads_c) __attribute__((always_inline)) {
-    constexpr bool kLoads = decltype(loads_c)::value;
+  auto fast_step = [&](long ks, auto loads_c, auto stores_c, auto par_c) __attribute__((always_inline)) {
+    constexpr bool kLoads = decltype(loads_c)::value, kStores = decltype(stores_c)::value;
+    constexpr int kLoadSet = decltype(par_c)::value, kStoreSet = (kLoadSet + 1) % kPF;   // tile ks + kPF in, tile ks + 1 out
     constexpr int kSub = kBK / 16, kPer = TM * TN, kAll = kSub * kPer, kHalf = kAll / 2;
     constexpr int kA = Stager<BM, AT, A_KC>::kOps, kL = kA + Stager<BN, BT, B_KC>::kOps, kR = TM + TN;
     const int cur = ks & 1;
-    const long kn = kbeg + (ks + 1) * kBK;
+    const long kn = kbeg + (ks + kPF) * kBK;
     const AT* const a_next = A_KC ? A + m0 * lda + kn : A + kn * lda + m0;
     const BT* const b_next = B_KC ? B + n0 * ldb + kn : B + kn * ldb + n0;
     unsigned short* const an = As0 + (cur ^ 1) * kAT;
@@ -460,15 +462,15 @@ gemm_bf16_kernel(const GemmArgs g) {
       if constexpr (kLoads && m < kHalf) {
         static_for<(m + 1) * kL / kHalf - m * kL / kHalf>([&](auto oc) OCN_LAMBDA_INLINE {
           constexpr int o = m * kL / kHalf + decltype(oc)::value;
-          if constexpr (o < kA) sa[0].template load_op<o>(a_next, lda);
-          else sb[0].template load_op<o - kA>(b_next, ldb);
+          if constexpr (o < kA) sa[kLoadSet].template load_op<o>(a_next, lda);
+          else sb[kLoadSet].template load_op<o - kA>(b_next, ldb);
         });
       }
-      if constexpr (kLoads && m >= kHalf) {
+      if constexpr (kStores && m >= kHalf) {
         static_for<(m - kHalf + 1) * kL / kHalf - (m - kHalf) * kL / kHalf>([&](auto oc) OCN_LAMBDA_INLINE {
           constexpr int o = (m - kHalf) * kL / kHalf + decltype(oc)::value;
-          if constexpr (o < kA) sa[0].template store_op<o>(an);
-          else sb[0].template store_op<o - kA>(bn);
+          if constexpr (o < kA) sa[kStoreSet].template store_op<o>(an);
+          else sb[kStoreSet].template store_op<o - kA>(bn);
         });
       }
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[fb][i], bf[fb][j], acc[i][j], 0, 0, 0);
@@ -477,16 +479,27 @@ gemm_bf16_kernel(const GemmArgs g) {
     __syncthreads();
   };
 
-  sa[0].init_ops(lda, tid);
-  sb[0].init_ops(ldb, tid);
+  static_for<kPF>([&](auto p) OCN_LAMBDA_INLINE { sa[decltype(p)::value].init_ops(lda, tid); sb[decltype(p)::value].init_ops(ldb, tid); });
   // (fp32 sources stage twice the registers: with double-buffered fragments on top the loop
   // spills, so they keep the plain loop)
-  constexpr bool kInterleave = kPF == 1 && sizeof(AT) == 2 && sizeof(BT) == 2;
+  constexpr bool kInterleave = sizeof(AT) == 2 && sizeof(BT) == 2 && kPF <= 2;
   const bool full_tile = kInterleave && m0 + BM <= g.M && n0 + BN <= g.N && ksteps > 0 && kbeg + ksteps * kBK <= kend;
   if constexpr (kInterleave) {
     if (full_tile) {
-      for (long ks = 0; ks + 1 < ksteps; ++ks) fast_step(ks, std::true_type{});
-      fast_step(ksteps - 1, std::false_type{});
+      using Y = std::true_type; using N = std::false_type;
+      using P0 = std::integral_constant<int, 0>; using P1 = std::integral_constant<int, 1 % kPF>;
+      if constexpr (kPF == 1) {
+        for (long ks = 0; ks + 1 < ksteps; ++ks) fast_step(ks, Y{}, Y{}, P0{});
+        fast_step(ksteps - 1, N{}, N{}, P0{});
+      } else {
+        // two register sets: steps come in pairs so that the set numbers are compile-time constants
+        long ks = 0;
+        for (; ks + 3 < ksteps; ks += 2) { fast_step(ks, Y{}, Y{}, P0{}); fast_step(ks + 1, Y{}, Y{}, P1{}); }
+        const long rem = ksteps - ks;   // 1, 2 or 3 steps left; ks is even
+        if (rem == 3) { fast_step(ks, Y{}, Y{}, P0{}); fast_step(ks + 1, N{}, Y{}, P1{}); fast_step(ks + 2, N{}, N{}, P0{}); }
+        else if (rem == 2) { fast_step(ks, N{}, Y{}, P0{}); fast_step(ks + 1, N{}, N{}, P1{}); }
+        else fast_step(ks, N{}, N{}, P0{});
+      }
     }
   }
   if (!full_tile) {
