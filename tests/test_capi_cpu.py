@@ -82,3 +82,28 @@ def test_plan_pool_segments_matches_reference_rule():
     assert assign == [(0, 0), (0, 256)] and sizes == [264]
     with pytest.raises(B.User_error):
         B.plan_pool_segments([(200, 8)], cap=128)
+
+
+def test_planner_rewrites_show_in_the_generated_source():
+    # compile-only checks (no GPU): the kernel-fusing rewrites fire on shapes that call for them and
+    # each can be switched off
+    import re
+    from ocannl_amd import llir as L
+    kw = dict(batch=4, seq=128, d_model=128, heads=2, d_ff=256, layers=1, vocab=2048, prec="bfloat16", grad_prec="single")
+    w = W.transformer(**kw)
+    full = B.compile(w.routine)
+    src = full.source()
+    assert "row0_" in src                                   # row groups
+    assert re.search(r"bf\d+_\w+\[[^\]]*\] = single_to_bfloat16\(", src)   # bf16 operand copies kept by producers
+    fills = lambda code: sum(k["kind"] == "fill" for k in code.kernels())
+    assert fills(full) <= 1                                 # zero fills folded into their consumers
+    plain = B.compile(w.routine, "rows=0;bf16_copies=0")
+    assert "row0_" not in plain.source() and len(plain.kernels()) > len(full.kernels())
+    assert all(k["name"].startswith("gemm_bf16_kernel") for k in full.kernels() if k["kind"] == "mfma")
+    # a column sum over many rows is split into partial sums + a combine
+    L.reset_symbols(0)
+    x = L.Node(1, "x", "single", (4096, 256)); out = L.Node(2, "out", "single", (256,))
+    j, i = L.fresh_symbol(), L.fresh_symbol()
+    r = L.Routine("colsum", [L.For(j, 0, 255, [L.For(i, 0, 4095, [
+        L.Set(out, (L.It(j),), L.Binop("add", L.Get(out, (L.It(j),)), L.Get(x, (L.It(i), L.It(j)))))])])])
+    assert len(B.compile(r).kernels()) == 2 and len(B.compile(r, "coop=0").kernels()) == 1
