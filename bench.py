@@ -7,8 +7,8 @@ A "step" is one run of the compiled routine (for the training configurations: fo
 + optimiser update compiled as ONE routine, as ``Train.to_routine`` does) on synthetic inputs that
 are resident in device memory before the timed region starts.  Prints one JSON line.
 
-workloads: transformer (BASELINE config 4, default), dense_bf16 / dense_f32 (config 3),
-attention (config 5), char_mlp (config 2), moons (config 1), copy (a 2 x 256 MiB plain copy: the
+workloads: transformer (benchmark configuration 4, default), dense_bf16 / dense_f32 (configuration 3),
+attention (configuration 5), char_mlp (configuration 2), moons (configuration 1), copy (a 2 x 256 MiB plain copy: the
 yardstick that memory-traffic counters are scaled by).
 """
 from __future__ import annotations

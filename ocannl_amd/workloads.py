@@ -53,7 +53,7 @@ def to_float(a: np.ndarray, prec: str) -> np.ndarray:
 # ------------------------------------------------------------------------------------------------
 
 def half_moons(n: int, noise: float, seed: int):
-    """1024-point half-moons as BASELINE config 1 defines them: two unit-radius half circles, the
+    """1024-point half-moons as benchmark configuration 1 defines them: two unit-radius half circles, the
     second shifted by (1, -0.5) and flipped, N(0, noise) jitter, labels +-1."""
     rng = np.random.default_rng(seed)
     half = n // 2

@@ -102,7 +102,7 @@ def test_dense_contraction_mfma_small(prec, out_prec, tol, order):
 
 @pytest.mark.parametrize("prec,tol", [("bfloat16", 2e-2), ("single", 1e-4)])
 def test_dense_contraction_full_size_sampled_rows(prec, tol):
-    """BASELINE config 3 at full size (b=8192, i=o=4096): too large for the serial checker, so a
+    """Benchmark configuration 3 at full size (b=8192, i=o=4096): too large for the serial checker, so a
     random sample of output rows is recomputed in float64 on the host from the same inputs."""
     b, i, o = 8192, 4096, 4096
     w = W.dense_contraction(b=b, i=i, o=o, prec=prec, out_prec="single")
