@@ -1,0 +1,121 @@
+"""The MFMA contraction kernels against an fp64 recomputation, over every operand layout /
+precision / epilogue combination and over ragged, batched and split-K shapes.  The kernels take
+their inputs exactly (bf16 operands are exact in fp64; fp32 operands of a bf16 contraction are
+rounded to bf16 first, as the kernel does), so the only error is fp32 accumulation order."""
+import numpy as np
+import pytest
+
+from ocannl_amd import llir as L
+from ocannl_amd import workloads as W
+from parity import HipRun
+
+pytestmark = pytest.mark.gpu
+
+
+def _routine(M, N, K, a_prec, b_prec, c_prec, a_kc, b_kc, accumulate, batch=0):
+    """C[(z,) m, n] (+)= sum_k A * B with A stored [m][k] (a_kc) or [k][m], B stored [n][k] (b_kc) or [k][n]."""
+    L.reset_symbols(0)
+    bd = (batch,) if batch else ()
+    A = L.Node(1, "a", a_prec, bd + ((M, K) if a_kc else (K, M)))
+    B = L.Node(2, "b", b_prec, bd + ((N, K) if b_kc else (K, N)))
+    C = L.Node(3, "c", c_prec, bd + (M, N))
+    z, m, n, k = (L.fresh_symbol() for _ in range(4))
+    zi = (L.It(z),) if batch else ()
+    ai = zi + ((L.It(m), L.It(k)) if a_kc else (L.It(k), L.It(m)))
+    bi = zi + ((L.It(n), L.It(k)) if b_kc else (L.It(k), L.It(n)))
+    ci = zi + (L.It(m), L.It(n))
+    nest = L.For(m, 0, M - 1, [L.For(n, 0, N - 1, [L.For(k, 0, K - 1, [
+        L.Set(C, ci, L.Ternop("fma", L.Get(A, ai), L.Get(B, bi), L.Get(C, ci)))])])])
+    if batch:
+        nest = L.For(z, 0, batch - 1, [nest])
+    body = ([] if accumulate else [L.ZeroOut(C)]) + [nest]
+    return L.Routine("contract", body), A, B, C
+
+
+def _check(M, N, K, a_prec, b_prec, c_prec, a_kc, b_kc, accumulate, batch=0, seed=0, copies=True):
+    r, A, B, C = _routine(M, N, K, a_prec, b_prec, c_prec, a_kc, b_kc, accumulate, batch)
+    rng = np.random.default_rng(seed)
+    av = rng.standard_normal(A.dims).astype(np.float32); bv = rng.standard_normal(B.dims).astype(np.float32)
+    cv = rng.standard_normal(C.dims).astype(np.float32)
+    init = {1: W.as_prec(av, a_prec), 2: W.as_prec(bv, b_prec), 3: W.as_prec(cv, c_prec)}
+    hip = HipRun(r, init, "min_mfma_flops=1" + ("" if copies else ";bf16_copies=0"))
+    ks = hip.code.kernels()
+    mixed = copies and (a_prec == "single") != (b_prec == "single")
+    # (a contraction with one fp32 operand gets a pass that rounds that operand to bf16 first)
+    assert [k["kind"] for k in ks] == (["generated", "mfma"] if mixed else ["mfma"]), ks
+    hip.step()
+    got = W.to_float(hip.get(C), c_prec).astype(np.float64)
+    bf16_compute = not (a_prec == "single" and b_prec == "single")
+    a64 = W.to_float(W.as_prec(av, "bfloat16" if bf16_compute else a_prec), "bfloat16" if bf16_compute else a_prec).astype(np.float64)
+    b64 = W.to_float(W.as_prec(bv, "bfloat16" if bf16_compute else b_prec), "bfloat16" if bf16_compute else b_prec).astype(np.float64)
+    if not a_kc: a64 = np.swapaxes(a64, -1, -2)
+    if not b_kc: b64 = np.swapaxes(b64, -1, -2)
+    want = a64 @ np.swapaxes(b64, -1, -2)
+    if accumulate:
+        want = want + W.to_float(init[3], c_prec).astype(np.float64)
+    scale = np.max(np.abs(want))
+    err = np.max(np.abs(got - want)) / scale
+    tol = 2.0 ** -8 if c_prec == "bfloat16" else 2e-6 * max(1.0, np.sqrt(K) / 8)
+    assert err <= tol, (err, tol, ks[-1]["name"])
+    hip.close()
+    return ks[-1]["name"]
+
+
+@pytest.mark.parametrize("a_kc", [True, False])
+@pytest.mark.parametrize("b_kc", [True, False])
+@pytest.mark.parametrize("precs", [("bfloat16", "bfloat16", "single"), ("bfloat16", "bfloat16", "bfloat16"),
+                                   ("single", "bfloat16", "single"), ("bfloat16", "single", "single"),
+                                   ("single", "single", "single")])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_layouts_precisions_epilogues_on_a_ragged_shape(a_kc, b_kc, precs, accumulate):
+    # 136 x 72 x 200: no extent is a multiple of the tile or of the K stage; contiguous extents are
+    # multiples of 8 as the planner requires
+    name = _check(136, 72, 200, precs[0], precs[1], precs[2], a_kc, b_kc, accumulate)
+    assert ("gemm_f32" in name) == (precs[0] == "single" and precs[1] == "single")
+
+
+@pytest.mark.parametrize("a_kc", [True, False])
+@pytest.mark.parametrize("b_kc", [True, False])
+@pytest.mark.parametrize("which", ["a", "b"])
+def test_fp32_operand_rounded_inside_the_kernel(a_kc, b_kc, which):
+    # without the bf16 scratch copy the kernel itself rounds the fp32 operand on the way into LDS
+    precs = ("single", "bfloat16") if which == "a" else ("bfloat16", "single")
+    name = _check(264, 136, 328, precs[0], precs[1], "single", a_kc, b_kc, True, seed=6, copies=False)
+    assert "float" in name
+    _check(1024, 1024, 512, precs[0], precs[1], "bfloat16", a_kc, b_kc, False, seed=7, copies=False)
+
+
+@pytest.mark.parametrize("shape", [(128, 128, 64), (256, 256, 64), (264, 520, 72), (1000, 24, 1032), (512, 384, 1024),
+                                   (2048, 1024, 512)])
+@pytest.mark.parametrize("layout", [(True, True), (True, False), (False, False)])
+def test_shapes_full_and_ragged_tiles(shape, layout):
+    M, N, K = shape
+    _check(M, N, K, "bfloat16", "bfloat16", "single", layout[0], layout[1], True, seed=1)
+
+
+@pytest.mark.parametrize("layout", [(True, True), (False, False), (True, False)])
+@pytest.mark.parametrize("c_prec", ["single", "bfloat16"])
+def test_split_k(layout, c_prec):
+    # small output, long K: split over workgroups, partial tiles summed in index order
+    _check(128, 256, 8192, "bfloat16", "bfloat16", c_prec, layout[0], layout[1], True, seed=2)
+    _check(72, 136, 4096, "single", "bfloat16", c_prec, layout[0], layout[1], False, seed=3)
+
+
+@pytest.mark.parametrize("layout", [(True, True), (True, False), (False, True)])
+def test_batched(layout):
+    _check(136, 64, 72, "bfloat16", "bfloat16", "single", layout[0], layout[1], False, batch=12, seed=4)
+    _check(256, 256, 64, "single", "bfloat16", "single", layout[0], layout[1], True, batch=16, seed=5)
+
+
+def test_split_k_is_deterministic():
+    r, A, B, C = _routine(128, 128, 8192, "bfloat16", "bfloat16", "single", False, False, False)
+    rng = np.random.default_rng(9)
+    init = {1: W.as_prec(rng.standard_normal(A.dims).astype(np.float32), "bfloat16"),
+            2: W.as_prec(rng.standard_normal(B.dims).astype(np.float32), "bfloat16")}
+    outs = []
+    for _ in range(3):
+        hip = HipRun(r, init, "min_mfma_flops=1")
+        hip.step(); hip.step()
+        outs.append(hip.get(C).copy())
+        hip.close()
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
