@@ -514,64 +514,43 @@ gemm_bf16_kernel(const GemmArgs g) {
 }
 
 // ---- fp32 compute -------------------------------------------------------------------------------
-// LDS holds [row][k] floats, k contiguous; a lane reads 4 consecutive k of its row with one
-// ds_read_b128 and feeds four v_mfma_f32_32x32x2_f32: instruction q multiplies k = q (lanes 0-31)
-// and k = 4 + q (lanes 32-63) -- A and B use the same assignment, so the sum is complete.
+// v_mfma_f32_32x32x2_f32: a lane supplies one float of its row per instruction; instruction q of a
+// group of four multiplies k = q (lanes 0-31) and k = 4 + q (lanes 32-63) of an 8-k sub-step -- A
+// and B use the same assignment, so the sum is complete.
+//   K-contiguous operand:   LDS [row][k], row stride kBKf + kPadf: a lane reads its four k with one
+//     ds_read_b128.
+//   row-contiguous operand: LDS [k][row] as it lies in memory, row stride ROWS + kPadTf: a lane
+//     reads its four k with four ds_read_b32 (lanes of a half read 32 consecutive floats; the two
+//     halves sit 4 k-rows = 32 banks apart): no transposition anywhere.
+constexpr int kPadTf = 8;
+
+template <int ROWS, bool KC>
+constexpr int lds_tile_floats() { return KC ? ROWS * (kBKf + kPadf) : kBKf * (ROWS + kPadTf); }
+
 template <int ROWS, bool KC>
 struct StagerF {
   static constexpr int kChunks = ROWS * (kBKf / 4) / kThreads;   // 16-byte chunks per thread
+  static constexpr int kPerLine = KC ? kBKf / 4 : ROWS / 4;      // chunks per contiguous line
+  static constexpr int kLineStride = KC ? kBKf + kPadf : ROWS + kPadTf;
   f32x4 regs[kChunks];
 
   __device__ __forceinline__ void load(const float* base, long ld, long row0, long k0, long rows, long K, int tid) {
-    if (KC) {
 #pragma unroll
-      for (int j = 0; j < kChunks; ++j) {
-        const int c = tid + kThreads * j;
-        const long row = row0 + c / (kBKf / 4);
-        const long k = k0 + (c % (kBKf / 4)) * 4;
-        f32x4 v = {0, 0, 0, 0};
-        if (row < rows && k < K) v = *reinterpret_cast<const f32x4*>(base + row * ld + k);
-        regs[j] = v;
-      }
-    } else {
-      // 4(k) x 4(row) blocks: (kBKf/4) k-groups x (ROWS/4) row-chunks
-#pragma unroll
-      for (int jb = 0; jb < kChunks / 4; ++jb) {
-        const int blk = tid + kThreads * jb;
-        const long row = row0 + (blk % (ROWS / 4)) * 4;
-        const long kg = k0 + (blk / (ROWS / 4)) * 4;
-        f32x4 in[4];
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          f32x4 v = {0, 0, 0, 0};
-          if (row < rows && kg + kk < K) v = *reinterpret_cast<const f32x4*>(base + (kg + kk) * ld + row);
-          in[kk] = v;
-        }
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-          f32x4 o = {in[0][m], in[1][m], in[2][m], in[3][m]};
-          regs[jb * 4 + m] = o;
-        }
-      }
+    for (int j = 0; j < kChunks; ++j) {
+      const int c = tid + kThreads * j;
+      const long line = c / kPerLine, pos = (c % kPerLine) * 4;
+      f32x4 v = {0, 0, 0, 0};
+      if (KC) { if (row0 + line < rows && k0 + pos < K) v = *reinterpret_cast<const f32x4*>(base + (row0 + line) * ld + k0 + pos); }
+      else    { if (k0 + line < K && row0 + pos < rows) v = *reinterpret_cast<const f32x4*>(base + (k0 + line) * ld + row0 + pos); }
+      regs[j] = v;
     }
   }
 
   __device__ __forceinline__ void store(float* lds, int tid) const {
-    constexpr int kStride = kBKf + kPadf;
-    if (KC) {
 #pragma unroll
-      for (int j = 0; j < kChunks; ++j) {
-        const int c = tid + kThreads * j;
-        *reinterpret_cast<f32x4*>(lds + (c / (kBKf / 4)) * kStride + (c % (kBKf / 4)) * 4) = regs[j];
-      }
-    } else {
-#pragma unroll
-      for (int jb = 0; jb < kChunks / 4; ++jb) {
-        const int blk = tid + kThreads * jb;
-        const int row = (blk % (ROWS / 4)) * 4, kg = (blk / (ROWS / 4)) * 4;
-#pragma unroll
-        for (int m = 0; m < 4; ++m) *reinterpret_cast<f32x4*>(lds + (row + m) * kStride + kg) = regs[jb * 4 + m];
-      }
+    for (int j = 0; j < kChunks; ++j) {
+      const int c = tid + kThreads * j;
+      *reinterpret_cast<f32x4*>(lds + (c / kPerLine) * kLineStride + (c % kPerLine) * 4) = regs[j];
     }
   }
 };
@@ -579,12 +558,13 @@ struct StagerF {
 template <int BM, int BN, bool A_KC, bool B_KC>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, BM >= 256 ? 1 : 2)))
 gemm_f32_kernel(const GemmArgs g) {
-  constexpr int kStride = kBKf + kPadf;
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+  constexpr int kAT = lds_tile_floats<BM, A_KC>(), kBT = lds_tile_floats<BN, B_KC>();
+  constexpr int kAS = StagerF<BM, A_KC>::kLineStride, kBS = StagerF<BN, B_KC>::kLineStride;
   extern __shared__ __align__(16) unsigned short smem[];
   float* fsm = reinterpret_cast<float*>(smem);
   float* const As0 = fsm;
-  float* const Bs0 = fsm + 2 * BM * kStride;
+  float* const Bs0 = fsm + 2 * kAT;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
@@ -626,15 +606,27 @@ gemm_f32_kernel(const GemmArgs g) {
       sa.load(A, lda, m0, kbeg + (ks + 1) * kBKf, g.M, kend, tid);
       sb.load(B, ldb, n0, kbeg + (ks + 1) * kBKf, g.N, kend, tid);
     }
-    const float* as = As0 + cur * BM * kStride + (wm0 + (lane & 31)) * kStride + (lane >> 5) * 4;
-    const float* bs = Bs0 + cur * BN * kStride + (wn0 + (lane & 31)) * kStride + (lane >> 5) * 4;
+    const float* as = As0 + cur * kAT + (A_KC ? (wm0 + (lane & 31)) * kAS + (lane >> 5) * 4 : (lane >> 5) * 4 * kAS + wm0 + (lane & 31));
+    const float* bs = Bs0 + cur * kBT + (B_KC ? (wn0 + (lane & 31)) * kBS + (lane >> 5) * 4 : (lane >> 5) * 4 * kBS + wn0 + (lane & 31));
 #pragma unroll
     for (int kk = 0; kk < kBKf / 8; ++kk) {
       f32x4 af[TM], bf[TN];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const f32x4*>(as + i * 32 * kStride + kk * 8);
+      for (int i = 0; i < TM; ++i) {
+        if (A_KC) af[i] = *reinterpret_cast<const f32x4*>(as + i * 32 * kAS + kk * 8);
+        else {
+          const float* p = as + kk * 8 * kAS + i * 32;
+          af[i] = f32x4{p[0], p[kAS], p[2 * kAS], p[3 * kAS]};
+        }
+      }
 #pragma unroll
-      for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const f32x4*>(bs + j * 32 * kStride + kk * 8);
+      for (int j = 0; j < TN; ++j) {
+        if (B_KC) bf[j] = *reinterpret_cast<const f32x4*>(bs + j * 32 * kBS + kk * 8);
+        else {
+          const float* p = bs + kk * 8 * kBS + j * 32;
+          bf[j] = f32x4{p[0], p[kBS], p[2 * kBS], p[3 * kBS]};
+        }
+      }
       static_for<4>([&](auto qc) OCN_LAMBDA_INLINE {
         static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
           static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
@@ -645,8 +637,8 @@ gemm_f32_kernel(const GemmArgs g) {
       });
     }
     if (more) {
-      sa.store(As0 + (cur ^ 1) * BM * kStride, tid);
-      sb.store(Bs0 + (cur ^ 1) * BN * kStride, tid);
+      sa.store(As0 + (cur ^ 1) * kAT, tid);
+      sb.store(Bs0 + (cur ^ 1) * kBT, tid);
     }
     __syncthreads();
   }
@@ -656,8 +648,8 @@ gemm_f32_kernel(const GemmArgs g) {
 
 template <int BM, int BN, bool A_KC, bool B_KC>
 constexpr size_t bf16_smem() { return 2ull * (lds_tile_elems<BM, A_KC>() + lds_tile_elems<BN, B_KC>()) * sizeof(unsigned short); }
-template <int BM, int BN>
-constexpr size_t f32_smem() { return 2ull * (BM + BN) * (kBKf + kPadf) * sizeof(float); }
+template <int BM, int BN, bool A_KC, bool B_KC>
+constexpr size_t f32_smem() { return 2ull * (lds_tile_floats<BM, A_KC>() + lds_tile_floats<BN, B_KC>()) * sizeof(float); }
 
 // Sums the split-K partials in split order (deterministic) and applies them to C.
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const GemmArgs g) {
@@ -763,11 +755,10 @@ hipError_t launch_bf16_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t
 
 template <int BM, int BN>
 hipError_t launch_f32_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t s, hipEvent_t ev) {
-  constexpr size_t sm = f32_smem<BM, BN>();
-  if (akc && bkc) return launch(gemm_f32_kernel<BM, BN, true, true>, sm, BM, BN, a, s, ev);
-  if (akc && !bkc) return launch(gemm_f32_kernel<BM, BN, true, false>, sm, BM, BN, a, s, ev);
-  if (!akc && bkc) return launch(gemm_f32_kernel<BM, BN, false, true>, sm, BM, BN, a, s, ev);
-  return launch(gemm_f32_kernel<BM, BN, false, false>, sm, BM, BN, a, s, ev);
+  if (akc && bkc) return launch(gemm_f32_kernel<BM, BN, true, true>, f32_smem<BM, BN, true, true>(), BM, BN, a, s, ev);
+  if (akc && !bkc) return launch(gemm_f32_kernel<BM, BN, true, false>, f32_smem<BM, BN, true, false>(), BM, BN, a, s, ev);
+  if (!akc && bkc) return launch(gemm_f32_kernel<BM, BN, false, true>, f32_smem<BM, BN, false, true>(), BM, BN, a, s, ev);
+  return launch(gemm_f32_kernel<BM, BN, false, false>, f32_smem<BM, BN, false, false>(), BM, BN, a, s, ev);
 }
 
 bool a_kcontig(const GemmDesc& d) { return d.a.s_k == 1 || d.K == 1; }
