@@ -322,6 +322,24 @@ struct Printer {
     if (!mirror_lhs.empty()) line += " " + mirror_lhs + " = single_to_bfloat16(" + it->second + ");";
     return line + " }";
   }
+  // Lines that leave in `var` (of every lane) the combination of the lane group's partial values:
+  // xor butterfly inside a wave; a group of 256 lanes is a whole workgroup, whose four waves
+  // exchange their results through LDS (`red_`, declared by the kernel) and combine them in a
+  // fixed order.
+  void group_reduce(const std::string& var, Binop accum, bool dbl, int lanes, const std::string& ind,
+                    std::vector<std::string>& out) {
+    for (int o = std::min(lanes, 64) / 2; o > 0; o >>= 1)
+      out.push_back(ind + var + " = " + combine_expr(accum, dbl, var, "ocn_xshfl(" + var + ", " + std::to_string(o) + ")") + ";");
+    if (lanes > 64) {
+      const std::string red = dbl ? "redd_" : "red_";
+      out.push_back(ind + "if ((threadIdx.x & 63u) == 0) " + red + "[threadIdx.x >> 6] = " + var + ";");
+      out.push_back(ind + "__syncthreads();");
+      out.push_back(ind + var + " = " + combine_expr(accum, dbl, combine_expr(accum, dbl, red + "[0]", red + "[1]"),
+                                                    combine_expr(accum, dbl, red + "[2]", red + "[3]")) + ";");
+      out.push_back(ind + "__syncthreads();");
+    }
+  }
+
   // header of a loop over the row position shared by `lanes` lanes
   std::string row_loop(const std::string& sym, int64_t from, int64_t to, int lanes, const std::string& ind) {
     if (row_iters > 0 && from == 0)
@@ -476,8 +494,7 @@ struct Printer {
     }
     with_defs(inner_defs, {line}, ci, d.lines);
     for (size_t i = 0; i < loops.size(); ++i) { ci.resize(ci.size() - 2); d.lines.push_back(ci + "}"); }
-    for (int o = coop_lanes / 2; o > 0; o >>= 1)
-      d.lines.push_back(ind + part + " = " + combine_expr(coop_accum, dbl, part, "ocn_xshfl(" + part + ", " + std::to_string(o) + ")") + ";");
+    group_reduce(part, coop_accum, dbl, coop_lanes, ind, d.lines);
     Pair narrow = convert_precision(accP, sp);
     d.lines.push_back(ind + c_typ(sp) + " " + scope_name(s.scope) + " = " + narrow.first + part + narrow.second + ";");
     defs.push_back(std::move(d));
@@ -654,8 +671,7 @@ void emit_phase_statements(const Routine& r, Printer& pr, const Phase& ph, int G
     }
     pr.with_defs(defs, lines, ci, body);
     close_seq_loops(ci);
-    for (int o = G / 2; o > 0; o >>= 1)
-      body.push_back(ind + "part_ = " + combine_expr(accum, dbl, "part_", "ocn_xshfl(part_, " + std::to_string(o) + ")") + ";");
+    pr.group_reduce("part_", accum, dbl, G, ind, body);
     const std::string lhs = n.ident + "[" + offset_str(set->idcs, n.dims) + "]";
     Pair narrow = convert_precision(accP, n.prec);
     Pair wide = convert_precision(n.prec, accP);
@@ -737,6 +753,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
           body.push_back(line);
         }
+        if (QG > 64) body.push_back(pind + "__shared__ float red_[4]; __shared__ double redd_[4];");
         // short rows: everything the group produces stays in registers as well (no read-back)
         const bool cached = q.row_len % QG == 0 && q.row_len / QG <= 16;
         if (cached) {

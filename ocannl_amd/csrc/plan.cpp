@@ -992,6 +992,9 @@ void group_rows(const Routine& r, Plan& plan) {
       g.row_len = shape.len;
       int lanes = 1;
       while (lanes * 2 <= 64 && lanes * 2 <= shape.len) lanes *= 2;
+      // a long row (more than 16 elements per lane of a wave) goes to a whole workgroup when that
+      // brings it down to <= 16 per thread: everything the group produces then fits in registers
+      if (shape.len / lanes > 16 && shape.len % 256 == 0 && shape.len / 256 <= 16) lanes = 256;
       g.coop_lanes = lanes;
       // algorithmic bytes: every array the group writes, once, plus every array it reads without
       // having produced it, once; an array indexed by the row position counts rows x T elements,
