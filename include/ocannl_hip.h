@@ -130,7 +130,9 @@ void ocannl_hip_routine_free(ocannl_hip_routine* routine);
 /* lowered_bindings: the `int ref` behind a Static_idx (arrayjit/lib/indexing.ml:60-93). */
 int ocannl_hip_routine_set_static(ocannl_hip_routine* routine, int symbol, int64_t value);
 /* Task.run of the launch closure (cuda_backend.ml:991-1044): range-checks static indices
-   (E_USER on failure, :1015-1030), then enqueues the routine's kernels on the device stream. */
+   (E_USER on failure, :1015-1030), binds the merge buffer for a routine that reads one (pool 0 as it
+   is now, :1009-1011; E_USER when no transfer has filled it or it is smaller than the merge node),
+   then enqueues the routine's kernels on the device stream. */
 int ocannl_hip_routine_run(ocannl_hip_routine* routine);
 /* Same, bracketing every kernel with HIP events on the device stream; synchronises and writes the
    per-kernel milliseconds (cap >= number of kernels).  For measurement only. */

@@ -285,6 +285,7 @@ struct Printer {
   const Routine& r;
   std::set<int> used_nodes;
   std::set<int> used_statics;
+  bool used_merge = false;
   // when set, this inlined scalar reduction is shared by `coop_lanes` adjacent lanes (lane id in
   // `lane_`): they stride its innermost loop, accumulate in float and combine by butterfly
   // shuffles; the enclosing store is done by lane 0
@@ -390,6 +391,7 @@ struct Printer {
       case Scalar::GetMerge: {
         const Node& n = r.node(s.node);
         for (auto& a : s.idcs) note_idx(a);
+        used_merge = true;
         Pair c = convert_precision(n.prec, prec);
         return c.first + "merge_buffer[" + offset_str(s.idcs, n.dims) + "]" + c.second;
       }
@@ -857,6 +859,11 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
       const Node& n = r.node(id);
       decls.push_back(std::string(c_typ(n.prec)) + " * __restrict__ " + n.ident);
       gk.params.push_back({KernelParam::NodePtr, id});
+    }
+    if (pr.used_merge) {
+      if (r.merge_node < 0) throw InvalidArgument("hip backend: routine " + r.name + " reads a merge buffer it does not declare");
+      decls.push_back(std::string("const ") + c_typ(r.node(r.merge_node).prec) + " * __restrict__ merge_buffer");
+      gk.params.push_back({KernelParam::MergeBuffer, r.merge_node});
     }
     for (auto& s : r.statics) {
       if (!pr.used_statics.count(s.sym)) continue;

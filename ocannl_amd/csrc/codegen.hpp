@@ -16,8 +16,8 @@
 namespace ocannl {
 
 struct KernelParam {
-  enum Kind { NodePtr, StaticIdx } kind;
-  int id;   // node id or static symbol
+  enum Kind { NodePtr, StaticIdx, MergeBuffer } kind;
+  int id;   // node id (NodePtr; MergeBuffer: the node whose layout the buffer has) or static symbol
 };
 
 struct GeneratedKernel {

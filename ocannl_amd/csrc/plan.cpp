@@ -1274,7 +1274,13 @@ void lift_routine_locals(Routine& r, Plan& plan) {
 
 }  // namespace
 
-Plan make_plan(Routine& r, const PlanOptions& opt) {
+Plan make_plan(Routine& r, const PlanOptions& requested) {
+  PlanOptions opt = requested;
+  if (r.merge_node >= 0) {
+    // routines that read the merge buffer are short pointwise accumulations (cuda_backend.ml:1009-1011
+    // binds the buffer at launch): plain one-kernel-per-statement plans, no fusing rewrites
+    opt.enable_mfma = opt.enable_row_groups = opt.enable_serial_group = opt.enable_bf16_copies = false;
+  }
   Plan plan;
   std::string label;
   int next_sym = 0;

@@ -140,6 +140,7 @@ struct ocannl_hip_routine {
     std::vector<void*> ptr_vals;       // storage for pointer arguments
     std::vector<uint32_t> idx_vals;    // storage for static-index arguments
     std::vector<int> idx_syms;
+    int merge_slot = -1;               // index in ptr_vals of the merge-buffer argument, bound at launch
     std::vector<void*> args;
     unsigned grid = 1, block = 256;
     void* fill_ptr = nullptr; uint64_t fill_bytes = 0;
@@ -183,6 +184,17 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
       throw UserError("hip backend: static index " + sym_ident(s.sym) + " is too big: " + std::to_string(v) +
                       " (range 0.." + std::to_string(s.range - 1) + ")");
   }
+  // the merge buffer is bound when the routine is scheduled, not when it is linked: it may have been
+  // regrown since (cuda_backend.ml:1009-1011, :130-134)
+  void* merge_base = nullptr;
+  if (r.merge_node >= 0) {
+    auto it = dev.pools.find(0);
+    const uint64_t need = (uint64_t)r.node(r.merge_node).size_in_bytes();
+    if (it == dev.pools.end() || it->second.second < need)
+      throw UserError("hip backend: routine " + r.name + " reads the merge buffer as " + r.node(r.merge_node).ident +
+                      " but no transfer has filled it (device_to_device ~into_merge_buffer first)");
+    merge_base = it->second.first;
+  }
   const bool timed = kernel_ms != nullptr;
   if (timed) {
     if (cap < (int)rt.launches.size()) throw InvalidArgument("run_timed: kernel_ms too small");
@@ -209,6 +221,7 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
       hip_check(hipMemsetAsync(l.fill_ptr, 0, l.fill_bytes, dev.stream), "hipMemsetAsync");
     } else if (ph.kind == Phase::Generic) {
       for (size_t i = 0; i < l.idx_syms.size(); ++i) l.idx_vals[i] = (uint32_t)rt.statics[l.idx_syms[i]];
+      if (l.merge_slot >= 0) l.ptr_vals[l.merge_slot] = merge_base;
       hip_check(hipModuleLaunchKernel(l.fn, l.grid, 1, 1, l.block, 1, 1, 0, dev.stream, l.args.data(), nullptr),
                 "hipModuleLaunchKernel");
     } else {
@@ -593,7 +606,6 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
     auto rt = std::make_unique<ocannl_hip_routine>();
     rt->dev = dev;
     rt->code = &cr;
-    if (cr.r.merge_node >= 0) throw UserError("hip backend: merge-buffer routines need a second device and are not supported");
     // ctx nodes from the caller's table
     std::map<int, const ocannl_hip_node_loc*> by_id;
     for (int i = 0; i < n_locs; ++i) by_id[locs[i].node_id] = &locs[i];
@@ -654,15 +666,16 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
         l.grid = (unsigned)blocks;
         l.block = (unsigned)gk.block;
         size_t np = 0, ni = 0;
-        for (auto& p : gk.params) (p.kind == KernelParam::NodePtr ? np : ni)++;
+        for (auto& p : gk.params) (p.kind != KernelParam::StaticIdx ? np : ni)++;
         l.ptr_vals.reserve(np); l.idx_vals.reserve(ni);
         for (auto& p : gk.params) {
           if (p.kind == KernelParam::NodePtr) { l.ptr_vals.push_back(rt->node_ptr.at(p.id)); }
+          else if (p.kind == KernelParam::MergeBuffer) { l.merge_slot = (int)l.ptr_vals.size(); l.ptr_vals.push_back(nullptr); }
           else { l.idx_vals.push_back(0); l.idx_syms.push_back(p.id); }
         }
         size_t ip = 0, ii = 0;
         for (auto& p : gk.params) {
-          if (p.kind == KernelParam::NodePtr) l.args.push_back(&l.ptr_vals[ip++]);
+          if (p.kind != KernelParam::StaticIdx) l.args.push_back(&l.ptr_vals[ip++]);
           else l.args.push_back(&l.idx_vals[ii++]);
         }
       }
@@ -674,7 +687,7 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
       const GeneratedKernel* gk = nullptr;
       for (auto& k : cr.mod.kernels) if (k.phase_index == l.phase) gk = &k;
       size_t ip = 0, ii = 0, ai = 0;
-      for (auto& p : gk->params) l.args[ai++] = p.kind == KernelParam::NodePtr ? (void*)&l.ptr_vals[ip++] : (void*)&l.idx_vals[ii++];
+      for (auto& p : gk->params) l.args[ai++] = p.kind != KernelParam::StaticIdx ? (void*)&l.ptr_vals[ip++] : (void*)&l.idx_vals[ii++];
     }
     dev->live_routines++;
     *out = rt.release();
