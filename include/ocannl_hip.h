@@ -109,7 +109,9 @@ int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** code);
    (lanes sharing reductions; off = the summation order of the serial C code), rows=0|1 (fusing
    consecutive row-wise phases into one kernel), bf16_copies=0|1 (rounding an fp32 operand of a
    bf16 contraction once into scratch instead of in every kernel that reads it), serial=0|1 (a routine
-   of tiny phases as one single-workgroup kernel), min_mfma_flops=<n>. */
+   of tiny phases as one single-workgroup kernel), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
+   indices and offsets in generated kernels, the `large_models` setting of c_syntax.ml:111-112; a
+   routine with a node of more than 2^31 - 1 elements gets them without asking). */
 int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, ocannl_hip_code** code);
 void ocannl_hip_code_free(ocannl_hip_code* code);
 int ocannl_hip_code_num_routines(ocannl_hip_code* code, int* n);

@@ -286,6 +286,9 @@ struct Printer {
   std::set<int> used_nodes;
   std::set<int> used_statics;
   bool used_merge = false;
+  // type of loop iterators and offsets: 64-bit when a node is too large for 32-bit offsets
+  // (the `large_models` setting, c_syntax.ml:111-112)
+  std::string idx_t = "uint32_t";
   // when set, this inlined scalar reduction is shared by `coop_lanes` adjacent lanes (lane id in
   // `lane_`): they stride its innermost loop, accumulate in float and combine by butterfly
   // shuffles; the enclosing store is done by lane 0
@@ -344,9 +347,9 @@ struct Printer {
   // header of a loop over the row position shared by `lanes` lanes
   std::string row_loop(const std::string& sym, int64_t from, int64_t to, int lanes, const std::string& ind) {
     if (row_iters > 0 && from == 0)
-      return ind + "_Pragma(\"unroll\") for (uint32_t it_ = 0; it_ < " + std::to_string(row_iters) + "; ++it_) { const uint32_t " +
+      return ind + "_Pragma(\"unroll\") for (uint32_t it_ = 0; it_ < " + std::to_string(row_iters) + "; ++it_) { const " + idx_t + " " +
              sym + " = lane_ + it_ * " + std::to_string(lanes) + ";";
-    return ind + "for (uint32_t " + sym + " = " + std::to_string(from) + " + lane_; " + sym + " <= " + std::to_string(to) +
+    return ind + "for (" + idx_t + " " + sym + " = " + std::to_string(from) + " + lane_; " + sym + " <= " + std::to_string(to) +
            "; " + sym + " += " + std::to_string(lanes) + ") {";
   }
   // when set, a read of exactly this (node, indices) prints as `self_name`
@@ -407,7 +410,7 @@ struct Printer {
         const Node& n = r.node(s.node);
         note(s.node, s.idcs);
         Pair c = convert_precision(n.prec, prec);
-        std::string dyn = std::string("((") + c_typ(Prec::Uint32) + ")(" + scalar(s.arg_prec, *s.a, ind, defs) + "))";
+        std::string dyn = std::string("((") + idx_t + ")(" + scalar(s.arg_prec, *s.a, ind, defs) + "))";
         return c.first + n.ident + "[" + offset_str(s.idcs, n.dims, s.dyn_axis, dyn) + "]" + c.second;
       }
       case Scalar::Const: {
@@ -422,7 +425,7 @@ struct Printer {
       }
       case Scalar::Index: {
         note_idx(s.index);
-        Pair c = convert_precision(Prec::Uint32, prec);
+        Pair c = convert_precision(idx_t == "uint64_t" ? Prec::Uint64 : Prec::Uint32, prec);
         return c.first + axis_str(s.index) + c.second;
       }
       case Scalar::Tern: {
@@ -478,7 +481,7 @@ struct Printer {
       if (i + 1 == loops.size())
         d.lines.push_back(row_loop(sy, loops[i]->from, loops[i]->to, coop_lanes, ci));
       else
-        d.lines.push_back(ci + "for (uint32_t " + sy + " = " + std::to_string(loops[i]->from) + "; " + sy + " <= " +
+        d.lines.push_back(ci + "for (" + idx_t + " " + sy + " = " + std::to_string(loops[i]->from) + "; " + sy + " <= " +
                           std::to_string(loops[i]->to) + "; ++" + sy + ") {");
       ci += "  ";
     }
@@ -524,7 +527,7 @@ struct Printer {
       case Stmt::Comment: out.push_back(ind + "/* " + c.text + " */"); break;
       case Stmt::For: {
         const std::string s = sym_ident(c.sym);
-        out.push_back(ind + "for (uint32_t " + s + " = " + std::to_string(c.from) + "; " + s + " <= " +
+        out.push_back(ind + "for (" + idx_t + " " + s + " = " + std::to_string(c.from) + "; " + s + " <= " +
                       std::to_string(c.to) + "; ++" + s + ") {");
         block(c.body, ind + "  ", out);
         out.push_back(ind + "}");
@@ -536,7 +539,7 @@ struct Printer {
         used_nodes.insert(c.node);
         const std::string v = "z" + std::to_string(fresh++);
         Pair cv = convert_precision(Prec::Double, n.prec);
-        out.push_back(ind + "for (uint32_t " + v + " = 0; " + v + " < " + std::to_string(n.num_elems()) + "; ++" + v +
+        out.push_back(ind + "for (" + idx_t + " " + v + " = 0; " + v + " < " + std::to_string(n.num_elems()) + "; ++" + v +
                       ") " + n.ident + "[" + v + "] = " + cv.first + "0" + cv.second + ";");
         break;
       }
@@ -636,7 +639,7 @@ void emit_phase_statements(const Routine& r, Printer& pr, const Phase& ph, int G
       if (coop_last && i + 1 == ph.seq_syms.size())
         body.push_back(pr.row_loop(s, ph.seq_from[i], ph.seq_to[i], G, cur_ind));
       else
-        body.push_back(cur_ind + "for (uint32_t " + s + " = " + std::to_string(ph.seq_from[i]) + "; " + s + " <= " +
+        body.push_back(cur_ind + "for (" + pr.idx_t + " " + s + " = " + std::to_string(ph.seq_from[i]) + "; " + s + " <= " +
                        std::to_string(ph.seq_to[i]) + "; ++" + s + ") {");
       cur_ind += "  ";
     }
@@ -729,6 +732,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     const Phase& ph = plan.phases[pi];
     if (ph.kind != Phase::Generic) continue;
     Printer pr(r);
+    if (plan.large_index) pr.idx_t = "uint64_t";
     pr.mirrors = &plan.mirrors;
     std::vector<std::string> body;
     const std::string ind = "  ";
@@ -750,7 +754,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
         const size_t n = q.row_outer_ext.size();
         for (int k = (int)n - 1; k >= 0; --k) {
           const std::string ext = std::to_string(q.row_outer_ext[k]) + "ull";
-          std::string line = pind + "const uint32_t row" + std::to_string(k) + "_ = (uint32_t)(";
+          std::string line = pind + "const " + pr.idx_t + " row" + std::to_string(k) + "_ = (" + pr.idx_t + ")(";
           if (k == 0) line += "pt_);";
           else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
           body.push_back(line);
@@ -783,7 +787,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           body.push_back(pind + "{  /* " + m.label + " */");
           const std::string mi_ind = pind + "  ";
           for (size_t k = 0; k < m.row_outer_syms.size(); ++k)
-            body.push_back(mi_ind + "const uint32_t " + sym_ident(m.row_outer_syms[k]) + " = row" + std::to_string(k) + "_;");
+            body.push_back(mi_ind + "const " + pr.idx_t + " " + sym_ident(m.row_outer_syms[k]) + " = row" + std::to_string(k) + "_;");
           if (m.row_role == Phase::RowPointwise) {
             body.push_back(pr.row_loop(sym_ident(m.row_sym), 0, q.row_len - 1, QG, mi_ind));
             emit_phase_statements(r, pr, m, 1, false, mi_ind + "  ", body);
@@ -804,7 +808,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           const size_t i = order[k];
           const std::string sy = sym_ident(q.par_syms[i]);
           const std::string ext = std::to_string(q.par_ext[i]) + "ull";
-          std::string line = pind + "const uint32_t " + sy + " = (uint32_t)(" + std::to_string(q.par_from[i]) + " + ";
+          std::string line = pind + "const " + pr.idx_t + " " + sy + " = (" + pr.idx_t + ")(" + std::to_string(q.par_from[i]) + " + ";
           if (k == 0) line += "pt_);";
           else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
           body.push_back(line);
@@ -824,7 +828,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           const Node& fn = r.node(q.fill_node);
           pr.used_nodes.insert(q.fill_node);
           Pair cv = convert_precision(Prec::Double, fn.prec);
-          body.push_back(ind + "for (uint32_t z_ = threadIdx.x; z_ < " + std::to_string(fn.num_elems()) + "u; z_ += 256u) " +
+          body.push_back(ind + "for (" + pr.idx_t + " z_ = threadIdx.x; z_ < " + std::to_string(fn.num_elems()) + "ull; z_ += 256u) " +
                          fn.ident + "[z_] = " + cv.first + "0" + cv.second + ";");
         } else {
           uint64_t qt = (uint64_t)q.coop_lanes;
@@ -838,7 +842,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
       }
       total_threads = 256;
     } else {
-      body.push_back(ind + "const uint64_t gtid_ = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;");
+      body.push_back(ind + "const uint64_t gtid_ = ((uint64_t)blockIdx.y * gridDim.x + blockIdx.x) * blockDim.x + threadIdx.x;");
       total_threads = emit_points(ph, ind, "return");
     }
 
@@ -867,7 +871,12 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     }
     for (auto& s : r.statics) {
       if (!pr.used_statics.count(s.sym)) continue;
-      decls.push_back("const uint32_t " + sym_ident(s.sym));
+      if (plan.large_index) {   // widen before any offset arithmetic
+        decls.push_back("const uint32_t " + sym_ident(s.sym) + "_arg");
+        body.insert(body.begin(), "  const uint64_t " + sym_ident(s.sym) + " = " + sym_ident(s.sym) + "_arg;");
+      } else {
+        decls.push_back("const uint32_t " + sym_ident(s.sym));
+      }
       gk.params.push_back({KernelParam::StaticIdx, s.sym});
     }
     src << "/* phase " << pi << ": " << ph.label << " */\n";

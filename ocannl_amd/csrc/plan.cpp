@@ -883,6 +883,9 @@ bool row_member(const Routine& r, Phase& ph, RowShape& shape, bool first) {
   if (ph.seq_syms.size() == 1 && reduction_shape(r, ph, &accum)) {          // a row reduction
     const int64_t T = ph.seq_to[0] + 1;
     if (!outer_matches(ext.size()) || (shape.len >= 0 && shape.len != T) || T < 16) return false;
+    // lanes share a row through a float (or double) accumulator: integer rows stay sequential and exact
+    const Prec rp = r.node(ph.inner[0]->node).prec;
+    if (!(rp == Prec::Single || rp == Prec::Double || rp == Prec::Bfloat16 || rp == Prec::Half)) return false;
     // the reduced operand must be walked contiguously
     std::vector<Access> acc; bool fl = false; std::set<ScopeId> d;
     scalar_accesses(*ph.inner[0]->value, acc, fl, d);
@@ -1282,6 +1285,8 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     opt.enable_mfma = opt.enable_row_groups = opt.enable_serial_group = opt.enable_bf16_copies = false;
   }
   Plan plan;
+  plan.large_index = opt.large_models;
+  for (auto& kv : r.nodes) if (kv.second.num_elems() > (int64_t)0x7FFFFFFF) plan.large_index = true;
   std::string label;
   int next_sym = 0;
   Bf16Copies copies;

@@ -88,6 +88,7 @@ struct PlanOptions {
   bool enable_coop = true;
   bool enable_row_groups = true;
   bool enable_serial_group = true;   // tiny routines as one single-workgroup kernel
+  bool large_models = false;        // 64-bit offsets in generated kernels even when every node is small
   bool enable_bf16_copies = true;   // keep bf16 copies of fp32 operands of mixed contractions (written by the producing kernels)
 };
 
@@ -97,6 +98,7 @@ struct Plan {
   // fp32 node -> bf16 scratch copy kept in step by every generated store to the node (a store to
   // the node also stores the rounded value to the copy): the copy feeds bf16 contractions
   std::map<int, int> mirrors;
+  bool large_index = false;    // generated kernels compute offsets in 64 bits
 };
 
 Plan make_plan(Routine& r, const PlanOptions& opt);

@@ -112,6 +112,7 @@ PlanOptions parse_options(const char* options) {
     else if (k == "rows") o.enable_row_groups = v != "0";
     else if (k == "bf16_copies") o.enable_bf16_copies = v != "0";
     else if (k == "serial") o.enable_serial_group = v != "0";
+    else if (k == "large_models") o.large_models = v != "0";
     else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
     else throw InvalidArgument("compile options: unknown key '" + k + "'");
   }
@@ -142,7 +143,7 @@ struct ocannl_hip_routine {
     std::vector<int> idx_syms;
     int merge_slot = -1;               // index in ptr_vals of the merge-buffer argument, bound at launch
     std::vector<void*> args;
-    unsigned grid = 1, block = 256;
+    unsigned grid = 1, grid_y = 1, block = 256;
     void* fill_ptr = nullptr; uint64_t fill_bytes = 0;
   };
   std::vector<Launch> launches;
@@ -222,7 +223,7 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
     } else if (ph.kind == Phase::Generic) {
       for (size_t i = 0; i < l.idx_syms.size(); ++i) l.idx_vals[i] = (uint32_t)rt.statics[l.idx_syms[i]];
       if (l.merge_slot >= 0) l.ptr_vals[l.merge_slot] = merge_base;
-      hip_check(hipModuleLaunchKernel(l.fn, l.grid, 1, 1, l.block, 1, 1, 0, dev.stream, l.args.data(), nullptr),
+      hip_check(hipModuleLaunchKernel(l.fn, l.grid, l.grid_y, 1, l.block, 1, 1, 0, dev.stream, l.args.data(), nullptr),
                 "hipModuleLaunchKernel");
     } else {
       const GemmDesc& g = ph.gemm;
@@ -662,8 +663,11 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
         if (gk.phase_index != (int)pi) throw InvalidArgument("link: kernel table out of step with the plan");
         hip_check(hipModuleGetFunction(&l.fn, rt->module, gk.name.c_str()), "hipModuleGetFunction");
         const uint64_t blocks = (gk.threads + gk.block - 1) / gk.block;
-        if (blocks == 0 || blocks > 0x7FFFFFFFull) throw UserError("hip backend: phase too large for one launch: " + gk.name);
-        l.grid = (unsigned)blocks;
+        // a launch may not exceed 2^32 threads along one grid dimension: rows of 2^22 workgroups
+        constexpr uint64_t kRow = 1ull << 22;
+        if (blocks == 0 || blocks > kRow * 65535ull) throw UserError("hip backend: phase too large for one launch: " + gk.name);
+        l.grid = (unsigned)std::min(blocks, kRow);
+        l.grid_y = (unsigned)((blocks + kRow - 1) / kRow);
         l.block = (unsigned)gk.block;
         size_t np = 0, ni = 0;
         for (auto& p : gk.params) (p.kind != KernelParam::StaticIdx ? np : ni)++;

@@ -9,7 +9,8 @@ Follows, function by function:
 * ``C_syntax.pp_ll``             c_syntax.ml:441-704                 -> :meth:`_Emitter.stmt`
 * ``C_syntax.pp_scalar``         c_syntax.ml:706-855                 -> :meth:`_Emitter.scalar`
 * ``C_syntax.pp_array_offset``   c_syntax.ml:367-379                 -> :func:`array_offset`
-* ``Pure_C_config``              c_syntax.ml:96-321 (uint32_t loop indices, no prefixes)
+* ``Pure_C_config``              c_syntax.ml:96-321 (uint32_t loop indices, uint64_t under the
+  ``large_models`` setting; no prefixes)
 * ``CC_syntax_config`` overrides arrayjit/lib/cc_backend.ml:155-323 (bf16/half/fp8 computed in
   float with a conversion around every single operation)
 * op spelling tables             arrayjit/lib/ops.ml:579-863
@@ -42,6 +43,16 @@ C_TYP = {  # Ops.c_typ_of_prec, ops.ml:324-337
     "bfloat16": "unsigned short", "fp8": "unsigned char", "single": "float", "double": "double",
     "void": "void",
 }
+
+# ``Utils.settings.large_models``: a startup-fixed global of the reference, read when the source is
+# generated (c_syntax.ml:17-24). It widens loop indices and integer arguments to 64 bits
+# (c_syntax.ml:111-112) and ``Ops.index_prec ()`` to uint64 (ops.ml:64).
+LARGE_MODELS = False
+
+
+def index_prec() -> str:
+    return "uint64" if LARGE_MODELS else L.INDEX_PREC
+
 
 _INTISH = ("byte", "uint16", "int32", "uint32", "int64", "uint64", "fp8")
 _DBL_OR_INTISH = ("double",) + _INTISH
@@ -367,7 +378,7 @@ class _Emitter:
             return [f"{ind}/* {c.text} */"]
         if isinstance(c, L.For):
             s = L.sym_ident(c.sym)
-            head = f"{ind}for (uint32_t {s} = {c.from_}; {s} <= {c.to}; ++{s}) {{"
+            head = f"{ind}for ({C_TYP[index_prec()]} {s} = {c.from_}; {s} <= {c.to}; ++{s}) {{"
             return [head] + self.stmts(c.body, ind + "  ", True) + [ind + "}"]
         if isinstance(c, L.ZeroOut):
             first = c.node.id not in self.zero_out_seen
@@ -443,7 +454,7 @@ class _Emitter:
         if isinstance(s, L.GetDynamic):
             p, q = convert_precision(s.node.prec, prec)
             ddefs, dexpr = self.scalar(s.dyn_prec, s.dyn_value, ind)
-            dyn = f"(({C_TYP[L.INDEX_PREC]})({dexpr}))"
+            dyn = f"(({C_TYP[index_prec()]})({dexpr}))"
             dims = s.node.dims
             parts = [dyn if i == s.dyn_axis else L.axis_index_str(ix)
                      for i, ix in enumerate(s.idcs)]
@@ -461,7 +472,7 @@ class _Emitter:
             p, q = convert_precision("int64", prec)
             return [], f"{p}{int(s.value)}LL{q}"
         if isinstance(s, L.EmbedIndex):
-            p, q = convert_precision(L.INDEX_PREC, prec)
+            p, q = convert_precision(index_prec(), prec)
             return [], f"{p}{L.axis_index_str(s.idx)}{q}"
         if isinstance(s, L.Binop) and s.op == "arg1":
             return self.scalar(prec, s.a, ind)
@@ -495,7 +506,7 @@ def kernel_params(r: L.Routine) -> List[Tuple[str, object]]:
     if r.merge_node is not None:
         params.append((f"const {C_TYP[r.merge_node.prec]} *merge_buffer", "merge"))
     for s in r.static_indices:
-        params.append((f"const uint32_t {L.sym_ident(s.sym)}", s))
+        params.append((f"const {C_TYP[index_prec()]} {L.sym_ident(s.sym)}", s))
     for n in r.nodes():
         if n.mode == "ctx":
             params.append((f"{C_TYP[n.prec]} *{n.ident}", n))

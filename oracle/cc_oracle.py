@@ -88,7 +88,7 @@ class CompiledOracle:
                 v = int(static[src.sym])
                 if v < 0 or (src.range is not None and v >= src.range):
                     raise ValueError(f"static index {L.sym_ident(src.sym)}={v} out of range")
-                args.append(ctypes.c_uint32(v))
+                args.append((ctypes.c_uint64 if cc_emit.LARGE_MODELS else ctypes.c_uint32)(v))
             else:
                 args.append(ctypes.c_void_p(merge.ctypes.data))
         fn = getattr(self.lib, name)

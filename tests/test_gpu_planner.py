@@ -116,3 +116,21 @@ def test_tiny_routine_is_one_workgroup_with_identical_results():
         assert np.array_equal(one.get(w.nodes[name]), many.get(w.nodes[name])), name
         assert rel_err(one.get(w.nodes[name]), ora.get(w.nodes[name]), "single") <= 1e-5, name
     one.close(); many.close()
+
+
+def test_integer_row_sums_stay_exact():
+    # lanes share a row only through floating-point accumulators: a uint32 sum (wrapping, values far
+    # beyond 2^24) must come out bit-exact, so integer rows are walked sequentially
+    rows, cols = 96, 2048
+    L.reset_symbols(0)
+    x = L.Node(1, "x", "uint32", (rows, cols)); s = L.Node(2, "s", "uint32", (rows,))
+    i, j = L.fresh_symbol(), L.fresh_symbol()
+    r = L.Routine("usum", [L.For(i, 0, rows - 1, [L.For(j, 0, cols - 1, [
+        L.Set(s, (L.It(i),), L.Binop("add", L.Get(s, (L.It(i),)), L.Get(x, (L.It(i), L.It(j)))))])])])
+    xv = np.random.default_rng(3).integers(0, 1 << 32, size=(rows, cols), dtype=np.uint64).astype(np.uint32)
+    hip, ora = HipRun(r, {x.id: xv}), OracleRun(r, {x.id: xv})
+    hip.step(); ora.step()
+    want = xv.sum(axis=1, dtype=np.uint64).astype(np.uint32)
+    assert np.array_equal(ora.get(s), want)
+    assert np.array_equal(hip.get(s), want)
+    hip.close()
