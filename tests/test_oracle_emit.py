@@ -225,3 +225,30 @@ def test_param_order_is_by_declaration_string():
     decls = [d for d, _ in cc_emit.kernel_params(r)]
     assert decls == ["HALF_T *a_then_val", "float *where", "unsigned char *cond_condition",
                      "unsigned short *b_else_val"]
+
+
+def test_large_models_widens_loop_indices_and_integer_arguments():
+    # c_syntax.ml:111-112: `loop_index_type` and `arg_int_prefix` turn uint64_t under large_models;
+    # the results of a routine do not depend on the setting
+    import numpy as np
+    from oracle import cc_oracle
+    L.reset_symbols(0)
+    a = L.Node(1, "a", "single", (5, 7)); b = L.Node(2, "b", "single", (7,))
+    st = L.StaticSymbol(L.fresh_symbol(), 5)
+    j = L.fresh_symbol()
+    r = L.Routine("row_of", [L.For(j, 0, 6, [L.Set(b, (L.It(j),), L.Binop(
+        "add", L.Get(a, (L.It(st.sym), L.It(j))), L.EmbedIndex(L.It(j))))])], static_indices=[st])
+    av = np.arange(35, dtype=np.float32).reshape(5, 7)
+    outs = []
+    for large in (False, True):
+        cc_emit.LARGE_MODELS = large
+        try:
+            lib = cc_oracle.CompiledOracle([r])
+            typ = "uint64_t" if large else "uint32_t"
+            assert f"for ({typ} " in lib.source and f"const {typ} {L.sym_ident(st.sym)}" in lib.source
+            bufs = {a.id: av.copy(), b.id: np.zeros(7, np.float32)}
+            lib.run(r.name, bufs, {st.sym: 3})
+            outs.append(bufs[b.id])
+        finally:
+            cc_emit.LARGE_MODELS = False
+    assert np.array_equal(outs[0], av[3] + np.arange(7)) and np.array_equal(outs[0], outs[1])
