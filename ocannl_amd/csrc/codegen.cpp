@@ -632,6 +632,9 @@ void emit_phase_statements(const Routine& r, Printer& pr, const Phase& ph, int G
     if (v.kind == Scalar::Tern && v.tern == Ternop::Fma && is_self(*v.c)) { is_reduction = true; accum = Binop::Add; }
     else if (v.kind == Scalar::Bin && (v.bin == Binop::Add || v.bin == Binop::Max || v.bin == Binop::Min) &&
              (is_self(*v.a) || is_self(*v.b))) { is_reduction = true; accum = v.bin; }
+    // the accumulator lives in a register across the sequential loops only when they all update
+    // one and the same element (not so for sums of symbols on an axis, convolution-style)
+    for (auto& ix : set->idcs) for (int q : ph.seq_syms) if (ix.mentions(q)) is_reduction = false;
   }
   auto open_seq_loops = [&](std::string& cur_ind, bool coop_last) {
     for (size_t i = 0; i < ph.seq_syms.size(); ++i) {

@@ -72,8 +72,8 @@ int axis_of(const Indices& idcs, int sym) {
   for (size_t p = 0; p < idcs.size(); ++p) {
     const AxisIndex& a = idcs[p];
     if (a.kind == AxisIndex::Iter && a.sym == sym) return (int)p;
-    if (a.kind == AxisIndex::Affine && a.terms.size() == 1 && a.terms[0].second == sym && a.terms[0].first != 0)
-      return (int)p;
+    if (a.kind == AxisIndex::Affine)
+      for (auto& t : a.terms) if (t.second == sym && t.first != 0) return (int)p;
   }
   return -1;
 }
@@ -81,7 +81,29 @@ int axis_of(const Indices& idcs, int sym) {
 // A chain symbol is parallel when every array written below the chain is touched, in every access
 // (reads included), through one and the same index expression driven by that symbol on one and the
 // same axis: different values of the symbol then work on disjoint slices.
-bool symbol_is_parallel(int sym, const std::vector<Access>& acc) {
+// A sum of loop symbols on one axis (`stride * o + k`, convolution-style) sends distinct tuples of
+// symbol values to distinct positions only when the coefficients form a mixed radix over the extents:
+// sorted by magnitude, each coefficient exceeds the reach of all smaller terms together.  Symbols
+// without an extent (static indices) are constants here.
+bool affine_is_injective(const AxisIndex& e, const std::map<int, int64_t>& ext, int64_t unit_run = 1) {
+  std::vector<std::pair<int64_t, int64_t>> terms;   // (|coefficient|, extent)
+  if (unit_run > 1) terms.push_back({1, unit_run});   // a vector access covers [e, e + unit_run)
+  for (auto& t : e.terms) {
+    auto it = ext.find(t.second);
+    if (it == ext.end() || it->second <= 1) continue;
+    if (t.first == 0) return false;
+    terms.push_back({std::abs(t.first), it->second});
+  }
+  std::sort(terms.begin(), terms.end());
+  int64_t reach = 0;   // largest offset the smaller terms can add up to
+  for (auto& t : terms) {
+    if (t.first <= reach) return false;
+    reach += t.first * (t.second - 1);
+  }
+  return true;
+}
+
+bool symbol_is_parallel(int sym, const std::vector<Access>& acc, const std::map<int, int64_t>& ext) {
   std::set<int> written;
   for (auto& a : acc) if (a.write) written.insert(a.node);
   for (int w : written) {
@@ -94,11 +116,13 @@ bool symbol_is_parallel(int sym, const std::vector<Access>& acc) {
       const AxisIndex& e = (*a.idcs)[p];
       if (a.vec_len > 0 && p == (int)a.idcs->size() - 1) {
         // a vector write covers [e, e+len): needs a stride of at least len along sym
-        if (!(e.kind == AxisIndex::Affine && std::abs(e.terms[0].first) >= a.vec_len)) return false;
+        if (!(e.kind == AxisIndex::Affine && affine_is_injective(e, ext, a.vec_len))) return false;
       }
       // the symbol must not also appear on another axis of this access
       for (size_t q = 0; q < a.idcs->size(); ++q)
         if ((int)q != p && (*a.idcs)[q].mentions(sym)) return false;
+      // threads of different symbols sharing the axis must not meet on one element
+      if (a.write && e.kind == AxisIndex::Affine && !affine_is_injective(e, ext)) return false;
       if (axis < 0) { axis = p; expr = &e; }
       else if (axis != p || !(*expr == e)) return false;
     }
@@ -271,6 +295,8 @@ bool reduction_shape(const Routine& r, const Phase& ph, Binop* accum_out) {
   if (ph.inner.size() != 1 || ph.inner[0]->kind != Stmt::Set) return false;
   const Stmt& set = *ph.inner[0];
   const Scalar& v = *set.value;
+  // the accumulated element must be the same through all sequential loops
+  for (auto& ix : set.idcs) for (int q : ph.seq_syms) if (ix.mentions(q)) return false;
   auto is_self = [&](const Scalar& s) {
     return s.kind == Scalar::Get && s.node == set.node && same_indices(s.idcs, set.idcs); };
   std::function<bool(const Scalar&)> reads_lhs = [&](const Scalar& s) -> bool {
@@ -492,9 +518,22 @@ static bool analyze_nest(const Routine& r, const StmtP& sp, Phase& ph) {
   bool whole = false, foreign = false;
   std::set<ScopeId> declared;
   block_accesses(inner, acc, whole, foreign, declared);
+  std::map<int, int64_t> extents;   // of every loop symbol in the nest
+  for (const Stmt* l : chain) extents[l->sym] = l->to - l->from + 1;
+  std::function<void(const Block&)> inner_loops = [&](const Block& b) {
+    for (auto& s : b) {
+      if (s->kind == Stmt::For) { extents[s->sym] = s->to - s->from + 1; inner_loops(s->body); }
+      std::function<void(const Scalar&)> sc = [&](const Scalar& x) {
+        if (x.kind == Scalar::LocalScope) inner_loops(x.body);
+        if (x.a) sc(*x.a); if (x.b) sc(*x.b); if (x.c) sc(*x.c);
+      };
+      if (s->value) sc(*s->value);
+    }
+  };
+  inner_loops(inner);
   for (const Stmt* l : chain) {
     const int64_t ext = l->to - l->from + 1;
-    const bool par = !whole && !foreign && symbol_is_parallel(l->sym, acc);
+    const bool par = !whole && !foreign && symbol_is_parallel(l->sym, acc, extents);
     if (par) { ph.par_syms.push_back(l->sym); ph.par_from.push_back(l->from); ph.par_ext.push_back(ext); }
     else { ph.seq_syms.push_back(l->sym); ph.seq_from.push_back(l->from); ph.seq_to.push_back(l->to); }
   }
