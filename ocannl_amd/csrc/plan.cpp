@@ -522,7 +522,8 @@ static bool analyze_nest(const Routine& r, const StmtP& sp, Phase& ph) {
   for (const Stmt* l : chain) extents[l->sym] = l->to - l->from + 1;
   std::function<void(const Block&)> inner_loops = [&](const Block& b) {
     for (auto& s : b) {
-      if (s->kind == Stmt::For) { extents[s->sym] = s->to - s->from + 1; inner_loops(s->body); }
+      // (sibling loops may share a symbol, low_level.ml:2741-2775: keep the longer range)
+      if (s->kind == Stmt::For) { extents[s->sym] = std::max(extents[s->sym], s->to - s->from + 1); inner_loops(s->body); }
       std::function<void(const Scalar&)> sc = [&](const Scalar& x) {
         if (x.kind == Scalar::LocalScope) inner_loops(x.body);
         if (x.a) sc(*x.a); if (x.b) sc(*x.b); if (x.c) sc(*x.c);

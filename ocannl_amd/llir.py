@@ -468,6 +468,38 @@ def loop_over_dims(dims: Sequence[int], body) -> List[Stmt]:
     return rec([], list(dims))
 
 
+def loop_over_padding_region(dims: Sequence[int], padding: Sequence[Tuple[int, int]], body) -> List[Stmt]:
+    """``Low_level.loop_over_padding_region`` (low_level.ml:2705-2802): loops that visit exactly the
+    margin of a padded node, never its data region. ``padding[axis] = (left, right)``. Per padded
+    axis: the left strip over all remaining axes, the middle range recursing into the later axes,
+    the right strip over all remaining axes; the left strip and the middle share one symbol, the
+    right strip takes a fresh one. ``body(idcs) -> [Stmt]``."""
+    dims = list(dims)
+
+    def build(any_padding: bool, axis: int, rev_idcs) -> List[Stmt]:
+        if axis >= len(dims):
+            return body(tuple(reversed(rev_idcs))) if any_padding else []
+        dim, (left, right) = dims[axis], padding[axis]
+        index = fresh_symbol()
+        if left <= 0 and right <= 0:
+            return [For(index, 0, dim - 1, build(any_padding, axis + 1, [It(index)] + rev_idcs))]
+
+        def strip(sym):
+            return loop_over_dims(dims[axis + 1:], lambda rest: body(tuple(reversed(rev_idcs)) + (It(sym),) + tuple(rest)))
+
+        out: List[Stmt] = []
+        if left > 0:
+            out.append(For(index, 0, left - 1, strip(index)))
+        if left <= dim - right - 1:
+            out.append(For(index, left, dim - right - 1, build(any_padding, axis + 1, [It(index)] + rev_idcs)))
+        if right > 0:
+            right_index = fresh_symbol()
+            out.append(For(right_index, dim - right, dim - 1, strip(right_index)))
+        return out
+
+    return build(False, 0, [])
+
+
 # --------------------------------------------------------------------------------------
 # ``.ll`` text (low_level.ml:2544-2648)
 # --------------------------------------------------------------------------------------

@@ -107,3 +107,26 @@ def test_planner_rewrites_show_in_the_generated_source():
     r = L.Routine("colsum", [L.For(j, 0, 255, [L.For(i, 0, 4095, [
         L.Set(out, (L.It(j),), L.Binop("add", L.Get(out, (L.It(j),)), L.Get(x, (L.It(i), L.It(j)))))])])])
     assert len(B.compile(r).kernels()) == 2 and len(B.compile(r, "coop=0").kernels()) == 1
+
+
+def test_padding_region_loops_visit_exactly_the_margin():
+    # low_level.ml:2705-2802 by brute force: run the loops in Python and count visits per cell
+    import itertools
+    import numpy as np
+    for dims, padding in (((4, 5), ((1, 2), (0, 0))), ((3, 6, 5), ((0, 0), (2, 1), (1, 1))), ((5,), ((0, 3),)),
+                          ((2, 4, 4, 3), ((0, 0), (1, 1), (1, 1), (0, 0))), ((3, 3), ((0, 0), (0, 0)))):
+        L.reset_symbols(0)
+        visits = np.zeros(dims, int)
+        stmts = L.loop_over_padding_region(dims, padding, lambda idcs: [L.Set(L.Node(1, "t", "single", dims), idcs, L.Const(0.0))])
+
+        def run(body, env):
+            for st in body:
+                if isinstance(st, L.For):
+                    for v in range(st.from_, st.to + 1):
+                        run(st.body, {**env, st.sym: v})
+                else:
+                    visits[tuple(env[ix.sym] if isinstance(ix, L.It) else ix.i for ix in st.idcs)] += 1
+        run(stmts, {})
+        want = np.ones(dims, int)
+        want[tuple(slice(l, d - r) for d, (l, r) in zip(dims, padding))] = 0
+        assert np.array_equal(visits, want), (dims, padding)

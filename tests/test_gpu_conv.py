@@ -88,3 +88,54 @@ def test_overlapping_windows_are_not_spread_over_threads():
             assert threads > b * ic
         else:
             assert threads == b * ic
+
+
+def _padded_same_conv(b=2, h=7, w=6, ic=3, oc=5, ksz=3, neutral=0.0):
+    L.reset_symbols(0)
+    pad = ksz // 2
+    padding = ((0, 0), (pad, pad), (pad, pad), (0, 0))
+    xp = L.Node(1, "x_padded", "single", (b, h + 2 * pad, w + 2 * pad, ic))
+    wt = L.Node(2, "w", "single", (oc, ksz, ksz, ic))
+    y = L.Node(3, "y", "single", (b, h, w, oc))
+    mp = L.Node(4, "maxpool", "single", (b, h, w, ic))
+    body = [L.Comment("reset padding margins of x_padded")]
+    body += L.loop_over_padding_region(xp.dims, padding, lambda idcs: [L.Set(xp, idcs, L.Const(neutral))])
+    s = [L.fresh_symbol() for _ in range(7)]
+    bb, o1, o2, c, k1, k2, i = s
+    xi = (L.It(bb), L.Affine(((1, o1), (1, k1)), 0), L.Affine(((1, o2), (1, k2)), 0), L.It(i))
+    yi = (L.It(bb), L.It(o1), L.It(o2), L.It(c))
+    nest = [L.Set(y, yi, L.Ternop("fma", L.Get(xp, xi), L.Get(wt, (L.It(c), L.It(k1), L.It(k2), L.It(i))), L.Get(y, yi)))]
+    for sym, ext in reversed(list(zip(s, (b, h, w, oc, ksz, ksz, ic)))):
+        nest = [L.For(sym, 0, ext - 1, nest)]
+    body += [L.ZeroOut(y)] + nest
+    s = [L.fresh_symbol() for _ in range(6)]
+    bb, o1, o2, i, k1, k2 = s
+    pi = (L.It(bb), L.It(o1), L.It(o2), L.It(i))
+    xi = (L.It(bb), L.Affine(((1, o1), (1, k1)), 0), L.Affine(((1, o2), (1, k2)), 0), L.It(i))
+    pb = [L.Set(mp, pi, L.Binop("max", L.Get(mp, pi), L.Get(xp, xi)))]
+    for sym, ext in reversed(list(zip(s, (b, h, w, ic, ksz, ksz)))):
+        pb = [L.For(sym, 0, ext - 1, pb)]
+    body += L.loop_over_dims(mp.dims, lambda idcs: [L.Set(mp, idcs, L.Const(float("-inf")))]) + pb
+    return L.Routine("same_conv", body), xp, wt, y, mp, pad
+
+
+@pytest.mark.parametrize("neutral", [0.0, float("-inf")])
+@pytest.mark.parametrize("options", ["mfma=0;coop=0;serial=0", None])
+def test_padded_node_margins_are_reset_before_a_same_convolution(neutral, options):
+    # the margin of a padded node is reset to the operation's neutral value by loops that visit
+    # only the margin (assignments.ml:281-298); accesses carry the left padding as an offset (:202-218)
+    r, xp, wt, y, mp, pad = _padded_same_conv(neutral=neutral)
+    rng = np.random.default_rng(5)
+    xv = rng.uniform(-1, 1, xp.dims).astype(np.float32)      # margins start as garbage
+    init = {xp.id: xv, wt.id: rng.uniform(-1, 1, wt.dims).astype(np.float32)}
+    hip, ora = HipRun(r, init, options), OracleRun(r, init)
+    hip.step(); ora.step()
+    got = hip.get(xp)
+    assert np.array_equal(got, ora.get(xp))
+    assert np.array_equal(got[:, pad:-pad, pad:-pad, :], xv[:, pad:-pad, pad:-pad, :])      # data untouched
+    margin = np.ones(xp.dims, bool); margin[:, pad:-pad, pad:-pad, :] = False
+    assert np.all(got[margin] == np.float32(neutral))
+    assert np.array_equal(hip.get(mp), ora.get(mp))
+    if neutral == 0.0:
+        assert np.allclose(hip.get(y), ora.get(y), rtol=1e-5, atol=1e-5)
+    hip.close()
