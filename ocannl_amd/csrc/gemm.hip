@@ -61,9 +61,6 @@ __device__ long long g_gemm_stamps[8 * 4096];
 #define OCANNL_PROBE_SKIP(bit) 0
 #endif
 
-#ifndef OCANNL_GEMM_DEEP_PREFETCH
-#define OCANNL_GEMM_DEEP_PREFETCH 0   // 1: two global-load register sets for bf16 sources
-#endif
 
 constexpr int kThreads = 256;
 constexpr int kBK = 64;        // K elements per stage (bf16 compute)
@@ -307,9 +304,13 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, f32x16 (&acc)[TM][TN
 
 // One wavefront per SIMD for the 256x256 tile (the 256 accumulator registers live in AGPRs and the
 // whole 512-register budget is available); two for the 128x128 tile.
-template <int BM, int BN, typename AT, typename BT, bool A_KC, bool B_KC>
+// PF = 2: global loads run two K stages ahead in two register sets, for launches of at most one
+// workgroup per CU, where nothing else hides the HBM latency of a stage; that needs the whole
+// register file, so one wavefront per SIMD.
+template <int BM, int BN, typename AT, typename BT, bool A_KC, bool B_KC, int PF>
 __global__ void __launch_bounds__(kThreads)
-__attribute__((amdgpu_waves_per_eu((BM < 256 && sizeof(AT) == 2 && sizeof(BT) == 2) ? 2 : 1, BM >= 256 ? 1 : 2)))
+__attribute__((amdgpu_waves_per_eu((BM < 256 && sizeof(AT) == 2 && sizeof(BT) == 2 && PF == 1) ? 2 : 1,
+                                   (BM >= 256 || PF > 1) ? 1 : 2)))
 gemm_bf16_kernel(const GemmArgs g) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int kAT = lds_tile_elems<BM, A_KC>(), kBT = lds_tile_elems<BN, B_KC>();   // one stage of each operand
@@ -359,10 +360,9 @@ gemm_bf16_kernel(const GemmArgs g) {
   const long ksteps = kend > kbeg ? (kend - kbeg + kBK - 1) / kBK : 0;
 
   // Software pipeline.  LDS is double buffered; global loads run kPF tiles ahead of the tile being
-  // multiplied, held in kPF register sets.  The code is written for one or two sets; two were
-  // measured slower for both tile sizes (the second set spills next to the double-buffered
-  // fragments), so one it is unless OCANNL_GEMM_DEEP_PREFETCH is defined.
-  constexpr int kPF = (OCANNL_GEMM_DEEP_PREFETCH && sizeof(AT) == 2 && sizeof(BT) == 2) ? 2 : 1;
+  // multiplied, held in kPF register sets (one or two).
+  constexpr int kPF = PF;
+  static_assert(PF == 1 || (PF == 2 && sizeof(AT) == 2 && sizeof(BT) == 2), "two register sets: bf16 sources only");
   Stager<BM, AT, A_KC> sa[kPF];
   Stager<BN, BT, B_KC> sb[kPF];
   sa[0].load(A, lda, m0, kbeg, g.M, kend, tid);
@@ -685,7 +685,7 @@ long batch_count(const GemmDesc& d) {
 }
 
 #ifdef OCANNL_GEMM_TIMING
-int g_force_tile = 0, g_force_splits = 0;   // tuning overrides of the probe build
+int g_force_tile = 0, g_force_splits = 0, g_force_prefetch = 0;   // tuning overrides of the probe build
 #endif
 
 // Tile size and split-K factor, from a measured sweep on MI355X (bf16 operands).  256x256 tiles
@@ -694,7 +694,7 @@ int g_force_tile = 0, g_force_splits = 0;   // tuning overrides of the probe bui
 // runs 128x128 tiles, two workgroups per CU, and when those are fewer than 256 K is split
 // towards ~512 workgroups, never below 8 K stages per split.  Splits are summed in index order by
 // splitk_reduce_kernel (deterministic).
-struct TileConfig { bool big; int splits; };
+struct TileConfig { bool big; int splits; int prefetch; };
 
 TileConfig tile_config(const GemmDesc& d) {
   const long nb = batch_count(d);
@@ -714,11 +714,19 @@ TileConfig tile_config(const GemmDesc& d) {
   if (g_force_tile) c.big = g_force_tile == 256;
   if (g_force_splits) c.splits = g_force_splits;
 #endif
+  // two stages of global loads in flight when the launch puts at most one workgroup on a CU and
+  // each runs at least 8 K stages (measured: 8192x512x2048 bf16 595 -> 738 TFLOP/s)
+  const bool bf16_sources = d.a.prec == Prec::Bfloat16 && d.b.prec == Prec::Bfloat16;
+  c.prefetch = (!c.big && bf16_sources && t128 * c.splits <= 256 && d.K / c.splits >= 512) ? 2 : 1;
+#ifdef OCANNL_GEMM_TIMING
+  if (g_force_prefetch) c.prefetch = (!c.big && bf16_sources) ? g_force_prefetch : 1;
+#endif
   return c;
 }
 
 bool big_tile(const GemmDesc& d) { return tile_config(d).big; }
 int split_count(const GemmDesc& d) { return tile_config(d).splits; }
+int prefetch_depth(const GemmDesc& d) { return tile_config(d).prefetch; }
 
 template <typename K>
 hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t s, hipEvent_t after_main) {
@@ -745,12 +753,12 @@ hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t
   return hipGetLastError();
 }
 
-template <int BM, int BN, typename AT, typename BT>
+template <int BM, int BN, typename AT, typename BT, int PF = 1>
 hipError_t launch_bf16_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t s, hipEvent_t ev) {
-  if (akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, true>, bf16_smem<BM, BN, true, true>(), BM, BN, a, s, ev);
-  if (akc && !bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, false>, bf16_smem<BM, BN, true, false>(), BM, BN, a, s, ev);
-  if (!akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, true>, bf16_smem<BM, BN, false, true>(), BM, BN, a, s, ev);
-  return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, false>, bf16_smem<BM, BN, false, false>(), BM, BN, a, s, ev);
+  if (akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, true, PF>, bf16_smem<BM, BN, true, true>(), BM, BN, a, s, ev);
+  if (akc && !bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, false, PF>, bf16_smem<BM, BN, true, false>(), BM, BN, a, s, ev);
+  if (!akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, true, PF>, bf16_smem<BM, BN, false, true>(), BM, BN, a, s, ev);
+  return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, false, PF>, bf16_smem<BM, BN, false, false>(), BM, BN, a, s, ev);
 }
 
 template <int BM, int BN>
@@ -775,8 +783,8 @@ const char* gemm_kernel_name(const GemmDesc& d) {
   if (af && bf)
     snprintf(buf, sizeof buf, "gemm_f32_kernel<%d, %d, %s, %s>", tile, tile, tf[a_kcontig(d)], tf[b_kcontig(d)]);
   else
-    snprintf(buf, sizeof buf, "gemm_bf16_kernel<%d, %d, %s, %s, %s, %s>", tile, tile, af ? "float" : "unsigned short",
-             bf ? "float" : "unsigned short", tf[a_kcontig(d)], tf[b_kcontig(d)]);
+    snprintf(buf, sizeof buf, "gemm_bf16_kernel<%d, %d, %s, %s, %s, %s, %d>", tile, tile, af ? "float" : "unsigned short",
+             bf ? "float" : "unsigned short", tf[a_kcontig(d)], tf[b_kcontig(d)], prefetch_depth(d));
   return buf;
 }
 
@@ -808,9 +816,11 @@ hipError_t launch_gemm(const GemmDesc& d, const GemmArgs& a_in, void* workspace,
   }
   const bool af = d.a.prec == Prec::Single, bf = d.b.prec == Prec::Single;
   if (af && bf) return big ? launch_f32_layout<256, 256>(akc, bkc, a, s, ev) : launch_f32_layout<128, 128>(akc, bkc, a, s, ev);
-  if (!af && !bf)
-    return big ? launch_bf16_layout<256, 256, unsigned short, unsigned short>(akc, bkc, a, s, ev)
-               : launch_bf16_layout<128, 128, unsigned short, unsigned short>(akc, bkc, a, s, ev);
+  if (!af && !bf) {
+    if (big) return launch_bf16_layout<256, 256, unsigned short, unsigned short>(akc, bkc, a, s, ev);
+    return prefetch_depth(d) == 2 ? launch_bf16_layout<128, 128, unsigned short, unsigned short, 2>(akc, bkc, a, s, ev)
+                                  : launch_bf16_layout<128, 128, unsigned short, unsigned short>(akc, bkc, a, s, ev);
+  }
   if (af && !bf)
     return big ? launch_bf16_layout<256, 256, float, unsigned short>(akc, bkc, a, s, ev)
                : launch_bf16_layout<128, 128, float, unsigned short>(akc, bkc, a, s, ev);
