@@ -692,7 +692,7 @@ int g_force_tile = 0, g_force_splits = 0, g_force_prefetch = 0;   // tuning over
 // (one workgroup per CU) win only when the output alone gives >= 256 of them and K runs at least
 // 8 stages (below that a launch is all prologue and epilogue); anything else
 // runs 128x128 tiles, two workgroups per CU, and when those are fewer than 256 K is split
-// towards ~512 workgroups, never below 8 K stages per split.  Splits are summed in index order by
+// towards ~512 workgroups (~256 for bf16 sources), never below 8 K stages per split.  Splits are summed in index order by
 // splitk_reduce_kernel (deterministic).
 struct TileConfig { bool big; int splits; int prefetch; };
 
@@ -701,12 +701,16 @@ TileConfig tile_config(const GemmDesc& d) {
   const long t256 = ((d.M + 255) / 256) * ((d.N + 255) / 256) * nb;
   const long t128 = ((d.M + 127) / 128) * ((d.N + 127) / 128) * nb;
   TileConfig c;
+  const bool bf16_sources = d.a.prec == Prec::Bfloat16 && d.b.prec == Prec::Bfloat16;
   if (t256 >= 256 && d.M > 128 && d.N > 128 && d.K >= 512) { c.big = true; c.splits = 1; }
   else {
     c.big = false;
     long s = 1;
+    // bf16 sources: towards one workgroup per CU, which then loads two stages ahead (below);
+    // otherwise towards two per CU
+    const long target = bf16_sources ? 256 : 512;
     if (t128 < 256) {
-      while (s * 2 * t128 <= 512 && s * 2 <= d.K / 512 && s < 64) s *= 2;
+      while (s * 2 * t128 <= target && s * 2 <= d.K / 512 && s < 64) s *= 2;
     }
     c.splits = (int)s;
   }
@@ -716,7 +720,6 @@ TileConfig tile_config(const GemmDesc& d) {
 #endif
   // two stages of global loads in flight when the launch puts at most one workgroup on a CU and
   // each runs at least 8 K stages (measured: 8192x512x2048 bf16 595 -> 738 TFLOP/s)
-  const bool bf16_sources = d.a.prec == Prec::Bfloat16 && d.b.prec == Prec::Bfloat16;
   c.prefetch = (!c.big && bf16_sources && t128 * c.splits <= 256 && d.K / c.splits >= 512) ? 2 : 1;
 #ifdef OCANNL_GEMM_TIMING
   if (g_force_prefetch) c.prefetch = (!c.big && bf16_sources) ? g_force_prefetch : 1;

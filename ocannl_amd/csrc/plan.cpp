@@ -452,7 +452,10 @@ void account_bytes(const Routine& r, Phase& ph) {
   block_accesses(ph.inner, acc, w, f, d);
   std::set<std::pair<int, std::string>> seen;
   double bytes = 0;
+  // an accumulation whose zero fill was folded in starts from zero: its target is not read
+  const int unread = ph.fused_zero_init && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set ? ph.inner[0]->node : -1;
   for (auto& a : acc) {
+    if (!a.write && a.node == unread) continue;
     std::set<int> syms;
     std::string key = a.write ? "w" : "r";
     for (auto& ix : *a.idcs) {
@@ -1054,8 +1057,9 @@ void group_rows(const Routine& r, Plan& plan) {
       for (auto& m : run) {
         std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
         block_accesses(m.inner, acc, w, f, d);
+        const int unread = m.fused_zero_init && m.inner.size() == 1 && m.inner[0]->kind == Stmt::Set ? m.inner[0]->node : -1;
         for (auto& a : acc)
-          if (!a.write && !produced.count(a.node) && counted_r.insert(a.node).second) bytes += touched(m, a);
+          if (!a.write && a.node != unread && !produced.count(a.node) && counted_r.insert(a.node).second) bytes += touched(m, a);
         for (auto& a : acc)
           if (a.write) { produced.insert(a.node); if (counted_w.insert(a.node).second) bytes += touched(m, a); }
       }
