@@ -957,9 +957,10 @@ bool row_member(const Routine& r, Phase& ph, RowShape& shape, bool first) {
     ph.row_role = Phase::RowScalar; ph.row_outer_syms = syms; ph.row_sym = -1;
     return true;
   }
-  if (ext.size() < 2) return false;                                           // pointwise over rows x T
+  if (ext.empty()) return false;                                              // pointwise over rows x T
   const int64_t T = ext.back();
-  if (!outer_matches(ext.size() - 1) || (shape.len >= 0 && shape.len != T) || T < 16) return false;
+  // (short rows leave lanes idle: the caller takes such a group only when it is launch-bound anyway)
+  if (!outer_matches(ext.size() - 1) || (shape.len >= 0 && shape.len != T) || T < 2) return false;
   // the row position must be the unit-stride axis of the store
   if (get_stride(strides_of(r, ph.inner[0]->node, ph.inner[0]->idcs), syms.back()) != 1) return false;
   ph.row_role = Phase::RowPointwise;
@@ -1010,6 +1011,9 @@ struct RowDeps {
 };
 
 void group_rows(const Routine& r, Plan& plan) {
+  double routine_bytes = 0;
+  for (auto& ph : plan.phases) routine_bytes += ph.bytes;
+  const bool launch_bound = routine_bytes < 8e6;
   std::vector<Phase> out;
   size_t i = 0;
   while (i < plan.phases.size()) {
@@ -1030,7 +1034,10 @@ void group_rows(const Routine& r, Plan& plan) {
     // a group must know its row length and be worth a launch of its own
     int64_t rows = 1;
     for (auto e : shape.outer) rows *= e;
-    if (run.size() >= 2 && shape.len >= 16 && rows * shape.len >= (1 << 16)) {
+    // ... or sit in a routine so small that launches are all there is to save (in a large routine
+    // such a group was measured slower than its members as separate, overlapping launches)
+    const int64_t points = rows * std::max<int64_t>(shape.len, 1);
+    if (run.size() >= 2 && shape.len >= 2 && ((shape.len >= 16 && points >= (1 << 16)) || (launch_bound && points < 8192))) {
       Phase g;
       g.kind = Phase::Generic;
       g.label = run.front().label + " .. " + run.back().label;
