@@ -627,7 +627,9 @@ static void devirtualise(Routine& r, const StmtP& sp, const PlanOptions& opt, Pl
     Node t;
     t.id = new_id;
     t.ident = "ctr" + std::to_string(new_id) + "_" + r.node(ls->scope.node).ident;
-    t.prec = Prec::Single;
+    // a bf16 scalar is rounded by the serial code after every step; the scratch tensor keeps that
+    // precision (rounded once, from the fp32 accumulator) and half the traffic
+    t.prec = r.node(ls->scope.node).prec == Prec::Bfloat16 ? Prec::Bfloat16 : Prec::Single;
     t.mode = Mode::Local;
     for (const Stmt* l : dep) t.dims.push_back(l->to + 1);
     if (t.dims.empty()) t.dims.push_back(1);
