@@ -46,15 +46,13 @@ struct half8_t { _Float16 v[8]; };
 
 // ---- bf16 / fp8 ---------------------------------------------------------------------------------
 OCN_DEV float bfloat16_to_single(unsigned short b) { return __uint_as_float(((uint32_t)b) << 16); }
-// Round to nearest even.  The host does it through an integer add that does not special-case NaN
-// (builtins.c:620-627); for every other input that is exactly what the hardware conversion
-// (v_cvt_pk_bf16_f32) computes, so only NaN takes the integer path.
+// Round to nearest even through the integer add of the host code (builtins.c:620-627), NaN
+// included: three VALU operations (bit extract, three-operand add, shift), and the shift folds into
+// the mask of a following bfloat16_to_single.  (The hardware conversion gives the same bits for every
+// non-NaN input but needs a NaN guard around it to stay exact, which costs more than it saves.)
 OCN_DEV unsigned short single_to_bfloat16(float f) {
-  if (f != f) {
-    const uint32_t w = __float_as_uint(f);
-    return (unsigned short)((w + 0x7FFFu + ((w >> 16) & 1u)) >> 16);
-  }
-  return __builtin_bit_cast(unsigned short, (__bf16)f);
+  const uint32_t w = __float_as_uint(f);
+  return (unsigned short)((w + 0x7FFFu + ((w >> 16) & 1u)) >> 16);
 }
 OCN_DEV float fp8_to_single(unsigned char v) {
   if (v == 0) return 0.0f;
