@@ -1,0 +1,154 @@
+"""Every scalar operation of the op tables (arrayjit/lib/ops.ml:579-863) in every precision the
+generated kernels compute in, against the CPU checker on the same operands. Arithmetic, comparisons,
+gates, selections, conversions: bit for bit. libm functions: within a few units in the last place of
+the destination precision (two different libm implementations)."""
+import numpy as np
+import pytest
+
+from ocannl_amd import llir as L
+from ocannl_amd import workloads as W
+from parity import HipRun, OracleRun
+
+pytestmark = pytest.mark.gpu
+
+FLOATS = ("single", "double", "bfloat16", "half")
+INTS = ("int32", "uint32", "byte", "uint16", "int64", "uint64")
+EXACT_UN = ("id", "relu", "sat01", "neg", "trunc", "not", "sqrt", "recip")
+LIBM_UN = ("exp", "log", "exp2", "log2", "sin", "cos", "tanh", "recip_sqrt")
+EXACT_BIN = ("arg1", "arg2", "add", "sub", "mul", "div", "relu_gate", "sat01_gate", "max", "min", "lt", "eq", "ne", "or", "and")
+N = 512
+
+
+def _operands(prec, rng):
+    if prec in FLOATS:
+        special = np.array([0.0, -0.0, 1.0, -1.0, 0.5, -0.5, 2.0, -2.5, 1e-3, -1e-3, 100.0, -100.0, 3.14159, 0.999, 1.001,
+                            7.0, 0.25, 1.5, -3.0, 16.0], np.float64)
+        a = np.concatenate([special, rng.uniform(-4, 4, N - special.size)])
+        b = np.concatenate([special[::-1], rng.uniform(-4, 4, N - special.size)])
+        b[b == 0] = 0.75                                   # divisors
+        p = np.abs(rng.uniform(0.05, 8, N))
+        conv = lambda x: W.as_prec(x.astype(np.float32), prec) if prec != "double" else x.astype(np.float64)
+        return conv(a), conv(b), conv(p)
+    info = np.iinfo(cc_dtype(prec))
+    lo, hi = (0, min(info.max, 200)) if info.min == 0 else (-100, 100)
+    a = rng.integers(lo, hi, N).astype(cc_dtype(prec))
+    b = rng.integers(lo, hi, N).astype(cc_dtype(prec))
+    b[b == 0] = 3
+    p = rng.integers(1, 50, N).astype(cc_dtype(prec))
+    return a, b, p
+
+
+def cc_dtype(prec):
+    from oracle import cc_oracle
+    return cc_oracle.NP_DTYPE[prec]
+
+
+def _routine(prec, ops):
+    L.reset_symbols(0)
+    ident = [0]
+    def node(name, pr=prec):
+        ident[0] += 1
+        return L.Node(ident[0], name, pr, (N,))
+    a, b, p = node("a"), node("b"), node("p")
+    outs, body = {}, []
+    for kind, op in ops:
+        o = node(f"out_{kind}_{op}")
+        i = L.fresh_symbol()
+        ix = (L.It(i),)
+        ga, gb, gp = L.Get(a, ix), L.Get(b, ix), L.Get(p, ix)
+        if kind == "un":
+            arg = gp if op in ("log", "log2", "sqrt", "recip_sqrt", "recip") else ga
+            v = L.Unop(op, arg)
+        elif kind == "bin":
+            v = L.Binop(op, gp if op == "pow" else ga, gb)
+        else:
+            v = L.Ternop(op, ga, gb, gp)
+        body.append(L.For(i, 0, N - 1, [L.Set(o, ix, v)]))
+        outs[(kind, op)] = o
+    return L.Routine(f"ops_{prec}", body), (a, b, p), outs
+
+
+def _ulps(got, want, prec):
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    eps = {"single": 2.0 ** -23, "double": 2.0 ** -52, "bfloat16": 2.0 ** -7, "half": 2.0 ** -10}[prec]
+    with np.errstate(invalid="ignore", divide="ignore"):
+        same = (g == w) | (np.isnan(g) & np.isnan(w))
+        err = np.where(same, 0.0, np.abs(g - w) / (eps * np.maximum(np.abs(w), 2.0 ** -20)))
+    return float(np.nanmax(err))
+
+
+@pytest.mark.parametrize("prec", FLOATS + INTS)
+def test_operations_match_the_checker(prec):
+    rng = np.random.default_rng(11)
+    ops = [("un", o) for o in EXACT_UN] + [("bin", o) for o in EXACT_BIN] + [("tern", o) for o in ("where", "fma", "mul3")]
+    if prec in FLOATS:
+        ops += [("un", o) for o in LIBM_UN] + [("bin", "pow")]
+    else:
+        ops = [x for x in ops if x[1] not in ("sqrt", "recip", "sat01", "sat01_gate")] + [("bin", "mod")]
+    r, (a, b, p), outs = _routine(prec, ops)
+    av, bv, pv = _operands(prec, rng)
+    init = {a.id: av, b.id: bv, p.id: pv}
+    hip, ora = HipRun(r, init, "serial=0"), OracleRun(r, init)
+    hip.step(); ora.step()
+    report = []
+    for (kind, op), o in outs.items():
+        got, want = hip.get(o), ora.get(o)
+        if prec == "bfloat16":                 # as values: fmax(0.0, -0.0) may be either zero (IEEE 754 leaves it open)
+            got, want = W.to_float(got, prec), W.to_float(want, prec)
+        # `a * b * c` on _Float16 operands: rounded after each product by hardware with half arithmetic
+        # (the GPU, x86 with AVX512-FP16), once by a host compiler that evaluates in float: one ulp apart
+        loose = op in LIBM_UN + ("pow",) or (prec == "half" and op == "mul3")
+        if prec in INTS or not loose:
+            same = (got == want) | ((got != got) & (want != want)) if prec in FLOATS else (got == want)
+            if not np.all(same):
+                k = int(np.argmin(same))
+                report.append((op, "exact", int((~same).sum()), got[k], want[k], av[k], bv[k], pv[k]))
+        else:
+            # tanh is spelled tanhf in every precision (ops.ml:769): single-precision results in double too
+            u = _ulps(got, want, "single" if (prec == "double" and op == "tanh") else prec)
+            if u > 4.0:
+                report.append((op, "ulps", u))
+    hip.close()
+    assert not report, report
+
+
+CAST_PRECS = ("single", "double", "bfloat16", "half", "fp8", "int32", "uint32", "byte", "uint16", "int64", "uint64")
+
+
+def _cast_values(prec, rng):
+    from oracle import cc_oracle
+    n = 256
+    if prec in ("single", "double", "bfloat16", "half"):
+        v = np.concatenate([np.arange(0, 32, 0.25), rng.uniform(0, 100, n - 128)])
+        return W.as_prec(v.astype(np.float32), prec) if prec != "double" else v.astype(np.float64)
+    if prec == "fp8":
+        return rng.integers(0, 0x70, n).astype(np.uint8)       # positive finite e5m2 patterns
+    return rng.integers(0, 100, n).astype(cc_oracle.NP_DTYPE[prec])
+
+
+@pytest.mark.parametrize("dst", CAST_PRECS)
+def test_conversions_between_precisions(dst):
+    # out<dst>[i] = a<src>[i] and out<dst>[i] = a<src>[i] + b<dst>[i] for every source precision: the
+    # conversion tables (ops.ml:688-796 spellings, cc_backend.ml:155-323 for bf16 / half / fp8)
+    rng = np.random.default_rng(5)
+    L.reset_symbols(0)
+    n, ident, body, init, outs = 256, [0], [], {}, []
+    def node(name, pr):
+        ident[0] += 1
+        return L.Node(ident[0], name, pr, (n,))
+    b = node("b", dst)
+    init[b.id] = _cast_values(dst, rng)
+    for src in CAST_PRECS:
+        a = node(f"a_{src}", src)
+        init[a.id] = _cast_values(src, rng)
+        o1, o2 = node(f"cast_{src}", dst), node(f"sum_{src}", dst)
+        i, j = L.fresh_symbol(), L.fresh_symbol()
+        body.append(L.For(i, 0, n - 1, [L.Set(o1, (L.It(i),), L.Get(a, (L.It(i),)))]))
+        body.append(L.For(j, 0, n - 1, [L.Set(o2, (L.It(j),), L.Binop("add", L.Get(a, (L.It(j),)), L.Get(b, (L.It(j),))))]))
+        outs += [o1, o2]
+    r = L.Routine(f"casts_to_{dst}", body)
+    hip, ora = HipRun(r, init, "serial=0"), OracleRun(r, init)
+    hip.step(); ora.step()
+    bad = [(o.ident, int((hip.get(o) != ora.get(o)).sum())) for o in outs if not np.array_equal(hip.get(o), ora.get(o))]
+    hip.close()
+    assert not bad, bad
