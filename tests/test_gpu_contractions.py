@@ -119,3 +119,35 @@ def test_split_k_is_deterministic():
         outs.append(hip.get(C).copy())
         hip.close()
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+@pytest.mark.parametrize("prec", ["single", "bfloat16"])
+def test_operands_sliced_by_static_and_fixed_indices(prec):
+    # c[s2, m, n] = sum_k a[s1, m, k] * b[3, k, n]: one operand slice is chosen at run time by a
+    # static index (a kernel-launch argument folded into the operand's base address), one by a fixed
+    # position, and the result goes to a run-time slice too
+    S, M, N, K = 4, 192, 160, 256
+    L.reset_symbols(0)
+    A = L.Node(1, "a", prec, (S, M, K)); B = L.Node(2, "b", prec, (5, K, N)); C = L.Node(3, "c", "single", (S, M, N))
+    s1, s2 = L.StaticSymbol(L.fresh_symbol(), S), L.StaticSymbol(L.fresh_symbol(), S)
+    m, n, k = (L.fresh_symbol() for _ in range(3))
+    ci = (L.It(s2.sym), L.It(m), L.It(n))
+    nest = L.For(m, 0, M - 1, [L.For(n, 0, N - 1, [L.For(k, 0, K - 1, [L.Set(C, ci, L.Ternop(
+        "fma", L.Get(A, (L.It(s1.sym), L.It(m), L.It(k))), L.Get(B, (L.Fixed(3), L.It(k), L.It(n))), L.Get(C, ci)))])])])
+    r = L.Routine("sliced", [nest], static_indices=[s1, s2])
+    rng = np.random.default_rng(2)
+    av, bv = (rng.standard_normal(x.dims).astype(np.float32) for x in (A, B))
+    init = {1: W.as_prec(av, prec), 2: W.as_prec(bv, prec)}
+    hip = HipRun(r, init, "min_mfma_flops=1")
+    assert [k["kind"] for k in hip.code.kernels()] == ["mfma"]
+    a64, b64 = W.to_float(init[1], prec).astype(np.float64), W.to_float(init[2], prec).astype(np.float64)
+    want = np.zeros(C.dims)
+    for va, vc in ((0, 1), (3, 1), (2, 0)):          # accumulates: slice 1 of c receives two products
+        hip.step({s1.sym: va, s2.sym: vc})
+        want[vc] += a64[va] @ b64[3]
+    got = hip.get(C).astype(np.float64)
+    assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
+    assert not got[2:].any()
+    with pytest.raises(hip.B.User_error):
+        hip.step({s1.sym: S, s2.sym: 0})             # out of range: refused before anything is enqueued
+    hip.close()
