@@ -114,3 +114,30 @@ def test_full_size_transformer_step_properties():
         assert _err(W.to_float(a, n.prec), W.to_float(p, n.prec).astype(np.float64), n.prec) <= 2e-2, name
     for h in runs + [plain]:
         h.close()
+
+
+def test_full_size_attention_against_torch_autograd():
+    # benchmark configuration 5 at its real size (b=16 h=16 q=k=1024 d=64, bf16 values, fp32 grads)
+    # against plain PyTorch in fp32 on the same device: softmax(Q K^T / sqrt(d)) V and, through
+    # autograd, dQ dK dV from the same d out. bf16 storage of scores / probabilities bounds the
+    # agreement (Frobenius-relative 2e-2, as for every bf16 routine); rows of the soft-max sum to one.
+    import torch
+    w = W.attention()
+    hip = HipRun(w.routine, w.init)
+    hip.step()
+    dev = torch.device("cuda:0")
+    f32 = lambda name: torch.tensor(W.to_float(w.init[w.nodes[name].id], w.nodes[name].prec).astype(np.float32), device=dev)
+    q, k, v = (f32(n).requires_grad_(True) for n in ("q", "k", "v"))
+    dout = f32("dout")
+    scores = torch.einsum("bshd,bthd->bsht", q, k) / float(np.sqrt(64.0))
+    attn = torch.softmax(scores, dim=-1)
+    out = torch.einsum("bsht,bthe->bshe", attn, v)
+    out.backward(dout)
+    def rel(name, ref):
+        got = torch.tensor(W.to_float(hip.get(w.nodes[name]), w.nodes[name].prec).astype(np.float32), device=dev)
+        return float(torch.linalg.norm(got - ref) / torch.linalg.norm(ref))
+    errs = {"out": rel("out", out.detach()), "dq": rel("dq", q.grad), "dk": rel("dk", k.grad), "dv": rel("dv", v.grad)}
+    assert all(e <= 2e-2 for e in errs.values()), errs
+    sums = W.to_float(hip.get(w.nodes["attn"]), w.nodes["attn"].prec).reshape(-1, 1024)[::997].sum(axis=1)
+    assert np.all(np.abs(sums - 1.0) < 2e-2), (sums.min(), sums.max())
+    hip.close()
