@@ -91,8 +91,8 @@ def test_full_size_transformer_step_properties():
     # copies) and a plan without any of them (`mfma=0;rows=0;bf16_copies=0`: one generated kernel per
     # statement, contractions as per-element loops) agree to the bf16 bar on the loss and on updated
     # parameters. (c) The first loss of a randomly initialised model is ln(vocabulary). (With `coop=0`
-    # as well the bf16 batch-loss sum over 8192 tokens is rounded after every addition, as in the
-    # serial C code, stalls, and reads 6.24 instead of 8.32: the documented case where lanes sharing a
+    # as well the bf16 soft-max denominator over 4096 logits is rounded after every addition, as in the
+    # serial C code, stalls at 256, and the loss reads 6.24 instead of 8.32: the documented case where lanes sharing a
     # reduction in fp32 are closer to the mathematics than the reference's order.)
     w = W.transformer()
     runs = [HipRun(w.routine, w.init) for _ in range(2)]
