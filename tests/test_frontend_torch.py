@@ -106,3 +106,29 @@ def test_char_mlp_adam_step_of_the_harness_equals_pytorch():
         a, b = ora.get(w.nodes[k]), p.detach().numpy()
         assert np.max(np.abs(a - b)) <= 1e-4 * max(1.0, float(np.max(np.abs(b)))), k
         assert np.allclose(ora.get(w.nodes["m_" + k]), M[k].numpy(), rtol=1e-3, atol=1e-7), k
+
+
+def test_moons_sgd_momentum_step_of_the_harness_equals_pytorch():
+    # benchmark configuration 1: MLP 2->16->16->1, hinge loss mean relu(1 - y f(x)), Train.sgd_one with
+    # momentum (lib/train.ml:76-90): delta = g + wd p; m = mu m + delta; p -= lr m -- which is
+    # torch.optim.SGD(momentum=mu, dampening=0)
+    w = W.moons_mlp()
+    data = torch.tensor(np.array(w.init[w.nodes["data"].id])); cls = torch.tensor(np.array(w.init[w.nodes["classes"].id]))
+    P = {k: torch.tensor(np.array(w.init[w.nodes[k].id]), requires_grad=True) for k in ("w1", "b1", "w2", "b2", "w3")}
+    opt = torch.optim.SGD(list(P.values()), lr=0.1, momentum=0.9)
+    ora = OracleRun(w.routine, w.init)
+    sym = w.statics["batch_n"].sym
+    for step in range(6):
+        n = step % w.statics["batch_n"].range
+        ora.step({sym: n})
+        opt.zero_grad()
+        h1 = torch.relu(data[n] @ P["w1"].t() + P["b1"])
+        h2 = torch.relu(h1 @ P["w2"].t() + P["b2"])
+        f = (h2 @ P["w3"].t())[:, 0]
+        loss = torch.relu(1.0 - cls[n] * f).mean()
+        loss.backward()
+        opt.step()
+        assert abs(float(ora.get(w.nodes["loss"])[0]) - float(loss.detach())) <= 2e-5 * max(1.0, float(loss.detach())), step
+    for k, p in P.items():
+        a, b = ora.get(w.nodes[k]), p.detach().numpy()
+        assert np.max(np.abs(a - b)) <= 1e-4 * max(1.0, float(np.max(np.abs(b)))), k
