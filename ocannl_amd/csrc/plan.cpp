@@ -252,6 +252,11 @@ bool match_contraction(const Routine& r, Phase& ph, const PlanOptions& opt) {
   }
   if (g.flops() < (double)opt.min_mfma_flops) return false;
   if (g.M < 16 || g.N < 16 || g.K < 8) return false;   // matrix-vector shapes stay generic
+  {
+    int64_t nb = 1;   // the batch is the launch grid's z extent
+    for (int i = 0; i < g.nbatch; ++i) nb *= g.batch_ext[i];
+    if (nb > 65535) return false;
+  }
 
   // C must be contiguous along N; if it is contiguous along M instead, compute the transpose.
   if (g.c.s_k != 1) {
