@@ -112,6 +112,9 @@ AxisIndex parse_index(const Sx& x) {
   const std::string h = x.head();
   if (h == "fixed") { a.kind = AxisIndex::Fixed; a.fixed = to_int(x.at(1)); }
   else if (h == "it") { a.kind = AxisIndex::Iter; a.sym = (int)to_int(x.at(1)); }
+  // Sub_axis (indexing.ml:116): an axis spanned by an adjacent multi-axis index adds nothing to the
+  // offset (indexing.ml:429) -- position 0 of its axis
+  else if (h == "sub") { a.kind = AxisIndex::Fixed; a.fixed = 0; }
   else if (h == "affine") {
     a.kind = AxisIndex::Affine;
     for (auto& t : x.at(1).kids) a.terms.emplace_back(to_int(t.at(0)), (int)to_int(t.at(1)));

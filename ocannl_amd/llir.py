@@ -164,7 +164,15 @@ class Affine:
     offset: int = 0
 
 
-AxisIndex = Union[Fixed, It, Affine]
+@dataclass(frozen=True)
+class SubAxis:
+    """``Indexing.Sub_axis`` (indexing.ml:116): the axis belongs to an adjacent multi-axis index --
+    the vectorised initialisers (assignments.ml:684-763) walk a whole tensor through an ``Affine``
+    index on its last axis and mark the others ``Sub_axis``. It prints as nothing (indexing.ml:473)
+    and adds nothing to the offset (indexing.ml:429, c_syntax.ml:367-379): position 0 of its axis."""
+
+
+AxisIndex = Union[Fixed, It, Affine, SubAxis]
 
 
 def sym_ident(s: int) -> str:
@@ -177,6 +185,8 @@ def axis_index_str(idx: AxisIndex) -> str:
         return sym_ident(idx.sym)
     if isinstance(idx, Fixed):
         return str(idx.i)
+    if isinstance(idx, SubAxis):
+        return ""
     terms = [sym_ident(s) if c == 1 else f"{c}*{sym_ident(s)}" for c, s in idx.terms]
     if idx.offset > 0:
         terms.append(str(idx.offset))
@@ -593,6 +603,8 @@ def _wire_idx(i: AxisIndex) -> str:
         return f"(fixed {i.i})"
     if isinstance(i, It):
         return f"(it {i.sym})"
+    if isinstance(i, SubAxis):
+        return "(sub)"
     terms = " ".join(f"({c} {s})" for c, s in i.terms)
     return f"(affine ({terms}) {i.offset})"
 

@@ -279,7 +279,13 @@ def array_offset(idcs: Sequence[L.AxisIndex], dims: Sequence[int]) -> str:
         return "0"
     doc = L.axis_index_str(idcs[0])
     for i in range(1, len(idcs)):
-        doc = f"({doc}) * {dims[i]} + {L.axis_index_str(idcs[i])}"
+        ix = L.axis_index_str(idcs[i])
+        if doc == "":                       # only Sub_axis so far: nothing to scale yet
+            doc = ix
+        elif ix == "":                      # Sub_axis: the axis is spanned, no position of its own
+            doc = f"({doc}) * {dims[i]}"
+        else:
+            doc = f"({doc}) * {dims[i]} + {ix}"
     return doc
 
 

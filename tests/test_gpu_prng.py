@@ -72,3 +72,30 @@ def test_param_init_uniform1(variant):
     assert np.array_equal(g.view(np.uint32), o.view(np.uint32))
     assert g.min() >= -0.25 and g.max() < 0.25 and abs(float(g.mean())) < 0.02
     hip.close()
+
+
+@pytest.mark.parametrize("prec,length", [("single", 4), ("bfloat16", 8)])
+def test_vectorised_init_of_a_matrix_through_sub_axis_indices(prec, length):
+    # a 2-D parameter filled by the vectorised initialiser (assignments.ml:684-763): one loop over the
+    # counters, the last axis indexed `length * i` across row boundaries, the row axis `Sub_axis`
+    # (indexing.ml:116: spanned by the adjacent index, nothing of its own in the offset)
+    rows, cols = 12, 10
+    n = rows * cols // length
+    L.reset_symbols(0)
+    out = L.Node(1, "w", prec, (rows, cols))
+    i = L.fresh_symbol()
+    bits = L.Binop("threefry4x32_light", L.ConstBits(7), L.EmbedIndex(L.It(i)))
+    r = L.Routine("init_w", [L.For(i, 0, n - 1, [L.SetFromVec(
+        out, (L.SubAxis(), L.Affine(((length, i),), 0)), length, "uint4x32_to_prec_uniform", bits, "uint4x32")])])
+    hip, ora = HipRun(r, {}), OracleRun(r, {})
+    assert f"w[{length}*i{i} + 1]" in ora.lib.source                 # flat offset: no row term
+    hip.step(); ora.step()
+    got, want = hip.get(out), ora.get(out)
+    assert np.array_equal(got, want)
+    # the same numbers as a flat vector of the same length gets
+    r1, flat = _uniform_vec_routine(n, prec, length)
+    r1.body[0].body[0].arg.a.value = 7
+    flat_run = OracleRun(r1, {})
+    flat_run.step()
+    assert np.array_equal(want.reshape(-1), flat_run.get(flat))
+    hip.close()
