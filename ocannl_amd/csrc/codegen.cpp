@@ -817,6 +817,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           body.push_back(line);
         }
         if (QG > 1 && !q.coop_scope && q.seq_syms.empty()) throw InvalidArgument("planner: lane group without a reduction to share");
+        if (QG > 64) body.push_back(pind + "__shared__ float red_[4]; __shared__ double redd_[4];");
         emit_phase_statements(r, pr, q, QG, false, pind, body);
       }
       return QP * (uint64_t)QG;

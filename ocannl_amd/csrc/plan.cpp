@@ -404,6 +404,8 @@ void choose_scope_coop(const Routine& r, Phase& ph) {
   int lanes = 1;
   if (unit && rext >= 16) lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
   else if (P < 16384 && R >= 256 && rext >= 2) lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
+  // a handful of long reductions (a loss summed over all tokens): a whole workgroup each
+  if (lanes == 64 && P <= 16 && rext >= 256 && R >= 2048) lanes = 256;
   if (lanes > 1) { ph.coop_lanes = lanes; ph.coop_scope = found[0]; ph.coop_accum = accum; }
 }
 
@@ -434,6 +436,7 @@ void choose_coop(const Routine& r, Phase& ph, const PlanOptions& opt) {
   auto pow2_floor = [](int64_t x) { int64_t p2 = 1; while (p2 * 2 <= x) p2 *= 2; return p2; };
   if (unit && rext >= 16) ph.coop_lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
   else if (P < 16384 && R >= 256 && rext >= 2) ph.coop_lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
+  if (ph.coop_lanes == 64 && P <= 16 && rext >= 256 && R >= 2048) ph.coop_lanes = 256;
 }
 
 // Algorithmic bytes of a generic phase: every distinct (node, index tuple) read once, every
