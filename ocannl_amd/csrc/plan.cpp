@@ -1194,8 +1194,14 @@ void use_bf16_copies(Routine& r, Plan& plan, Phase& ph, Bf16Copies& copies, int*
     if (!stale) copy = it->second;
   }
   if (copy < 0) {
+    // a mirror is kept in step by generated stores and zero fills only: once a contraction has
+    // written the tensor it no longer stands for it
     auto m = plan.mirrors.find(src.id);
-    if (m != plan.mirrors.end()) copy = m->second;
+    if (m != plan.mirrors.end()) {
+      bool in_step = true;
+      for (auto& q : plan.phases) in_step &= !(q.kind == Phase::Contraction && q.gemm.c.node == src.id);
+      if (in_step) copy = m->second;
+    }
   }
   // Can the kernels that produce the tensor keep the copy themselves?  Yes when everything that
   // writes it in this routine is a generated kernel (or a zero fill), and some writer covers the
@@ -1366,6 +1372,13 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
       ph.fill_node = sp->node;
       ph.bytes = (double)n.size_in_bytes();
       plan.phases.push_back(std::move(ph));
+      auto mirror = plan.mirrors.find(sp->node);
+      if (mirror != plan.mirrors.end()) {   // the bf16 copy follows (bf16 zero is all-zero bits)
+        Phase f;
+        f.kind = Phase::Fill; f.label = "zero bf16 copy of " + n.ident; f.fill_node = mirror->second;
+        f.bytes = (double)r.node(mirror->second).size_in_bytes();
+        plan.phases.push_back(std::move(f));
+      }
       continue;
     }
     if (sp->kind == Stmt::DeclareLocal || sp->kind == Stmt::SetLocal)

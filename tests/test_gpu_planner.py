@@ -134,3 +134,43 @@ def test_integer_row_sums_stay_exact():
     assert np.array_equal(ora.get(s), want)
     assert np.array_equal(hip.get(s), want)
     hip.close()
+
+
+def test_bf16_operand_copy_follows_every_kind_of_writer():
+    # an fp32 tensor G feeds bf16 contractions three times: after generated stores (its bf16 copy is
+    # written by those stores), after a matrix-core contraction has accumulated into it (the copy no
+    # longer stands for it: a fresh conversion pass), and after a zero fill (the copy is zeroed too)
+    M, N, K = 128, 128, 128
+    L.reset_symbols(0)
+    ids = iter(range(1, 50))
+    node = lambda name, prec, dims: L.Node(next(ids), name, prec, dims)
+    X = node("x", "single", (M, K)); G = node("g", "single", (M, K)); Wb = node("w", "bfloat16", (N, K))
+    Ab = node("a", "bfloat16", (M, N)); outs = [node(f"out{k}", "single", (M, N)) for k in range(3)]
+    def nest(exts, body):
+        syms = [L.fresh_symbol() for _ in exts]
+        b = body(*[L.It(s) for s in syms])
+        for s, e in reversed(list(zip(syms, exts))):
+            b = [L.For(s, 0, e - 1, b)]
+        return b
+    fma = lambda p, q, c: L.Ternop("fma", p, q, c)
+    read_g = lambda o: nest((M, N, K), lambda m, n, k: [L.Set(o, (m, n), fma(L.Get(G, (m, k)), L.Get(Wb, (n, k)), L.Get(o, (m, n))))])
+    body = nest((M, K), lambda m, k: [L.Set(G, (m, k), L.Binop("mul", L.Const(0.5), L.Get(X, (m, k))))])
+    body += [L.ZeroOut(outs[0])] + read_g(outs[0])
+    body += nest((M, K, N), lambda m, k, n: [L.Set(G, (m, k), fma(L.Get(Ab, (m, n)), L.Get(Wb, (n, k)), L.Get(G, (m, k))))])
+    body += [L.ZeroOut(outs[1])] + read_g(outs[1])
+    body += [L.ZeroOut(G), L.ZeroOut(outs[2])] + read_g(outs[2])
+    r = L.Routine("mirror_chain", body)
+    rng = np.random.default_rng(4)
+    init = {X.id: rng.standard_normal(X.dims).astype(np.float32), Wb.id: W.as_prec(rng.standard_normal(Wb.dims).astype(np.float32), "bfloat16"),
+            Ab.id: W.as_prec(rng.standard_normal(Ab.dims).astype(np.float32) / 16, "bfloat16")}
+    hip = HipRun(r, init, "min_mfma_flops=1")
+    assert sum(k["kind"] == "mfma" for k in hip.code.kernels()) == 4
+    hip.step()
+    bf = lambda a: W.to_float(W.as_prec(np.asarray(a, np.float32), "bfloat16"), "bfloat16").astype(np.float64)
+    w64, a64 = W.to_float(init[Wb.id], "bfloat16").astype(np.float64), W.to_float(init[Ab.id], "bfloat16").astype(np.float64)
+    g1 = (0.5 * init[X.id]).astype(np.float32)
+    g2 = (g1.astype(np.float64) + a64 @ w64).astype(np.float32)
+    for got, want in ((hip.get(outs[0]), bf(g1) @ w64.T), (hip.get(outs[1]), bf(g2) @ w64.T)):
+        assert np.max(np.abs(got - want)) <= 2e-2 * np.max(np.abs(want))
+    assert not hip.get(outs[2]).any() and not hip.get(G).any()
+    hip.close()
