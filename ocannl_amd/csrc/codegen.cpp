@@ -286,6 +286,8 @@ struct Printer {
   std::set<int> used_nodes;
   std::set<int> used_statics;
   bool used_merge = false;
+  std::map<int, std::string> shadow;   // serial group: node -> LDS array every store is copied to
+  std::set<int> shadow_live;           // ... and whose contents reads may use by now
   // type of loop iterators and offsets: 64-bit when a node is too large for 32-bit offsets
   // (the `large_models` setting, c_syntax.ml:111-112)
   std::string idx_t = "uint32_t";
@@ -313,6 +315,20 @@ struct Printer {
         used_nodes.insert(m->second);
         mirror_lhs = r.node(m->second).ident + lhs.substr(lhs.find('['));   // same dims: same offset
       }
+    }
+    auto sh = shadow.find(node);
+    if (sh != shadow.end()) {
+      // (a shadowed tensor has no bf16 mirror: mirrors belong to matrix-core contractions, which a
+      // serial group does not contain)
+      const std::string sh_lhs = sh->second + lhs.substr(lhs.find('['));
+      auto itc = cache_name.find(node);
+      if (itc == cache_name.end()) {
+        const std::string t = "m" + std::to_string(fresh++) + "_";
+        return "{ const " + std::string(c_typ(r.node(node).prec)) + " " + t + " = " + value + "; " + guard + "{ " + lhs + " = " + t +
+               "; " + sh_lhs + " = " + t + "; } }";
+      }
+      cache_defined.insert(node);
+      return itc->second + " = " + value + "; " + guard + "{ " + lhs + " = " + itc->second + "; " + sh_lhs + " = " + itc->second + "; }";
     }
     auto it = cache_name.find(node);
     if (it == cache_name.end()) {
@@ -404,6 +420,7 @@ struct Printer {
         if (self_set && s.node == self_set->node && s.idcs == self_set->idcs) return c.first + self_name + c.second;
         if (cache_defined.count(s.node)) return c.first + cache_name.at(s.node) + c.second;
         note(s.node, s.idcs);
+        if (shadow_live.count(s.node)) return c.first + shadow.at(s.node) + "[" + offset_str(s.idcs, n.dims) + "]" + c.second;
         return c.first + n.ident + "[" + offset_str(s.idcs, n.dims) + "]" + c.second;
       }
       case Scalar::GetDyn: {
@@ -826,14 +843,24 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     uint64_t total_threads = 0;
     if (!ph.serial_members.empty()) {
       // ---- the whole routine in one workgroup: phases in order, a barrier after each
-      for (auto& q : ph.serial_members) {
+      for (auto& kv : ph.serial_shadows) {
+        const Node& sn = r.node(kv.first);
+        pr.shadow[kv.first] = "sh_" + sn.ident;
+        body.push_back(ind + "__shared__ " + c_typ(sn.prec) + " sh_" + sn.ident + "[" + std::to_string(sn.num_elems()) + "];");
+      }
+      for (size_t qi = 0; qi < ph.serial_members.size(); ++qi) {
+        const Phase& q = ph.serial_members[qi];
+        for (auto& kv : ph.serial_shadows) if (kv.second < (int)qi) pr.shadow_live.insert(kv.first);
         body.push_back(ind + "/* " + q.label + " */");
         if (q.kind == Phase::Fill) {
           const Node& fn = r.node(q.fill_node);
           pr.used_nodes.insert(q.fill_node);
           Pair cv = convert_precision(Prec::Double, fn.prec);
-          body.push_back(ind + "for (" + pr.idx_t + " z_ = threadIdx.x; z_ < " + std::to_string(fn.num_elems()) + "ull; z_ += 256u) " +
-                         fn.ident + "[z_] = " + cv.first + "0" + cv.second + ";");
+          const std::string zero = cv.first + "0" + cv.second;
+          std::string line = ind + "for (" + pr.idx_t + " z_ = threadIdx.x; z_ < " + std::to_string(fn.num_elems()) + "ull; z_ += 256u) ";
+          if (pr.shadow.count(q.fill_node)) line += "{ " + fn.ident + "[z_] = " + zero + "; " + pr.shadow.at(q.fill_node) + "[z_] = " + zero + "; }";
+          else line += fn.ident + "[z_] = " + zero + ";";
+          body.push_back(line);
         } else {
           uint64_t qt = (uint64_t)q.coop_lanes;
           for (auto e : (q.members.empty() ? q.par_ext : q.row_outer_ext)) qt *= (uint64_t)e;
@@ -844,6 +871,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
         }
         body.push_back(ind + "__syncthreads();");
       }
+      pr.shadow.clear(); pr.shadow_live.clear();
       total_threads = 256;
     } else {
       body.push_back(ind + "const uint64_t gtid_ = ((uint64_t)blockIdx.y * gridDim.x + blockIdx.x) * blockDim.x + threadIdx.x;");

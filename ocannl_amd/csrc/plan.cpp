@@ -1097,6 +1097,55 @@ void group_rows(const Routine& r, Plan& plan) {
 // ---- tiny routines ---------------------------------------------------------------------------------
 namespace {
 
+bool writes_whole_node(const Routine& r, const Phase& ph, int node);
+
+// LDS shadows for a serial group (see Phase::serial_shadows).
+void choose_shadows(const Routine& r, Phase& g) {
+  struct Flat { const Phase* ph; int member; };
+  std::vector<Flat> flat;
+  for (size_t q = 0; q < g.serial_members.size(); ++q) {
+    const Phase& m = g.serial_members[q];
+    if (m.members.empty()) flat.push_back({&m, (int)q});
+    else for (auto& sub : m.members) flat.push_back({&sub, (int)q});
+  }
+  int64_t budget = 48 * 1024;
+  for (auto& kv : r.nodes) {
+    const Node& n = kv.second;
+    if (n.mode == Mode::Virtual || n.prec == Prec::Uint4x32 || n.prec == Prec::Void) continue;
+    const int64_t bytes = (int64_t)n.size_in_bytes();
+    if (bytes > budget || bytes > 16 * 1024) continue;
+    int valid_after = -1;
+    bool ok = true;
+    for (auto& f : flat) {
+      const Phase& ph = *f.ph;
+      if (ph.kind == Phase::Fill) {
+        if (ph.fill_node == n.id && valid_after < 0) valid_after = f.member;
+        continue;
+      }
+      std::vector<Access> acc; bool w = false, fo = false; std::set<ScopeId> d;
+      block_accesses(ph.inner, acc, w, fo, d);
+      if (w) { ok = false; break; }   // a Zero_out inside a nest: stores the printer does not route
+      bool touches = false, writes = false, reads = false, vec = false;
+      for (auto& a : acc) if (a.node == n.id) {
+        touches = true;
+        if (a.write) { writes = true; vec |= a.vec_len > 0; }
+        else if (!(ph.fused_zero_init && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set && ph.inner[0]->node == n.id)) reads = true;
+      }
+      if (!touches) continue;
+      if (vec) { ok = false; break; }
+      if (valid_after < 0) {
+        // the first touch has to store the whole tensor without reading it
+        if (!writes || reads || !writes_whole_node(r, ph, n.id)) { ok = false; break; }
+        valid_after = f.member;
+      }
+    }
+    if (ok && valid_after >= 0 && valid_after + 1 < (int)g.serial_members.size()) {
+      g.serial_shadows[n.id] = valid_after;
+      budget -= bytes;
+    }
+  }
+}
+
 void serialise_tiny(const Routine& r, Plan& plan) {
   if (plan.phases.size() < 4) return;
   double bytes = 0;
@@ -1128,6 +1177,7 @@ void serialise_tiny(const Routine& r, Plan& plan) {
   g.label = "whole routine, one workgroup";
   g.bytes = bytes;
   g.serial_members = std::move(plan.phases);
+  choose_shadows(r, g);
   plan.phases.clear();
   plan.phases.push_back(std::move(g));
 }

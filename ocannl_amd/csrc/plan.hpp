@@ -74,6 +74,10 @@ struct Phase {
   // as ONE kernel of a single workgroup that executes the phases in order with a barrier in between
   // (dozens of launches of a few microseconds each would otherwise be pure launch latency).
   std::vector<Phase> serial_members;
+  // Serial group: tensors whose first touch in the kernel is a store to all of their elements are
+  // shadowed in LDS (node -> index of the member that makes the shadow valid): later members read
+  // the shadow instead of waiting on global memory; every store still goes to global memory too.
+  std::map<int, int> serial_shadows;
   // Fill
   int fill_node = -1;
   // Contraction
