@@ -967,6 +967,11 @@ bool row_member(const Routine& r, Phase& ph, RowShape& shape, bool first) {
     ph.row_role = Phase::RowScalar; ph.row_outer_syms = syms; ph.row_sym = -1;
     return true;
   }
+  if (first && ext.empty()) {                                                 // a chain of plain scalars
+    ph.row_role = Phase::RowScalar; ph.row_outer_syms = syms; ph.row_sym = -1;
+    shape.outer.clear();
+    return true;
+  }
   if (ext.empty()) return false;                                              // pointwise over rows x T
   const int64_t T = ext.back();
   // (short rows leave lanes idle: the caller takes such a group only when it is launch-bound anyway)
@@ -1046,8 +1051,9 @@ void group_rows(const Routine& r, Plan& plan) {
     for (auto e : shape.outer) rows *= e;
     // ... or sit in a routine so small that launches are all there is to save (in a large routine
     // such a group was measured slower than its members as separate, overlapping launches)
+    if (shape.len < 0 && shape.outer.empty() && run.size() >= 2) shape.len = 1;   // scalars only
     const int64_t points = rows * std::max<int64_t>(shape.len, 1);
-    if (run.size() >= 2 && shape.len >= 2 && ((shape.len >= 16 && points >= (1 << 16)) || (launch_bound && points < 8192))) {
+    if (run.size() >= 2 && shape.len >= 1 && ((shape.len >= 16 && points >= (1 << 16)) || (launch_bound && points < 8192))) {
       Phase g;
       g.kind = Phase::Generic;
       g.label = run.front().label + " .. " + run.back().label;
@@ -1171,7 +1177,9 @@ void serialise_tiny(const Routine& r, Plan& plan) {
     } else return;
     bytes += ph.bytes;
   }
-  if (iterations > 8 * (int64_t)plan.phases.size()) return;
+  int64_t statements = 0;   // a row group counts as the statements it fuses
+  for (auto& ph : plan.phases) statements += ph.members.empty() ? 1 : (int64_t)ph.members.size();
+  if (iterations > 8 * statements) return;
   Phase g;
   g.kind = Phase::Generic;
   g.label = "whole routine, one workgroup";
