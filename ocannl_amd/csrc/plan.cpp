@@ -1475,6 +1475,22 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
       }
       if (full) { ph.fused_zero_init = true; plan.phases.erase(plan.phases.begin() + fill_at); }
     }
+    // a dead fill: the nest stores to every element of a tensor without reading it, and nothing has
+    // touched the tensor since its Zero_out
+    if (!devirt && fill_at < 0 && ph.seq_syms.empty() && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set) {
+      const int target = ph.inner[0]->node;
+      std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+      block_accesses(ph.inner, acc, w, f, d);
+      bool reads_target = w || f;
+      for (auto& a : acc) if (!a.write && a.node == target) reads_target = true;
+      if (!reads_target && writes_whole_node(r, ph, target)) {
+        for (int q = (int)plan.phases.size() - 1; q >= 0; --q) {
+          const Phase& prev = plan.phases[q];
+          if (prev.kind == Phase::Fill && prev.fill_node == target) { plan.phases.erase(plan.phases.begin() + q); break; }
+          if (phase_touches(prev, target)) break;
+        }
+      }
+    }
 
     if (!match_contraction(r, ph, opt)) {
       ph.kind = Phase::Generic;
