@@ -224,7 +224,11 @@ class Gen:
             d, a = self.wide_acc(self.mats)[0], self.mats[1]
             k = L.fresh_symbol()
             lhs = (L.It(i), L.It(j))
-            return [L.ZeroOut(d)] + self.nest([(i, R), (j, C), (k, C)], [L.Set(d, lhs, L.Ternop(
+            # (from zero, or on top of what the tensor holds, scaled down so that values stay of order one)
+            start = [L.ZeroOut(d)] if rng.random() < 0.5 else self.nest([(i, R), (j, C)], [L.Set(d, lhs, L.Binop("mul", L.Const(0.01), L.Get(d, lhs)))])
+            i, j = L.fresh_symbol(), L.fresh_symbol()
+            lhs = (L.It(i), L.It(j))
+            return start + self.nest([(i, R), (j, C), (k, C)], [L.Set(d, lhs, L.Ternop(
                 "fma", L.Get(a, (L.It(i), L.It(k))), L.Get(self.sq, (L.It(k), L.It(j))), L.Get(d, lhs)))])
         d = pick(self.mats)
         return self.nest([(i, R), (j, C)], [L.Set(d, (L.It(i), L.It(j)), self.expr(i, j))])
