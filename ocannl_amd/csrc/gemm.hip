@@ -108,6 +108,20 @@ __device__ __forceinline__ void decode_batch(const GemmArgs& g, long z, long& ao
   if (g.nbatch > 0) { const long e = g.batch_ext[0], q = z % e; ao += q * g.a_batch[0]; bo += q * g.b_batch[0]; co += q * g.c_batch[0]; }
 }
 
+// Grouped launch: blockIdx.z = group * batches + batch.  Returns the batch index and the operands of
+// the group (constant array indices only, as above).
+__device__ __forceinline__ long decode_group(const GemmArgs& g, long z, const void*& a, const void*& b, void*& c) {
+  a = g.a; b = g.b; c = g.c;
+  if (g.ngroups > 1) {
+    const long grp = z / g.batches;
+    z -= grp * g.batches;
+    if (grp == 1) { a = g.a_more[0]; b = g.b_more[0]; c = g.c_more[0]; }
+    else if (grp == 2) { a = g.a_more[1]; b = g.b_more[1]; c = g.c_more[1]; }
+    else if (grp == 3) { a = g.a_more[2]; b = g.b_more[2]; c = g.c_more[2]; }
+  }
+  return z;
+}
+
 // XCD-aware tile order.  Consecutive hardware workgroup ids land on different XCDs (id % 8), each
 // with its own L2.  The tile grid is cut into xcd_m x (8 / xcd_m) rectangles, one per XCD, chosen
 // on the host so that the operand panels shared inside a rectangle are the expensive ones
@@ -274,7 +288,7 @@ __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, 
 // wave-uniform switch: that bounds what the compiler can hoist above the branch to one row's
 // registers (hoisting all 256 accumulator reads above one up-front branch spills them).
 template <int TM, int TN>
-__device__ __forceinline__ void epilogue(const GemmArgs& g, f32x16 (&acc)[TM][TN], long m, long n, long co, int lane) {
+__device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, f32x16 (&acc)[TM][TN], long m, long n, long co, int lane) {
   const long rows_left = g.M - m, cols_left = g.N - n;
   if (rows_left <= 0 || cols_left <= 0) return;
   const bool full = rows_left >= TM * 32 && cols_left >= TN * 32;
@@ -282,7 +296,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, f32x16 (&acc)[TM][TN
   const bool bf = !to_ws && g.c_is_bf16;
   const long ld = to_ws ? g.N : g.c_row;
   const long first = to_ws ? (((long)blockIdx.z * g.splits + blockIdx.y) * g.M + m) * g.N + n : co + m * g.c_row + n;
-  char* const origin = (to_ws ? reinterpret_cast<char*>(g.ws) : static_cast<char*>(g.c)) + first * (bf ? 2 : 4);
+  char* const origin = (to_ws ? reinterpret_cast<char*>(g.ws) : static_cast<char*>(cbase)) + first * (bf ? 2 : 4);
   const int variant = (bf ? 4 : 0) + ((!to_ws && g.accumulate) ? 2 : 0) + (full ? 0 : 1);
   static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
     constexpr int i = decltype(ic)::value;
@@ -327,9 +341,11 @@ gemm_bf16_kernel(const GemmArgs g) {
   tile_of_block(blockIdx.x, tiles_m, tiles_n, g.xcd_m, tmi, tni);
   const long m0 = tmi * BM, n0 = tni * BN;
   long ao, bo, co;
-  decode_batch(g, blockIdx.z, ao, bo, co);
-  const AT* A = static_cast<const AT*>(g.a) + ao;
-  const BT* B = static_cast<const BT*>(g.b) + bo;
+  const void *abase, *bbase;
+  void* cbase;
+  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase), ao, bo, co);
+  const AT* A = static_cast<const AT*>(abase) + ao;
+  const BT* B = static_cast<const BT*>(bbase) + bo;
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
 
   // per-lane offsets of the MFMA fragments inside a stage of each operand
@@ -509,7 +525,7 @@ gemm_bf16_kernel(const GemmArgs g) {
   }
   OCANNL_STAMP(2);
 
-  epilogue<TM, TN>(g, acc, m0 + wm0, n0 + wn0, co, lane);
+  epilogue<TM, TN>(g, cbase, acc, m0 + wm0, n0 + wn0, co, lane);
   OCANNL_STAMP(3);
 }
 
@@ -573,9 +589,11 @@ gemm_f32_kernel(const GemmArgs g) {
   tile_of_block(blockIdx.x, tiles_m, tiles_n, g.xcd_m, tmi, tni);
   const long m0 = tmi * BM, n0 = tni * BN;
   long ao, bo, co;
-  decode_batch(g, blockIdx.z, ao, bo, co);
-  const float* A = static_cast<const float*>(g.a) + ao;
-  const float* B = static_cast<const float*>(g.b) + bo;
+  const void *abase, *bbase;
+  void* cbase;
+  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase), ao, bo, co);
+  const float* A = static_cast<const float*>(abase) + ao;
+  const float* B = static_cast<const float*>(bbase) + bo;
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
 
   f32x16 acc[TM][TN];
@@ -643,7 +661,7 @@ gemm_f32_kernel(const GemmArgs g) {
     __syncthreads();
   }
 
-  epilogue<TM, TN>(g, acc, m0 + wm0, n0 + wn0, co, lane);
+  epilogue<TM, TN>(g, cbase, acc, m0 + wm0, n0 + wn0, co, lane);
 }
 
 template <int BM, int BN, bool A_KC, bool B_KC>
@@ -658,28 +676,31 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const GemmArgs g) {
   if (idx >= g.M * n4) return;
   const long m = idx / n4, n = (idx % n4) * 4;
   long ao, bo, co;
-  decode_batch(g, blockIdx.z, ao, bo, co);
+  const void *abase, *bbase;
+  void* cbase;
+  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase), ao, bo, co);
   f32x4 sum = {0, 0, 0, 0};
   for (int sp = 0; sp < g.splits; ++sp)
     sum += *reinterpret_cast<const f32x4*>(g.ws + (((long)blockIdx.z * g.splits + sp) * g.M + m) * g.N + n);
   const long off = co + m * g.c_row + n;
   if (g.c_is_bf16) {
-    unsigned short* C = static_cast<unsigned short*>(g.c);
+    unsigned short* C = static_cast<unsigned short*>(cbase);
     for (int q = 0; q < 4; ++q) {
       float v = sum[q];
       if (g.accumulate) v += __uint_as_float(((unsigned)C[off + q]) << 16);
       C[off + q] = (unsigned short)f2bf(v);
     }
   } else {
-    float* C = static_cast<float*>(g.c);
+    float* C = static_cast<float*>(cbase);
     f32x4 v = sum;
     if (g.accumulate) v += *reinterpret_cast<const f32x4*>(C + off);
     *reinterpret_cast<f32x4*>(C + off) = v;
   }
 }
 
+// Tile grids of one launch along z: batch entries times grouped contractions.
 long batch_count(const GemmDesc& d) {
-  long nb = 1;
+  long nb = 1 + (long)d.group.size();
   for (int i = 0; i < d.nbatch; ++i) nb *= d.batch_ext[i];
   return nb;
 }
@@ -745,6 +766,9 @@ hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t
   const long tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   long nb = 1;
   for (int i = 0; i < a.nbatch; ++i) nb *= a.batch_ext[i];
+  if (a.ngroups < 1 || a.ngroups > 4) return hipErrorInvalidValue;
+  a.batches = (int)nb;
+  nb *= a.ngroups;
   if (tiles <= 0 || tiles > 0x7FFFFFFFL || nb <= 0 || nb > 65535) return hipErrorInvalidValue;
   if (a.splits > 1 && !a.ws) return hipErrorInvalidValue;
   hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)a.splits, (unsigned)nb), dim3(kThreads), smem, s, a);

@@ -21,6 +21,14 @@ struct GemmArgs {
   int xcd_m;         // tile-grid rows of the XCD partition (set by launch_gemm; 0: none)
   int splits;        // split-K factor (set by launch_gemm)
   float* ws;         // split-K workspace [batch][split][M][N] (set by launch_gemm)
+  // One launch may cover up to four independent contractions of identical shapes, strides and
+  // precisions: member g > 0 uses a_more / b_more / c_more[g - 1], and the grid's z axis is
+  // member * batches + batch.
+  int ngroups;       // >= 1
+  int batches;       // product of batch_ext (set by launch_gemm)
+  const void* a_more[3];
+  const void* b_more[3];
+  void* c_more[3];
 };
 
 // Picks the kernel instance for the operand precisions / layouts and launches it on `stream`.

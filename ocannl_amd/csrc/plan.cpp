@@ -486,7 +486,10 @@ void account_bytes(const Routine& r, Phase& ph) {
 // Does the phase read or write `node`?
 bool phase_touches(const Phase& ph, int node) {
   if (ph.kind == Phase::Fill) return ph.fill_node == node;
-  if (ph.kind == Phase::Contraction) return ph.gemm.a.node == node || ph.gemm.b.node == node || ph.gemm.c.node == node;
+  if (ph.kind == Phase::Contraction) {
+    for (auto& m : ph.gemm.group) if (m.a.node == node || m.b.node == node || m.c.node == node) return true;
+    return ph.gemm.a.node == node || ph.gemm.b.node == node || ph.gemm.c.node == node;
+  }
   std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
   block_accesses(ph.inner, acc, w, f, d);
   if (w) return true;   // a Zero_out inside the nest: not tracked per node, assume the worst
@@ -1100,6 +1103,108 @@ void group_rows(const Routine& r, Plan& plan) {
 
 }  // namespace
 
+// ---- contractions that share a launch ---------------------------------------------------------------
+// Independent contractions of identical shapes, strides and precisions (the q / k / v projections of
+// one input; the weight gradients of those projections) ride in one launch whose z axis runs over
+// the members.  A small contraction alone puts at most one workgroup on a compute unit; several
+// together let workgroups hide each other's memory latency.
+// The statements need not be adjacent.  A later one is hoisted to the earlier one's position when
+// nothing in between touches its result or writes its operands; otherwise the earlier ones are sunk
+// to the later position under the same condition on them.
+namespace {
+
+bool phase_writes(const Phase& ph, int node);
+
+bool same_layout(const GemmOperand& x, const GemmOperand& y) {
+  if (x.prec != y.prec || x.s_row != y.s_row || x.s_k != y.s_k) return false;
+  for (int i = 0; i < 3; ++i) if (x.s_batch[i] != y.s_batch[i]) return false;
+  return true;
+}
+
+void group_contractions(Plan& plan) {
+  std::map<int, int> mirror_source;   // bf16 copy -> the tensor whose stores keep it in step
+  for (auto& kv : plan.mirrors) mirror_source[kv.second] = kv.first;
+  auto source_of = [&](int node) { auto m = mirror_source.find(node); return m == mirror_source.end() ? node : m->second; };
+  auto writes_operand = [&](const Phase& q, const GemmOperand& op) {
+    return phase_writes(q, op.node) || phase_writes(q, source_of(op.node));
+  };
+  auto touches_result = [&](const Phase& q, const GemmOperand& c) {
+    if (phase_touches(q, c.node)) return true;
+    auto m = plan.mirrors.find(c.node);
+    return m != plan.mirrors.end() && phase_touches(q, m->second);
+  };
+  struct Member { GemmOperand a, b, c; };
+  auto members_of = [](const GemmDesc& g) {
+    std::vector<Member> v{{g.a, g.b, g.c}};
+    for (auto& m : g.group) v.push_back({m.a, m.b, m.c});
+    return v;
+  };
+  // may the contraction `x` run at another place of phases (lo, hi), i.e. does nothing there touch
+  // its result or write its operands?
+  auto free_between = [&](const Member& x, size_t lo, size_t hi) {
+    for (size_t k = lo + 1; k < hi; ++k) {
+      const Phase& mid = plan.phases[k];
+      if (touches_result(mid, x.c) || writes_operand(mid, x.a) || writes_operand(mid, x.b)) return false;
+    }
+    return true;
+  };
+  for (size_t i = 0; i < plan.phases.size(); ++i) {
+    if (plan.phases[i].kind != Phase::Contraction) continue;
+    {
+      const GemmDesc& g = plan.phases[i].gemm;
+      // grouping pays where a launch alone leaves compute units idle or with one workgroup each
+      double tiles = (double)((g.M + 127) / 128) * (double)((g.N + 127) / 128);
+      for (int b = 0; b < g.nbatch; ++b) tiles *= (double)g.batch_ext[b];
+      if (tiles > 256) continue;
+    }
+    bool sunk = false;
+    for (size_t j = i + 1; j < plan.phases.size() && !sunk; ++j) {
+      Phase& p = plan.phases[i];
+      GemmDesc& g = p.gemm;
+      if (g.group.size() >= 3) break;
+      Phase& q = plan.phases[j];
+      const GemmDesc& h = q.gemm;
+      bool candidate = q.kind == Phase::Contraction && h.group.empty() && h.M == g.M && h.N == g.N &&
+                       h.K == g.K && h.nbatch == g.nbatch && same_layout(h.a, g.a) && same_layout(h.b, g.b) && same_layout(h.c, g.c);
+      for (int b = 0; b < g.nbatch && candidate; ++b) candidate = h.batch_ext[b] == g.batch_ext[b];
+      const std::vector<Member> mine = members_of(g);
+      if (candidate) {
+        candidate = h.accumulate == g.accumulate;
+        for (auto& x : mine) {
+          const int xc = x.c.node, hc = h.c.node;
+          candidate = candidate && hc != xc && source_of(h.a.node) != xc && source_of(h.b.node) != xc && h.a.node != xc && h.b.node != xc &&
+                      source_of(x.a.node) != hc && source_of(x.b.node) != hc && x.a.node != hc && x.b.node != hc;
+        }
+      }
+      if (!candidate) continue;
+      const Member joiner{h.a, h.b, h.c};
+      bool hoist = free_between(joiner, i, j), sink = false;
+      if (!hoist) {
+        sink = true;
+        for (auto& x : mine) sink = sink && free_between(x, i, j);
+      }
+      if (!hoist && !sink) continue;
+      g.group.push_back({h.a, h.b, h.c});
+      p.bytes += q.bytes;
+      p.flops = g.flops();
+      p.label += " | " + q.label;
+      if (hoist) {
+        plan.phases.erase(plan.phases.begin() + j);
+        --j;
+      } else {
+        // the merged launch takes the later statement's place; position i now holds what followed
+        // and is looked at again
+        plan.phases[j] = std::move(plan.phases[i]);
+        plan.phases.erase(plan.phases.begin() + i);
+        sunk = true;
+        --i;
+      }
+    }
+  }
+}
+
+}  // namespace
+
 // ---- tiny routines ---------------------------------------------------------------------------------
 namespace {
 
@@ -1203,7 +1308,10 @@ namespace {
 
 bool phase_writes(const Phase& ph, int node) {
   if (ph.kind == Phase::Fill) return ph.fill_node == node;
-  if (ph.kind == Phase::Contraction) return ph.gemm.c.node == node;
+  if (ph.kind == Phase::Contraction) {
+    for (auto& m : ph.gemm.group) if (m.c.node == node) return true;
+    return ph.gemm.c.node == node;
+  }
   auto writes = [&](const Phase& q) {
     std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
     block_accesses(q.inner, acc, w, f, d);
@@ -1503,6 +1611,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     }
     plan.phases.push_back(std::move(ph));
   }
+  if (opt.enable_mfma && opt.group_contractions) group_contractions(plan);
   if (opt.enable_coop && opt.enable_row_groups) group_rows(r, plan);
   if (opt.enable_serial_group) serialise_tiny(r, plan);
   return plan;

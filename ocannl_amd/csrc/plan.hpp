@@ -36,8 +36,14 @@ struct GemmDesc {
   int nbatch = 0;
   int64_t batch_ext[3] = {1, 1, 1};
   bool accumulate = false;   // beta = 1: add into existing C (gradient accumulation `=+`)
+  // Independent contractions of the same shapes, strides and precisions (the q / k / v projections of
+  // one input, their weight gradients) that ride in the same launch: {a, b, c} per extra member.  A
+  // small contraction alone puts at most one workgroup on a compute unit; several together let
+  // workgroups hide each other's memory latency.
+  struct Member { GemmOperand a, b, c; };
+  std::vector<Member> group;
   double flops() const {
-    double f = 2.0 * (double)M * (double)N * (double)K;
+    double f = 2.0 * (double)M * (double)N * (double)K * (double)(1 + group.size());
     for (int i = 0; i < nbatch; ++i) f *= (double)batch_ext[i];
     return f;
   }
@@ -92,6 +98,7 @@ struct PlanOptions {
   bool enable_coop = true;
   bool enable_row_groups = true;
   bool enable_serial_group = true;   // tiny routines as one single-workgroup kernel
+  bool group_contractions = true;   // independent contractions of equal shapes as one launch
   bool large_models = false;        // 64-bit offsets in generated kernels even when every node is small
   bool enable_bf16_copies = true;   // keep bf16 copies of fp32 operands of mixed contractions (written by the producing kernels)
 };

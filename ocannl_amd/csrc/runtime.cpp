@@ -113,6 +113,7 @@ PlanOptions parse_options(const char* options) {
     else if (k == "bf16_copies") o.enable_bf16_copies = v != "0";
     else if (k == "serial") o.enable_serial_group = v != "0";
     else if (k == "large_models") o.large_models = v != "0";
+    else if (k == "groups") o.group_contractions = v != "0";
     else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
     else throw InvalidArgument("compile options: unknown key '" + k + "'");
   }
@@ -243,6 +244,10 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
       }
       a.accumulate = g.accumulate ? 1 : 0;
       a.c_is_bf16 = g.c.prec == Prec::Bfloat16;
+      a.ngroups = 1 + (int)g.group.size();
+      for (size_t m = 0; m < g.group.size(); ++m) {
+        a.a_more[m] = base(g.group[m].a); a.b_more[m] = base(g.group[m].b); a.c_more[m] = base(g.group[m].c);
+      }
       // a bracketed contraction is timed without its split-K reduction (a kernel of its own)
       hip_check(launch_gemm(g, a, rt.gemm_ws, dev.stream, bracket ? rt.profile_events[rt.profile_used + 1] : nullptr),
                 "launch_gemm");
@@ -584,8 +589,9 @@ int ocannl_hip_code_kernel_info(ocannl_hip_code* code, int index, int kernel, oc
     info->bytes = ph.bytes;
     std::string name;
     if (ph.kind == Phase::Contraction) {
+      // grouped contractions read as more batch entries
       info->m = ph.gemm.M; info->n = ph.gemm.N; info->k = ph.gemm.K;
-      info->batch = 1;
+      info->batch = 1 + (int64_t)ph.gemm.group.size();
       for (int i = 0; i < ph.gemm.nbatch; ++i) info->batch *= ph.gemm.batch_ext[i];
       name = gemm_kernel_name(ph.gemm);
     } else if (ph.kind == Phase::Fill) {
@@ -642,7 +648,9 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
     // the MFMA kernels read 16-byte chunks relative to the node base
     for (auto& ph : cr.plan.phases) {
       if (ph.kind != Phase::Contraction) continue;
-      for (const GemmOperand* op : {&ph.gemm.a, &ph.gemm.b, &ph.gemm.c})
+      std::vector<const GemmOperand*> ops{&ph.gemm.a, &ph.gemm.b, &ph.gemm.c};
+      for (auto& m : ph.gemm.group) { ops.push_back(&m.a); ops.push_back(&m.b); ops.push_back(&m.c); }
+      for (const GemmOperand* op : ops)
         if (reinterpret_cast<uintptr_t>(rt->node_ptr.at(op->node)) % 16 != 0)
           throw UserError("hip backend link: node " + cr.r.node(op->node).ident +
                           " feeds a matrix-core contraction and must sit at a 16-byte aligned pool offset");

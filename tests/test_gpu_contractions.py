@@ -151,3 +151,84 @@ def test_operands_sliced_by_static_and_fixed_indices(prec):
     with pytest.raises(hip.B.User_error):
         hip.step({s1.sym: S, s2.sym: 0})             # out of range: refused before anything is enqueued
     hip.close()
+
+
+def _product_nest(A, B, C, M, N, K, a_kc, b_kc):
+    m, n, k = (L.fresh_symbol() for _ in range(3))
+    ai = (L.It(m), L.It(k)) if a_kc else (L.It(k), L.It(m))
+    bi = (L.It(n), L.It(k)) if b_kc else (L.It(k), L.It(n))
+    ci = (L.It(m), L.It(n))
+    return L.For(m, 0, M - 1, [L.For(n, 0, N - 1, [L.For(k, 0, K - 1, [
+        L.Set(C, ci, L.Ternop("fma", L.Get(A, ai), L.Get(B, bi), L.Get(C, ci)))])])])
+
+
+def _f64(x, prec, kc):
+    v = W.to_float(x, prec).astype(np.float64)
+    return v if kc else v.T
+
+
+@pytest.mark.parametrize("shape", [(256, 384, 512), (136, 72, 200), (128, 128, 4096)])
+@pytest.mark.parametrize("layout", [(True, True), (True, False), (False, False)])
+@pytest.mark.parametrize("precs", [("bfloat16", "single", True), ("bfloat16", "bfloat16", False), ("single", "single", False)])
+def test_independent_products_of_one_shape_share_a_launch(shape, layout, precs):
+    # y_g (+)= x w_g for three weights, with a pointwise statement on an unrelated tensor in between
+    M, N, K = shape
+    a_kc, b_kc = layout
+    prec, c_prec, accumulate = precs
+    L.reset_symbols(0)
+    X = L.Node(1, "x", prec, (M, K) if a_kc else (K, M))
+    Ws = [L.Node(2 + g, f"w{g}", prec, (N, K) if b_kc else (K, N)) for g in range(3)]
+    Ys = [L.Node(5 + g, f"y{g}", c_prec, (M, N)) for g in range(3)]
+    U = L.Node(8, "u", "single", (64,))
+    i = L.fresh_symbol()
+    bump = L.For(i, 0, 63, [L.Set(U, (L.It(i),), L.Binop("add", L.Get(U, (L.It(i),)), L.Const(1.0)))])
+    body = []
+    for g in range(3):
+        if not accumulate:
+            body.append(L.ZeroOut(Ys[g]))
+        body.append(_product_nest(X, Ws[g], Ys[g], M, N, K, a_kc, b_kc))
+        if g == 0:
+            body.append(bump)
+    r = L.Routine("group", body)
+    rng = np.random.default_rng(12)
+    init = {x.id: W.as_prec(rng.standard_normal(x.dims).astype(np.float32), x.prec) for x in [X] + Ws + Ys}
+    init[U.id] = np.zeros(64, np.float32)
+    x64 = _f64(init[X.id], prec, a_kc)
+    outs = {}
+    for opts, launches in (("min_mfma_flops=1", 1), ("min_mfma_flops=1;groups=0", 3)):
+        hip = HipRun(r, init, opts)
+        ks = hip.code.kernels()
+        assert sorted(k["kind"] for k in ks) == ["generated"] + ["mfma"] * launches, ks
+        hip.step()
+        outs[launches] = [W.to_float(hip.get(y), c_prec).astype(np.float64) for y in Ys]
+        assert np.array_equal(hip.get(U), np.ones(64, np.float32))
+        hip.close()
+    tol = 2.0 ** -8 if c_prec == "bfloat16" else 2e-6 * max(1.0, np.sqrt(K) / 8)
+    for g in range(3):
+        want = x64 @ _f64(init[Ws[g].id], prec, b_kc).T
+        if accumulate:
+            want = want + W.to_float(init[Ys[g].id], c_prec).astype(np.float64)
+        for got in outs.values():
+            assert np.max(np.abs(got[g] - want)) <= tol * np.max(np.abs(want)), (g, layout, precs)
+    # grouped and separate launches sum in the same order: identical bits
+    for g in range(3):
+        assert np.array_equal(outs[1][g], outs[3][g])
+
+
+def test_a_product_that_reads_another_products_result_is_not_grouped_with_it():
+    M = N = K = 256
+    L.reset_symbols(0)
+    X = L.Node(1, "x", "bfloat16", (M, K)); W0 = L.Node(2, "w0", "bfloat16", (N, K)); W1 = L.Node(3, "w1", "bfloat16", (N, K))
+    Y = L.Node(4, "y", "bfloat16", (M, N)); Z = L.Node(5, "z", "bfloat16", (M, N))
+    body = [L.ZeroOut(Y), _product_nest(X, W0, Y, M, N, K, True, True), L.ZeroOut(Z), _product_nest(Y, W1, Z, M, N, K, True, True)]
+    r = L.Routine("dependent", body)
+    rng = np.random.default_rng(13)
+    init = {x.id: W.as_prec(rng.standard_normal(x.dims).astype(np.float32) / 16, "bfloat16") for x in (X, W0, W1)}
+    hip = HipRun(r, init, "min_mfma_flops=1")
+    assert [k["kind"] for k in hip.code.kernels()] == ["mfma", "mfma"]
+    hip.step()
+    y = W.to_float(hip.get(Y), "bfloat16").astype(np.float64)
+    want = y @ W.to_float(init[3], "bfloat16").astype(np.float64).T
+    got = W.to_float(hip.get(Z), "bfloat16").astype(np.float64)
+    assert np.max(np.abs(got - want)) <= 2.0 ** -7 * np.max(np.abs(want))
+    hip.close()
