@@ -110,14 +110,14 @@ __device__ __forceinline__ void decode_batch(const GemmArgs& g, long z, long& ao
 
 // Grouped launch: blockIdx.z = group * batches + batch.  Returns the batch index and the operands of
 // the group (constant array indices only, as above).
-__device__ __forceinline__ long decode_group(const GemmArgs& g, long z, const void*& a, const void*& b, void*& c) {
-  a = g.a; b = g.b; c = g.c;
+__device__ __forceinline__ long decode_group(const GemmArgs& g, long z, const void*& a, const void*& b, void*& c, void*& c2) {
+  a = g.a; b = g.b; c = g.c; c2 = g.c2;
   if (g.ngroups > 1) {
     const long grp = z / g.batches;
     z -= grp * g.batches;
-    if (grp == 1) { a = g.a_more[0]; b = g.b_more[0]; c = g.c_more[0]; }
-    else if (grp == 2) { a = g.a_more[1]; b = g.b_more[1]; c = g.c_more[1]; }
-    else if (grp == 3) { a = g.a_more[2]; b = g.b_more[2]; c = g.c_more[2]; }
+    if (grp == 1) { a = g.a_more[0]; b = g.b_more[0]; c = g.c_more[0]; c2 = g.c2_more[0]; }
+    else if (grp == 2) { a = g.a_more[1]; b = g.b_more[1]; c = g.c_more[1]; c2 = g.c2_more[1]; }
+    else if (grp == 3) { a = g.a_more[2]; b = g.b_more[2]; c = g.c_more[2]; c2 = g.c2_more[2]; }
   }
   return z;
 }
@@ -239,13 +239,15 @@ __device__ __forceinline__ bf16x8 tr_fragment(const unsigned short* at_lane, int
 // origin + compile-time row/column: scalar registers) and one 32-bit per-lane offset computed
 // once.  ACC loads the whole row of tiles before the first store, so that TN * 16 reads are in
 // flight; CHECK guards ragged edges.
-enum : int { kOutF32 = 0, kOutBf16 = 1 };
+// kOutF32Copy: fp32 result plus its bf16 rounding at the same element offset of a second tensor.
+enum : int { kOutF32 = 0, kOutBf16 = 1, kOutF32Copy = 2 };
 
 template <int TN, int OUT, bool ACC, bool CHECK>
 __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, long ld, int lane,
-                                               long rows_left, long cols_left) {
+                                               long rows_left, long cols_left, void* origin2 = nullptr) {
   using T = typename std::conditional<OUT == kOutBf16, unsigned short, float>::type;
   T* const base = static_cast<T*>(origin);
+  unsigned short* const base2 = static_cast<unsigned short*>(origin2);
   const unsigned col = lane & 31, rb = (lane >> 5) * 4;
   const unsigned loff = rb * (unsigned)ld + col;
   // Pin the tiles to accumulation registers up to this point: without it the register allocator
@@ -278,6 +280,7 @@ __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, 
       if (!CHECK || ((long)(r + rb) < rows_left && (long)(j * 32 + col) < cols_left)) {
         if (OUT == kOutBf16) p[loff] = (unsigned short)f2bf(v);
         else p[loff] = v;
+        if (OUT == kOutF32Copy) (base2 + (long)r * ld + j * 32)[loff] = (unsigned short)f2bf(v);
       }
     });
     __builtin_amdgcn_sched_barrier(0);   // one tile's registers at a time
@@ -288,7 +291,7 @@ __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, 
 // wave-uniform switch: that bounds what the compiler can hoist above the branch to one row's
 // registers (hoisting all 256 accumulator reads above one up-front branch spills them).
 template <int TM, int TN>
-__device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, f32x16 (&acc)[TM][TN], long m, long n, long co, int lane) {
+__device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, void* c2base, f32x16 (&acc)[TM][TN], long m, long n, long co, int lane) {
   const long rows_left = g.M - m, cols_left = g.N - n;
   if (rows_left <= 0 || cols_left <= 0) return;
   const bool full = rows_left >= TM * 32 && cols_left >= TN * 32;
@@ -297,10 +300,13 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, f32x16 
   const long ld = to_ws ? g.N : g.c_row;
   const long first = to_ws ? (((long)blockIdx.z * g.splits + blockIdx.y) * g.M + m) * g.N + n : co + m * g.c_row + n;
   char* const origin = (to_ws ? reinterpret_cast<char*>(g.ws) : static_cast<char*>(cbase)) + first * (bf ? 2 : 4);
-  const int variant = (bf ? 4 : 0) + ((!to_ws && g.accumulate) ? 2 : 0) + (full ? 0 : 1);
+  const bool copy = !to_ws && !bf && c2base != nullptr;   // (with split-K the reduction pass writes the copy)
+  char* const origin2 = copy ? static_cast<char*>(c2base) + first * 2 : nullptr;
+  const int variant = (copy ? 8 : bf ? 4 : 0) + ((!to_ws && g.accumulate) ? 2 : 0) + (full ? 0 : 1);
   static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
     constexpr int i = decltype(ic)::value;
     void* o = origin + (long)i * 32 * ld * (bf ? 2 : 4);
+    void* o2 = origin2 + (long)i * 32 * ld * 2;
     const long rl = rows_left - i * 32;
     switch (variant) {
       case 0: store_tile_row<TN, kOutF32, false, false>(acc[i], o, ld, lane, rl, cols_left); break;
@@ -310,7 +316,11 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, f32x16 
       case 4: store_tile_row<TN, kOutBf16, false, false>(acc[i], o, ld, lane, rl, cols_left); break;
       case 5: store_tile_row<TN, kOutBf16, false, true>(acc[i], o, ld, lane, rl, cols_left); break;
       case 6: store_tile_row<TN, kOutBf16, true, false>(acc[i], o, ld, lane, rl, cols_left); break;
-      default: store_tile_row<TN, kOutBf16, true, true>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 7: store_tile_row<TN, kOutBf16, true, true>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 8: store_tile_row<TN, kOutF32Copy, false, false>(acc[i], o, ld, lane, rl, cols_left, o2); break;
+      case 9: store_tile_row<TN, kOutF32Copy, false, true>(acc[i], o, ld, lane, rl, cols_left, o2); break;
+      case 10: store_tile_row<TN, kOutF32Copy, true, false>(acc[i], o, ld, lane, rl, cols_left, o2); break;
+      default: store_tile_row<TN, kOutF32Copy, true, true>(acc[i], o, ld, lane, rl, cols_left, o2); break;
     }
     __builtin_amdgcn_sched_barrier(0);
   });
@@ -342,8 +352,8 @@ gemm_bf16_kernel(const GemmArgs g) {
   const long m0 = tmi * BM, n0 = tni * BN;
   long ao, bo, co;
   const void *abase, *bbase;
-  void* cbase;
-  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase), ao, bo, co);
+  void *cbase, *c2base;
+  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase, c2base), ao, bo, co);
   const AT* A = static_cast<const AT*>(abase) + ao;
   const BT* B = static_cast<const BT*>(bbase) + bo;
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
@@ -525,7 +535,7 @@ gemm_bf16_kernel(const GemmArgs g) {
   }
   OCANNL_STAMP(2);
 
-  epilogue<TM, TN>(g, cbase, acc, m0 + wm0, n0 + wn0, co, lane);
+  epilogue<TM, TN>(g, cbase, c2base, acc, m0 + wm0, n0 + wn0, co, lane);
   OCANNL_STAMP(3);
 }
 
@@ -590,8 +600,8 @@ gemm_f32_kernel(const GemmArgs g) {
   const long m0 = tmi * BM, n0 = tni * BN;
   long ao, bo, co;
   const void *abase, *bbase;
-  void* cbase;
-  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase), ao, bo, co);
+  void *cbase, *c2base;
+  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase, c2base), ao, bo, co);
   const float* A = static_cast<const float*>(abase) + ao;
   const float* B = static_cast<const float*>(bbase) + bo;
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
@@ -661,7 +671,7 @@ gemm_f32_kernel(const GemmArgs g) {
     __syncthreads();
   }
 
-  epilogue<TM, TN>(g, cbase, acc, m0 + wm0, n0 + wn0, co, lane);
+  epilogue<TM, TN>(g, cbase, c2base, acc, m0 + wm0, n0 + wn0, co, lane);
 }
 
 template <int BM, int BN, bool A_KC, bool B_KC>
@@ -677,8 +687,8 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const GemmArgs g) {
   const long m = idx / n4, n = (idx % n4) * 4;
   long ao, bo, co;
   const void *abase, *bbase;
-  void* cbase;
-  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase), ao, bo, co);
+  void *cbase, *c2base;
+  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase, c2base), ao, bo, co);
   f32x4 sum = {0, 0, 0, 0};
   for (int sp = 0; sp < g.splits; ++sp)
     sum += *reinterpret_cast<const f32x4*>(g.ws + (((long)blockIdx.z * g.splits + sp) * g.M + m) * g.N + n);
@@ -695,6 +705,10 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const GemmArgs g) {
     f32x4 v = sum;
     if (g.accumulate) v += *reinterpret_cast<const f32x4*>(C + off);
     *reinterpret_cast<f32x4*>(C + off) = v;
+    if (c2base) {
+      unsigned short* C2 = static_cast<unsigned short*>(c2base);
+      for (int q = 0; q < 4; ++q) C2[off + q] = (unsigned short)f2bf(v[q]);
+    }
   }
 }
 

@@ -29,6 +29,10 @@ struct GemmArgs {
   const void* a_more[3];
   const void* b_more[3];
   void* c_more[3];
+  // When not null: a bf16 tensor of C's shape that receives the rounded result at the same element
+  // offsets (C must be fp32).  It feeds later bf16 contractions that read C.
+  void* c2;
+  void* c2_more[3];
 };
 
 // Picks the kernel instance for the operand precisions / layouts and launches it on `stream`.

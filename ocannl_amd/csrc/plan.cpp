@@ -487,7 +487,8 @@ void account_bytes(const Routine& r, Phase& ph) {
 bool phase_touches(const Phase& ph, int node) {
   if (ph.kind == Phase::Fill) return ph.fill_node == node;
   if (ph.kind == Phase::Contraction) {
-    for (auto& m : ph.gemm.group) if (m.a.node == node || m.b.node == node || m.c.node == node) return true;
+    for (auto& m : ph.gemm.group) if (m.a.node == node || m.b.node == node || m.c.node == node || m.c_copy == node) return true;
+    if (ph.gemm.c_copy == node) return true;
     return ph.gemm.a.node == node || ph.gemm.b.node == node || ph.gemm.c.node == node;
   }
   std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
@@ -565,6 +566,7 @@ static void set_contraction_bytes(Phase& ph) {
   };
   ph.bytes = op_bytes(g.a, (double)g.M, (double)g.K) + op_bytes(g.b, (double)g.N, (double)g.K) +
              op_bytes(g.c, (double)g.M, (double)g.N) * (g.accumulate ? 2 : 1);
+  if (g.c_copy >= 0) ph.bytes += op_bytes(g.c, (double)g.M, (double)g.N) / prec_in_bytes(g.c.prec) * 2.0;
 }
 
 // De-virtualisation.  The optimiser inlines a contraction that is read once into its consumer as
@@ -1133,10 +1135,10 @@ void group_contractions(Plan& plan) {
     auto m = plan.mirrors.find(c.node);
     return m != plan.mirrors.end() && phase_touches(q, m->second);
   };
-  struct Member { GemmOperand a, b, c; };
+  using Member = GemmDesc::Member;
   auto members_of = [](const GemmDesc& g) {
-    std::vector<Member> v{{g.a, g.b, g.c}};
-    for (auto& m : g.group) v.push_back({m.a, m.b, m.c});
+    std::vector<Member> v{{g.a, g.b, g.c, g.c_copy}};
+    for (auto& m : g.group) v.push_back(m);
     return v;
   };
   // may the contraction `x` run at another place of phases (lo, hi), i.e. does nothing there touch
@@ -1145,6 +1147,7 @@ void group_contractions(Plan& plan) {
     for (size_t k = lo + 1; k < hi; ++k) {
       const Phase& mid = plan.phases[k];
       if (touches_result(mid, x.c) || writes_operand(mid, x.a) || writes_operand(mid, x.b)) return false;
+      if (x.c_copy >= 0 && phase_touches(mid, x.c_copy)) return false;
     }
     return true;
   };
@@ -1169,22 +1172,24 @@ void group_contractions(Plan& plan) {
       for (int b = 0; b < g.nbatch && candidate; ++b) candidate = h.batch_ext[b] == g.batch_ext[b];
       const std::vector<Member> mine = members_of(g);
       if (candidate) {
-        candidate = h.accumulate == g.accumulate;
+        candidate = h.accumulate == g.accumulate && (h.c_copy >= 0) == (g.c_copy >= 0);
         for (auto& x : mine) {
           const int xc = x.c.node, hc = h.c.node;
+          if (x.c_copy >= 0) candidate = candidate && h.a.node != x.c_copy && h.b.node != x.c_copy;
+          if (h.c_copy >= 0) candidate = candidate && x.a.node != h.c_copy && x.b.node != h.c_copy;
           candidate = candidate && hc != xc && source_of(h.a.node) != xc && source_of(h.b.node) != xc && h.a.node != xc && h.b.node != xc &&
                       source_of(x.a.node) != hc && source_of(x.b.node) != hc && x.a.node != hc && x.b.node != hc;
         }
       }
       if (!candidate) continue;
-      const Member joiner{h.a, h.b, h.c};
+      const Member joiner{h.a, h.b, h.c, h.c_copy};
       bool hoist = free_between(joiner, i, j), sink = false;
       if (!hoist) {
         sink = true;
         for (auto& x : mine) sink = sink && free_between(x, i, j);
       }
       if (!hoist && !sink) continue;
-      g.group.push_back({h.a, h.b, h.c});
+      g.group.push_back(joiner);
       p.bytes += q.bytes;
       p.flops = g.flops();
       p.label += " | " + q.label;
@@ -1309,8 +1314,8 @@ namespace {
 bool phase_writes(const Phase& ph, int node) {
   if (ph.kind == Phase::Fill) return ph.fill_node == node;
   if (ph.kind == Phase::Contraction) {
-    for (auto& m : ph.gemm.group) if (m.c.node == node) return true;
-    return ph.gemm.c.node == node;
+    for (auto& m : ph.gemm.group) if (m.c.node == node || m.c_copy == node) return true;
+    return ph.gemm.c.node == node || ph.gemm.c_copy == node;
   }
   auto writes = [&](const Phase& q) {
     std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
@@ -1410,6 +1415,30 @@ void use_bf16_copies(Routine& r, Plan& plan, Phase& ph, Bf16Copies& copies, int*
       op.prec = Prec::Bfloat16;
       set_contraction_bytes(ph);
       return;
+    }
+    // The tensor's last writer is a matrix-core contraction that stores all of it in fp32: its
+    // epilogue writes the rounded copy as well, instead of a conversion pass over the tensor.
+    for (int q = (int)plan.phases.size() - 1; q >= 0; --q) {
+      Phase& producer = plan.phases[q];
+      if (!phase_writes(producer, src.id)) continue;
+      GemmDesc& pg = producer.gemm;
+      int64_t written = pg.M * pg.N, total = 1;
+      for (int b = 0; b < pg.nbatch; ++b) written *= pg.batch_ext[b];
+      for (int64_t d : src.dims) total *= d;
+      if (producer.kind == Phase::Contraction && pg.c.node == src.id && pg.c_copy < 0 && pg.c.prec == Prec::Single &&
+          pg.c.offset == 0 && pg.c.static_terms.empty() && written == total) {
+        r.nodes.emplace(t.id, t);
+        plan.scratch.push_back(t);
+        pg.c_copy = t.id;
+        set_contraction_bytes(producer);
+        copies.copy_of[src.id] = t.id;
+        copies.made_at[src.id] = plan.phases.size();
+        op.node = t.id;
+        op.prec = Prec::Bfloat16;
+        set_contraction_bytes(ph);
+        return;
+      }
+      break;   // only the last writer can stand for the tensor's contents
     }
     Indices ix;
     std::vector<int> syms;

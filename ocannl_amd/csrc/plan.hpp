@@ -40,8 +40,11 @@ struct GemmDesc {
   // one input, their weight gradients) that ride in the same launch: {a, b, c} per extra member.  A
   // small contraction alone puts at most one workgroup on a compute unit; several together let
   // workgroups hide each other's memory latency.
-  struct Member { GemmOperand a, b, c; };
+  struct Member { GemmOperand a, b, c; int c_copy = -1; };
   std::vector<Member> group;
+  // >= 0: a bf16 scratch tensor of C's shape that the epilogue fills with the rounded result (C is
+  // fp32 and written whole): it feeds later bf16 contractions that read C, in place of a conversion pass
+  int c_copy = -1;
   double flops() const {
     double f = 2.0 * (double)M * (double)N * (double)K * (double)(1 + group.size());
     for (int i = 0; i < nbatch; ++i) f *= (double)batch_ext[i];

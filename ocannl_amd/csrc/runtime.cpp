@@ -244,9 +244,11 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
       }
       a.accumulate = g.accumulate ? 1 : 0;
       a.c_is_bf16 = g.c.prec == Prec::Bfloat16;
+      a.c2 = g.c_copy >= 0 ? rt.node_ptr.at(g.c_copy) : nullptr;
       a.ngroups = 1 + (int)g.group.size();
       for (size_t m = 0; m < g.group.size(); ++m) {
         a.a_more[m] = base(g.group[m].a); a.b_more[m] = base(g.group[m].b); a.c_more[m] = base(g.group[m].c);
+        a.c2_more[m] = g.group[m].c_copy >= 0 ? rt.node_ptr.at(g.group[m].c_copy) : nullptr;
       }
       // a bracketed contraction is timed without its split-K reduction (a kernel of its own)
       hip_check(launch_gemm(g, a, rt.gemm_ws, dev.stream, bracket ? rt.profile_events[rt.profile_used + 1] : nullptr),

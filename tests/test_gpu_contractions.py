@@ -232,3 +232,30 @@ def test_a_product_that_reads_another_products_result_is_not_grouped_with_it():
     got = W.to_float(hip.get(Z), "bfloat16").astype(np.float64)
     assert np.max(np.abs(got - want)) <= 2.0 ** -7 * np.max(np.abs(want))
     hip.close()
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 512), (136, 72, 200), (128, 128, 8192)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_producer_epilogue_writes_the_bf16_copy_its_consumer_reads(shape, accumulate):
+    # g (fp32) (+)= a b, then out = g w with bf16 w: the second contraction wants g in bf16, and the
+    # first one's epilogue (or its split-K reduction pass) writes that copy -- no conversion pass.
+    M, N, K = shape
+    L.reset_symbols(0)
+    A = L.Node(1, "a", "bfloat16", (M, K)); B = L.Node(2, "b", "bfloat16", (N, K)); G = L.Node(3, "g", "single", (M, N))
+    Wt = L.Node(4, "w", "bfloat16", (64, N)); Out = L.Node(5, "out", "single", (M, 64))
+    body = ([] if accumulate else [L.ZeroOut(G)]) + [_product_nest(A, B, G, M, N, K, True, True),
+                                                     L.ZeroOut(Out), _product_nest(G, Wt, Out, M, 64, N, True, True)]
+    r = L.Routine("producer_copy", body)
+    rng = np.random.default_rng(21)
+    init = {x.id: W.as_prec(rng.standard_normal(x.dims).astype(np.float32) / 4, x.prec) for x in (A, B, G, Wt)}
+    hip = HipRun(r, init, "min_mfma_flops=1")
+    assert [k["kind"] for k in hip.code.kernels()] == ["mfma", "mfma"], hip.code.kernels()
+    hip.step()
+    g = hip.get(G).astype(np.float64)
+    want_g = _f64(init[1], "bfloat16", True) @ _f64(init[2], "bfloat16", True).T + (init[3].astype(np.float64) if accumulate else 0.0)
+    assert np.max(np.abs(g - want_g)) <= 2e-6 * max(1.0, np.sqrt(K) / 8) * np.max(np.abs(want_g))
+    g_bf = W.to_float(W.as_prec(hip.get(G), "bfloat16"), "bfloat16").astype(np.float64)   # the copy: g as stored, rounded
+    want = g_bf @ _f64(init[4], "bfloat16", True).T
+    got = hip.get(Out).astype(np.float64)
+    assert np.max(np.abs(got - want)) <= 2e-6 * max(1.0, np.sqrt(N) / 8) * np.max(np.abs(want))
+    hip.close()

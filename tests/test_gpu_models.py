@@ -1,6 +1,9 @@
 """GPU parity of the language-model configurations at sizes the CPU checker finishes in seconds."""
 import numpy as np
 import pytest
+# PyTorch brings its own copy of the HIP runtime, which must be loaded before the backend library
+# brings up the system's: imported here (at collection), not inside the one test that uses it.
+import torch
 
 from ocannl_amd import workloads as W
 from parity import HipRun, OracleRun, rel_err
@@ -122,7 +125,6 @@ def test_full_size_attention_against_torch_autograd():
     # against plain PyTorch in fp32 on the same device: softmax(Q K^T / sqrt(d)) V and, through
     # autograd, dQ dK dV from the same d out. bf16 storage of scores / probabilities bounds the
     # agreement (Frobenius-relative 2e-2, as for every bf16 routine); rows of the soft-max sum to one.
-    import torch
     w = W.attention()
     hip = HipRun(w.routine, w.init)
     hip.step()
