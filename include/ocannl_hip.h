@@ -59,7 +59,9 @@ typedef struct {
   int32_t coop_lanes;      /* lanes cooperating on one output (generated reduction kernels)          */
   double flops;            /* algorithmic: 2 * product of all loop extents for a contraction         */
   double bytes;            /* algorithmic: distinct elements read once + written once, in bytes      */
-  int64_t m, n, k, batch;  /* contraction shape after symbol classification (0 otherwise)            */
+  int64_t m, n, k, batch;  /* contraction shape after symbol classification (0 otherwise); contractions
+                              sharing the launch count as batch entries, a chain of operand pairs into
+                              one result as a longer k                                                 */
   char name[96];
 } ocannl_hip_kernel_info;
 
@@ -109,7 +111,9 @@ int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** code);
    (lanes sharing reductions; off = the summation order of the serial C code), rows=0|1 (fusing
    consecutive row-wise phases into one kernel), bf16_copies=0|1 (rounding an fp32 operand of a
    bf16 contraction once into scratch instead of in every kernel that reads it), serial=0|1 (a routine
-   of tiny phases as one single-workgroup kernel), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
+   of tiny phases as one single-workgroup kernel), groups=0|1 (independent contractions of identical
+   shapes share a launch), chains=0|1 (`c =+ a * b` statements into one result with identical operand
+   shapes share a launch), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
    indices and offsets in generated kernels, the `large_models` setting of c_syntax.ml:111-112; a
    routine with a node of more than 2^31 - 1 elements gets them without asking). */
 int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, ocannl_hip_code** code);

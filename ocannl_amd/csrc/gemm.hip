@@ -331,7 +331,11 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, void* c
 // PF = 2: global loads run two K stages ahead in two register sets, for launches of at most one
 // workgroup per CU, where nothing else hides the HBM latency of a stage; that needs the whole
 // register file, so one wavefront per SIMD.
-template <int BM, int BN, typename AT, typename BT, bool A_KC, bool B_KC, int PF>
+// CHAIN: the launch accumulates several operand pairs into one C (`c =+ a_p * b_p`, p < npairs):
+// the K pipeline runs once per pair and the accumulators stay in registers in between.  Only the
+// 128x128 tile with two register sets is built that way (the loop around the pipeline costs
+// registers that the other variants do not have).
+template <int BM, int BN, typename AT, typename BT, bool A_KC, bool B_KC, int PF, bool CHAIN = false>
 __global__ void __launch_bounds__(kThreads)
 __attribute__((amdgpu_waves_per_eu((BM < 256 && sizeof(AT) == 2 && sizeof(BT) == 2 && PF == 1) ? 2 : 1,
                                    (BM >= 256 || PF > 1) ? 1 : 2)))
@@ -391,6 +395,10 @@ gemm_bf16_kernel(const GemmArgs g) {
   static_assert(PF == 1 || (PF == 2 && sizeof(AT) == 2 && sizeof(BT) == 2), "two register sets: bf16 sources only");
   Stager<BM, AT, A_KC> sa[kPF];
   Stager<BN, BT, B_KC> sb[kPF];
+  static_assert(!CHAIN || (BM == 128 && PF == 2), "chains: 128x128 tiles with two register sets");
+  // (the pipeline is a lambda so that the variants without chains hold no loop statement around it:
+  // a loop with one trip still cost the 256x256 variants registers)
+  auto pipeline = [&]() __attribute__((always_inline)) {
   sa[0].load(A, lda, m0, kbeg, g.M, kend, tid);
   sb[0].load(B, ldb, n0, kbeg, g.N, kend, tid);
   if (kPF > 1) {
@@ -532,6 +540,18 @@ gemm_bf16_kernel(const GemmArgs g) {
     long ks = 0;
     for (; ks + kPF <= ksteps; ks += kPF) static_for<kPF>([&](auto p) OCN_LAMBDA_INLINE { step(ks + decltype(p)::value, p); });
     static_for<kPF>([&](auto p) OCN_LAMBDA_INLINE { if (ks + decltype(p)::value < ksteps) step(ks + decltype(p)::value, p); });
+  }
+  };   // pipeline
+  if constexpr (CHAIN) {
+    for (int pair = 0; pair < g.npairs; ++pair) {
+      if (pair > 0) {
+        A = static_cast<const AT*>(pair == 1 ? g.a_more[0] : pair == 2 ? g.a_more[1] : g.a_more[2]) + ao;
+        B = static_cast<const BT*>(pair == 1 ? g.b_more[0] : pair == 2 ? g.b_more[1] : g.b_more[2]) + bo;
+      }
+      pipeline();
+    }
+  } else {
+    pipeline();
   }
   OCANNL_STAMP(2);
 
@@ -737,7 +757,7 @@ TileConfig tile_config(const GemmDesc& d) {
   const long t128 = ((d.M + 127) / 128) * ((d.N + 127) / 128) * nb;
   TileConfig c;
   const bool bf16_sources = d.a.prec == Prec::Bfloat16 && d.b.prec == Prec::Bfloat16;
-  if (t256 >= 256 && d.M > 128 && d.N > 128 && d.K >= 512) { c.big = true; c.splits = 1; }
+  if (d.more.empty() && t256 >= 256 && d.M > 128 && d.N > 128 && d.K >= 512) { c.big = true; c.splits = 1; }
   else {
     c.big = false;
     long s = 1;
@@ -756,6 +776,7 @@ TileConfig tile_config(const GemmDesc& d) {
   // two stages of global loads in flight when the launch puts at most one workgroup on a CU and
   // each runs at least 8 K stages (measured: 8192x512x2048 bf16 595 -> 738 TFLOP/s)
   c.prefetch = (!c.big && bf16_sources && t128 * c.splits <= 256 && d.K / c.splits >= 512) ? 2 : 1;
+  if (!d.more.empty()) c.prefetch = 2;   // the only variant built for chains
 #ifdef OCANNL_GEMM_TIMING
   if (g_force_prefetch) c.prefetch = (!c.big && bf16_sources) ? g_force_prefetch : 1;
 #endif
@@ -780,7 +801,7 @@ hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t
   const long tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   long nb = 1;
   for (int i = 0; i < a.nbatch; ++i) nb *= a.batch_ext[i];
-  if (a.ngroups < 1 || a.ngroups > 4) return hipErrorInvalidValue;
+  if (a.ngroups < 1 || a.ngroups > 4 || a.npairs < 1 || a.npairs > 4 || (a.npairs > 1 && a.ngroups > 1)) return hipErrorInvalidValue;
   a.batches = (int)nb;
   nb *= a.ngroups;
   if (tiles <= 0 || tiles > 0x7FFFFFFFL || nb <= 0 || nb > 65535) return hipErrorInvalidValue;
@@ -794,12 +815,12 @@ hipError_t launch(K kernel, size_t smem, int BM, int BN, GemmArgs a, hipStream_t
   return hipGetLastError();
 }
 
-template <int BM, int BN, typename AT, typename BT, int PF = 1>
+template <int BM, int BN, typename AT, typename BT, int PF = 1, bool CHAIN = false>
 hipError_t launch_bf16_layout(bool akc, bool bkc, const GemmArgs& a, hipStream_t s, hipEvent_t ev) {
-  if (akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, true, PF>, bf16_smem<BM, BN, true, true>(), BM, BN, a, s, ev);
-  if (akc && !bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, false, PF>, bf16_smem<BM, BN, true, false>(), BM, BN, a, s, ev);
-  if (!akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, true, PF>, bf16_smem<BM, BN, false, true>(), BM, BN, a, s, ev);
-  return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, false, PF>, bf16_smem<BM, BN, false, false>(), BM, BN, a, s, ev);
+  if (akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, true, PF, CHAIN>, bf16_smem<BM, BN, true, true>(), BM, BN, a, s, ev);
+  if (akc && !bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, true, false, PF, CHAIN>, bf16_smem<BM, BN, true, false>(), BM, BN, a, s, ev);
+  if (!akc && bkc) return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, true, PF, CHAIN>, bf16_smem<BM, BN, false, true>(), BM, BN, a, s, ev);
+  return launch(gemm_bf16_kernel<BM, BN, AT, BT, false, false, PF, CHAIN>, bf16_smem<BM, BN, false, false>(), BM, BN, a, s, ev);
 }
 
 template <int BM, int BN>
@@ -824,8 +845,8 @@ const char* gemm_kernel_name(const GemmDesc& d) {
   if (af && bf)
     snprintf(buf, sizeof buf, "gemm_f32_kernel<%d, %d, %s, %s>", tile, tile, tf[a_kcontig(d)], tf[b_kcontig(d)]);
   else
-    snprintf(buf, sizeof buf, "gemm_bf16_kernel<%d, %d, %s, %s, %s, %s, %d>", tile, tile, af ? "float" : "unsigned short",
-             bf ? "float" : "unsigned short", tf[a_kcontig(d)], tf[b_kcontig(d)], prefetch_depth(d));
+    snprintf(buf, sizeof buf, "gemm_bf16_kernel<%d, %d, %s, %s, %s, %s, %d, %s>", tile, tile, af ? "float" : "unsigned short",
+             bf ? "float" : "unsigned short", tf[a_kcontig(d)], tf[b_kcontig(d)], prefetch_depth(d), tf[!d.more.empty()]);
   return buf;
 }
 
@@ -857,7 +878,9 @@ hipError_t launch_gemm(const GemmDesc& d, const GemmArgs& a_in, void* workspace,
   }
   const bool af = d.a.prec == Prec::Single, bf = d.b.prec == Prec::Single;
   if (af && bf) return big ? launch_f32_layout<256, 256>(akc, bkc, a, s, ev) : launch_f32_layout<128, 128>(akc, bkc, a, s, ev);
+  if (a.npairs > 1 && (af || bf)) return hipErrorInvalidValue;   // chains: bf16 operands only
   if (!af && !bf) {
+    if (a.npairs > 1) return launch_bf16_layout<128, 128, unsigned short, unsigned short, 2, true>(akc, bkc, a, s, ev);
     if (big) return launch_bf16_layout<256, 256, unsigned short, unsigned short>(akc, bkc, a, s, ev);
     return prefetch_depth(d) == 2 ? launch_bf16_layout<128, 128, unsigned short, unsigned short, 2>(akc, bkc, a, s, ev)
                                   : launch_bf16_layout<128, 128, unsigned short, unsigned short>(akc, bkc, a, s, ev);

@@ -25,6 +25,9 @@ struct GemmArgs {
   // precisions: member g > 0 uses a_more / b_more / c_more[g - 1], and the grid's z axis is
   // member * batches + batch.
   int ngroups;       // >= 1
+  // A chain `c =+ a_p * b_p` into the same C (bf16 operands): K runs over a / b, then over
+  // a_more[p - 1] / b_more[p - 1].  Never together with ngroups > 1.
+  int npairs;        // >= 1
   int batches;       // product of batch_ext (set by launch_gemm)
   const void* a_more[3];
   const void* b_more[3];

@@ -489,6 +489,7 @@ bool phase_touches(const Phase& ph, int node) {
   if (ph.kind == Phase::Contraction) {
     for (auto& m : ph.gemm.group) if (m.a.node == node || m.b.node == node || m.c.node == node || m.c_copy == node) return true;
     if (ph.gemm.c_copy == node) return true;
+    for (auto& pr : ph.gemm.more) if (pr.first.node == node || pr.second.node == node) return true;
     return ph.gemm.a.node == node || ph.gemm.b.node == node || ph.gemm.c.node == node;
   }
   std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
@@ -1106,10 +1107,13 @@ void group_rows(const Routine& r, Plan& plan) {
 }  // namespace
 
 // ---- contractions that share a launch ---------------------------------------------------------------
-// Independent contractions of identical shapes, strides and precisions (the q / k / v projections of
-// one input; the weight gradients of those projections) ride in one launch whose z axis runs over
-// the members.  A small contraction alone puts at most one workgroup on a compute unit; several
-// together let workgroups hide each other's memory latency.
+// Two ways in which contractions of identical shapes, strides and precisions share a launch:
+//   * a group of independent ones (the q / k / v projections of one input; the weight gradients of
+//     those projections): the grid's z axis runs over the members.  A small contraction alone puts at
+//     most one workgroup on a compute unit; several together let workgroups hide each other's memory
+//     latency;
+//   * a chain `c =+ a1 * b1; c =+ a2 * b2; ...` into one result (the input gradient of a tensor that
+//     feeds several projections): K runs over every operand pair, C is read and written once.
 // The statements need not be adjacent.  A later one is hoisted to the earlier one's position when
 // nothing in between touches its result or writes its operands; otherwise the earlier ones are sunk
 // to the later position under the same condition on them.
@@ -1123,7 +1127,7 @@ bool same_layout(const GemmOperand& x, const GemmOperand& y) {
   return true;
 }
 
-void group_contractions(Plan& plan) {
+void merge_contractions(Plan& plan, bool chain) {
   std::map<int, int> mirror_source;   // bf16 copy -> the tensor whose stores keep it in step
   for (auto& kv : plan.mirrors) mirror_source[kv.second] = kv.first;
   auto source_of = [&](int node) { auto m = mirror_source.find(node); return m == mirror_source.end() ? node : m->second; };
@@ -1138,6 +1142,7 @@ void group_contractions(Plan& plan) {
   using Member = GemmDesc::Member;
   auto members_of = [](const GemmDesc& g) {
     std::vector<Member> v{{g.a, g.b, g.c, g.c_copy}};
+    for (auto& pr : g.more) v.push_back({pr.first, pr.second, g.c, g.c_copy});
     for (auto& m : g.group) v.push_back(m);
     return v;
   };
@@ -1155,23 +1160,32 @@ void group_contractions(Plan& plan) {
     if (plan.phases[i].kind != Phase::Contraction) continue;
     {
       const GemmDesc& g = plan.phases[i].gemm;
-      // grouping pays where a launch alone leaves compute units idle or with one workgroup each
-      double tiles = (double)((g.M + 127) / 128) * (double)((g.N + 127) / 128);
-      for (int b = 0; b < g.nbatch; ++b) tiles *= (double)g.batch_ext[b];
-      if (tiles > 256) continue;
+      if (chain ? !g.group.empty() : !g.more.empty()) continue;
+      if (chain) {
+        // the kernels built for operand-pair lists: bf16 operands, fp32 result
+        if (g.a.prec != Prec::Bfloat16 || g.b.prec != Prec::Bfloat16 || g.c.prec != Prec::Single) continue;
+      } else {
+        // grouping pays where a launch alone leaves compute units idle or with one workgroup each
+        double tiles = (double)((g.M + 127) / 128) * (double)((g.N + 127) / 128);
+        for (int b = 0; b < g.nbatch; ++b) tiles *= (double)g.batch_ext[b];
+        if (tiles > 256) continue;
+      }
     }
     bool sunk = false;
     for (size_t j = i + 1; j < plan.phases.size() && !sunk; ++j) {
       Phase& p = plan.phases[i];
       GemmDesc& g = p.gemm;
-      if (g.group.size() >= 3) break;
+      if (g.group.size() + g.more.size() >= 3) break;
       Phase& q = plan.phases[j];
       const GemmDesc& h = q.gemm;
-      bool candidate = q.kind == Phase::Contraction && h.group.empty() && h.M == g.M && h.N == g.N &&
+      bool candidate = q.kind == Phase::Contraction && h.group.empty() && h.more.empty() && h.M == g.M && h.N == g.N &&
                        h.K == g.K && h.nbatch == g.nbatch && same_layout(h.a, g.a) && same_layout(h.b, g.b) && same_layout(h.c, g.c);
       for (int b = 0; b < g.nbatch && candidate; ++b) candidate = h.batch_ext[b] == g.batch_ext[b];
       const std::vector<Member> mine = members_of(g);
-      if (candidate) {
+      if (candidate && chain)
+        candidate = h.accumulate && h.c_copy < 0 && h.c.node == g.c.node && h.c.offset == g.c.offset &&
+                    h.c.static_terms == g.c.static_terms && source_of(h.a.node) != g.c.node && source_of(h.b.node) != g.c.node;
+      if (candidate && !chain) {
         candidate = h.accumulate == g.accumulate && (h.c_copy >= 0) == (g.c_copy >= 0);
         for (auto& x : mine) {
           const int xc = x.c.node, hc = h.c.node;
@@ -1181,18 +1195,32 @@ void group_contractions(Plan& plan) {
                       source_of(x.a.node) != hc && source_of(x.b.node) != hc && x.a.node != hc && x.b.node != hc;
         }
       }
-      if (!candidate) continue;
+      if (!candidate) {
+        // someone else reads or writes C: the chain cannot reach past it
+        if (chain && (phase_touches(q, g.c.node) || (g.c_copy >= 0 && phase_touches(q, g.c_copy)))) break;
+        continue;
+      }
       const Member joiner{h.a, h.b, h.c, h.c_copy};
       bool hoist = free_between(joiner, i, j), sink = false;
       if (!hoist) {
         sink = true;
         for (auto& x : mine) sink = sink && free_between(x, i, j);
       }
-      if (!hoist && !sink) continue;
-      g.group.push_back(joiner);
-      p.bytes += q.bytes;
+      if (!hoist && !sink) {
+        if (chain) break;
+        continue;
+      }
+      if (chain) {
+        double c_bytes = (double)g.M * (double)g.N * prec_in_bytes(g.c.prec);
+        for (int b = 0; b < g.nbatch; ++b) c_bytes *= (double)g.batch_ext[b];
+        g.more.push_back({h.a, h.b});
+        p.bytes += q.bytes - 2.0 * c_bytes;   // C is read and written once less
+      } else {
+        g.group.push_back(joiner);
+        p.bytes += q.bytes;
+      }
       p.flops = g.flops();
-      p.label += " | " + q.label;
+      p.label += (chain ? " + " : " | ") + q.label;
       if (hoist) {
         plan.phases.erase(plan.phases.begin() + j);
         --j;
@@ -1640,7 +1668,8 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     }
     plan.phases.push_back(std::move(ph));
   }
-  if (opt.enable_mfma && opt.group_contractions) group_contractions(plan);
+  if (opt.enable_mfma && opt.merge_chains) merge_contractions(plan, true);
+  if (opt.enable_mfma && opt.group_contractions) merge_contractions(plan, false);
   if (opt.enable_coop && opt.enable_row_groups) group_rows(r, plan);
   if (opt.enable_serial_group) serialise_tiny(r, plan);
   return plan;

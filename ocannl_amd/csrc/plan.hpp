@@ -40,13 +40,17 @@ struct GemmDesc {
   // one input, their weight gradients) that ride in the same launch: {a, b, c} per extra member.  A
   // small contraction alone puts at most one workgroup on a compute unit; several together let
   // workgroups hide each other's memory latency.
+  // Further operand pairs of the same shapes, strides and precisions whose products go to the same C
+  // (`c =+ a_i * b_i` statements: the input gradient of a tensor that feeds several projections): one
+  // launch runs K over the first pair, then over these, and reads and writes C once.
+  std::vector<std::pair<GemmOperand, GemmOperand>> more;
   struct Member { GemmOperand a, b, c; int c_copy = -1; };
   std::vector<Member> group;
   // >= 0: a bf16 scratch tensor of C's shape that the epilogue fills with the rounded result (C is
   // fp32 and written whole): it feeds later bf16 contractions that read C, in place of a conversion pass
   int c_copy = -1;
   double flops() const {
-    double f = 2.0 * (double)M * (double)N * (double)K * (double)(1 + group.size());
+    double f = 2.0 * (double)M * (double)N * (double)K * (double)(1 + group.size()) * (double)(1 + more.size());
     for (int i = 0; i < nbatch; ++i) f *= (double)batch_ext[i];
     return f;
   }
@@ -102,6 +106,7 @@ struct PlanOptions {
   bool enable_row_groups = true;
   bool enable_serial_group = true;   // tiny routines as one single-workgroup kernel
   bool group_contractions = true;   // independent contractions of equal shapes as one launch
+  bool merge_chains = true;         // `c =+ a_i * b_i` chains of equal shapes as one launch
   bool large_models = false;        // 64-bit offsets in generated kernels even when every node is small
   bool enable_bf16_copies = true;   // keep bf16 copies of fp32 operands of mixed contractions (written by the producing kernels)
 };

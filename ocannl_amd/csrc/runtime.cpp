@@ -114,6 +114,7 @@ PlanOptions parse_options(const char* options) {
     else if (k == "serial") o.enable_serial_group = v != "0";
     else if (k == "large_models") o.large_models = v != "0";
     else if (k == "groups") o.group_contractions = v != "0";
+    else if (k == "chains") o.merge_chains = v != "0";
     else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
     else throw InvalidArgument("compile options: unknown key '" + k + "'");
   }
@@ -245,6 +246,8 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
       a.accumulate = g.accumulate ? 1 : 0;
       a.c_is_bf16 = g.c.prec == Prec::Bfloat16;
       a.c2 = g.c_copy >= 0 ? rt.node_ptr.at(g.c_copy) : nullptr;
+      a.npairs = 1 + (int)g.more.size();
+      for (size_t p = 0; p < g.more.size(); ++p) { a.a_more[p] = base(g.more[p].first); a.b_more[p] = base(g.more[p].second); }
       a.ngroups = 1 + (int)g.group.size();
       for (size_t m = 0; m < g.group.size(); ++m) {
         a.a_more[m] = base(g.group[m].a); a.b_more[m] = base(g.group[m].b); a.c_more[m] = base(g.group[m].c);
@@ -591,8 +594,8 @@ int ocannl_hip_code_kernel_info(ocannl_hip_code* code, int index, int kernel, oc
     info->bytes = ph.bytes;
     std::string name;
     if (ph.kind == Phase::Contraction) {
-      // grouped contractions read as more batch entries
-      info->m = ph.gemm.M; info->n = ph.gemm.N; info->k = ph.gemm.K;
+      // grouped contractions read as more batch entries, a chain of operand pairs as a longer K
+      info->m = ph.gemm.M; info->n = ph.gemm.N; info->k = ph.gemm.K * (int64_t)(1 + ph.gemm.more.size());
       info->batch = 1 + (int64_t)ph.gemm.group.size();
       for (int i = 0; i < ph.gemm.nbatch; ++i) info->batch *= ph.gemm.batch_ext[i];
       name = gemm_kernel_name(ph.gemm);
@@ -652,6 +655,7 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
       if (ph.kind != Phase::Contraction) continue;
       std::vector<const GemmOperand*> ops{&ph.gemm.a, &ph.gemm.b, &ph.gemm.c};
       for (auto& m : ph.gemm.group) { ops.push_back(&m.a); ops.push_back(&m.b); ops.push_back(&m.c); }
+      for (auto& pr : ph.gemm.more) { ops.push_back(&pr.first); ops.push_back(&pr.second); }
       for (const GemmOperand* op : ops)
         if (reinterpret_cast<uintptr_t>(rt->node_ptr.at(op->node)) % 16 != 0)
           throw UserError("hip backend link: node " + cr.r.node(op->node).ident +

@@ -259,3 +259,42 @@ def test_producer_epilogue_writes_the_bf16_copy_its_consumer_reads(shape, accumu
     got = hip.get(Out).astype(np.float64)
     assert np.max(np.abs(got - want)) <= 2e-6 * max(1.0, np.sqrt(N) / 8) * np.max(np.abs(want))
     hip.close()
+
+
+@pytest.mark.parametrize("shape", [(256, 384, 512), (136, 72, 200), (128, 128, 4096)])
+@pytest.mark.parametrize("layout", [(True, True), (True, False), (False, False)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_chain_of_products_into_one_result_is_one_launch(shape, layout, accumulate):
+    # c (+)= a0 b0; c =+ a1 b1; c =+ a2 b2 (the gradient of a tensor that feeds three projections),
+    # with a pointwise statement on an unrelated tensor in between: one launch runs K over the three
+    # operand pairs and touches c once; full, ragged and split-K shapes
+    M, N, K = shape
+    a_kc, b_kc = layout
+    L.reset_symbols(0)
+    As = [L.Node(1 + p, f"a{p}", "bfloat16", (M, K) if a_kc else (K, M)) for p in range(3)]
+    Bs = [L.Node(4 + p, f"b{p}", "bfloat16", (N, K) if b_kc else (K, N)) for p in range(3)]
+    C = L.Node(7, "c", "single", (M, N)); U = L.Node(8, "u", "single", (64,))
+    i = L.fresh_symbol()
+    bump = L.For(i, 0, 63, [L.Set(U, (L.It(i),), L.Binop("add", L.Get(U, (L.It(i),)), L.Const(1.0)))])
+    body = ([] if accumulate else [L.ZeroOut(C)]) + [_product_nest(As[0], Bs[0], C, M, N, K, a_kc, b_kc), bump] + \
+        [_product_nest(As[p], Bs[p], C, M, N, K, a_kc, b_kc) for p in (1, 2)]
+    r = L.Routine("chain", body)
+    rng = np.random.default_rng(11)
+    init = {x.id: W.as_prec(rng.standard_normal(x.dims).astype(np.float32), "bfloat16") for x in As + Bs}
+    init[C.id] = rng.standard_normal(C.dims).astype(np.float32)
+    init[U.id] = np.zeros(64, np.float32)
+    want = sum(_f64(init[As[p].id], "bfloat16", a_kc) @ _f64(init[Bs[p].id], "bfloat16", b_kc).T for p in range(3))
+    if accumulate:
+        want = want + init[C.id].astype(np.float64)
+    for opts, launches in (("min_mfma_flops=1", 1), ("min_mfma_flops=1;chains=0", 3)):
+        hip = HipRun(r, init, opts)
+        ks = hip.code.kernels()
+        assert sorted(k["kind"] for k in ks) == ["generated"] + ["mfma"] * launches, ks
+        if launches == 1:
+            mf = [k for k in ks if k["kind"] == "mfma"][0]
+            assert mf["k"] == 3 * K and mf["flops"] == 6.0 * M * N * K and mf["name"].endswith("2, true>")
+        hip.step()
+        got = hip.get(C).astype(np.float64)
+        assert np.max(np.abs(got - want)) <= 2e-6 * max(1.0, np.sqrt(3 * K) / 8) * np.max(np.abs(want)), launches
+        assert np.array_equal(hip.get(U), np.ones(64, np.float32))
+        hip.close()
