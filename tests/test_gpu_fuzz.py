@@ -167,3 +167,91 @@ def test_random_contractions_against_float64(seed):
         err = float(np.abs(got - W.to_float(ora.get(c), c.prec)).max())
     assert err <= tol * scale, (seed, spec, a, b, c, kinds, err, scale)
     hip.close()
+
+
+def _contraction_sequence(seed):
+    """8-14 statements over a family of 128 x 128 tensors: matrix products (either operand stored
+    row- or k-contiguous, bf16 or fp32, from zero or on top of the result) and pointwise statements
+    that overwrite operands and results in between -- so that products which may share a launch, and
+    products which only look as if they might, both occur.  Returns the routine, its nodes and a
+    float64 model of the statements (values as stored: fp32 / bf16 rounded)."""
+    from ocannl_amd import llir as L
+    rng = np.random.default_rng(seed)
+    L.reset_symbols(0)
+    S = 128
+    bf = [L.Node(1 + k, n, "bfloat16", (S, S)) for k, n in enumerate(("x0", "x1", "w0", "w1"))]
+    f32 = [L.Node(5 + k, n, "single", (S, S)) for k, n in enumerate(("g0", "g1", "y0", "y1", "y2"))]
+    pick = lambda xs: xs[int(rng.integers(len(xs)))]
+    rbf = lambda v: W.to_float(W.as_prec(np.asarray(v, np.float32), "bfloat16"), "bfloat16").astype(np.float64)
+    body, model = [], []
+    for k in range(int(rng.integers(8, 15))):
+        body.append(L.Comment(f"statement {k}"))
+        i, j = L.fresh_symbol(), L.fresh_symbol()
+        u = rng.random()
+        if u < 0.65:
+            c = pick(f32)
+            a = pick([n for n in bf + f32 if n is not c])
+            b = pick([n for n in bf + f32[:2] if n is not c and n is not a])
+            a_kc, b_kc, zero = bool(rng.random() < 0.5), bool(rng.random() < 0.5), bool(rng.random() < 0.3)
+            kk = L.fresh_symbol()
+            ai = (L.It(i), L.It(kk)) if a_kc else (L.It(kk), L.It(i))
+            bi = (L.It(j), L.It(kk)) if b_kc else (L.It(kk), L.It(j))
+            if zero:
+                body.append(L.ZeroOut(c))
+            body.append(L.For(i, 0, S - 1, [L.For(j, 0, S - 1, [L.For(kk, 0, S - 1, [L.Set(c, (L.It(i), L.It(j)), L.Ternop(
+                "fma", L.Get(a, ai), L.Get(b, bi), L.Get(c, (L.It(i), L.It(j)))))])])]))
+            def product(v, a=a, b=b, c=c, a_kc=a_kc, b_kc=b_kc, zero=zero):
+                low = "bfloat16" in (a.prec, b.prec)     # the matrix cores then take both operands in bf16
+                av, bv = (rbf(v[n.id]) if low else v[n.id] for n in (a, b))
+                av, bv = (av if a_kc else av.T), (bv if b_kc else bv.T)
+                v[c.id] = ((0.0 if zero else v[c.id]) + av @ bv.T).astype(np.float32).astype(np.float64)
+            model.append(product)
+        elif u < 0.85:
+            d, s1, s2 = pick(f32), pick(bf + f32), pick(bf + f32)
+            at = lambda n: L.Get(n, (L.It(i), L.It(j)))
+            body.append(L.For(i, 0, S - 1, [L.For(j, 0, S - 1, [L.Set(d, (L.It(i), L.It(j)), L.Binop(
+                "add", L.Binop("mul", L.Const(0.5), at(s1)), L.Binop("mul", L.Const(0.25), at(s2))))])]))
+            def blend(v, d=d, s1=s1, s2=s2):
+                f = lambda n: v[n.id].astype(np.float32)
+                v[d.id] = (np.float32(0.5) * f(s1) + np.float32(0.25) * f(s2)).astype(np.float64)
+            model.append(blend)
+        else:
+            d, s1 = pick(bf), pick(f32)
+            body.append(L.For(i, 0, S - 1, [L.For(j, 0, S - 1, [L.Set(d, (L.It(i), L.It(j)), L.Binop(
+                "mul", L.Const(0.5), L.Get(s1, (L.It(i), L.It(j)))))])]))
+            def halve(v, d=d, s1=s1):
+                v[d.id] = rbf(np.float32(0.5) * v[s1.id].astype(np.float32))
+            model.append(halve)
+    return L.Routine(f"products_{seed}", body), bf + f32, model
+
+
+@pytest.mark.parametrize("seed", range(4000, 4000 + 2 * int(__import__("os").environ.get("FUZZ_SEEDS", 24))))
+def test_random_sequences_of_products_that_may_share_launches(seed):
+    # the planner moves products to one another's position to merge them into one launch: results must
+    # not depend on that.  Judges: a float64 model of the statements, and the same routine planned with
+    # every product as a launch of its own.
+    r, nodes, model = _contraction_sequence(seed)
+    rng = np.random.default_rng(seed + 3)
+    init = {n.id: W.as_prec((rng.uniform(-1, 1, n.dims) / 8).astype(np.float32), n.prec) for n in nodes}
+    v = {n.id: W.to_float(init[n.id], n.prec).astype(np.float64) for n in nodes}
+    for step in model:
+        step(v)
+    nodes = [n for n in nodes if n.id in {m.id for m in r.param_nodes()}]     # (the ones the routine uses)
+    outs, launches = {}, {}
+    for options in ("min_mfma_flops=1", "min_mfma_flops=1;groups=0;chains=0"):
+        hip = HipRun(r, init, options)
+        launches[options] = len(hip.code.kernels())
+        hip.step()
+        outs[options] = {n.id: W.to_float(hip.get(n), n.prec).astype(np.float64) for n in nodes}
+        hip.close()
+    merged, separate = outs.values()
+    assert launches["min_mfma_flops=1"] <= launches["min_mfma_flops=1;groups=0;chains=0"]
+    for n in nodes:
+        scale = max(float(np.abs(v[n.id]).max()), 1e-3)
+        # (values pass through bf16 tensors and fp32 operands are rounded to bf16 for the matrix cores:
+        # where the model's and the device's fp32 values differ in the last bit, such a rounding can
+        # flip, and the flip travels on; a missed dependence shows as an error of order one)
+        tol = 2.0 ** -7
+        for label, got in (("merged", merged), ("separate", separate)):
+            err = float(np.abs(got[n.id] - v[n.id]).max())
+            assert err <= tol * scale, (seed, n.ident, label, err, scale, launches)
