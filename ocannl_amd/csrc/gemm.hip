@@ -127,14 +127,16 @@ __device__ __forceinline__ long decode_group(const GemmArgs& g, long z, const vo
 // on the host so that the operand panels shared inside a rectangle are the expensive ones
 // (fewest bytes re-read across XCDs).  Inside its rectangle an XCD walks column-bands of 8
 // row-tiles, so that tiles running at the same time share B panels.
-__device__ __forceinline__ void tile_of_block(long wg, long tiles_m, long tiles_n, int xcd_m, long& tm, long& tn) {
+// `nx`: the number of XCDs the tile grid is spread over (8, or fewer when the members of a grouped
+// launch each keep to their own XCDs); wg % nx then names the XCD among them.
+__device__ __forceinline__ void tile_of_block(long wg, long tiles_m, long tiles_n, int xcd_m, int nx, long& tm, long& tn) {
   long t = wg, rm = tiles_m, rn = tiles_n, m_off = 0, n_off = 0;
   if (xcd_m > 0) {
-    const int xcd_n = 8 / xcd_m;
-    const long x = wg % 8;
+    const int xcd_n = nx / xcd_m;
+    const long x = wg % nx;
     rm = tiles_m / xcd_m; rn = tiles_n / xcd_n;
     m_off = (x / xcd_n) * rm; n_off = (x % xcd_n) * rn;
-    t = wg / 8;
+    t = wg / nx;
   }
   constexpr long kGroup = 8;
   const long band = kGroup * rn;
@@ -144,6 +146,22 @@ __device__ __forceinline__ void tile_of_block(long wg, long tiles_m, long tiles_
   const long r = t % band;
   tm = m_off + first_m + r % gm;
   tn = n_off + r / gm;
+}
+
+// Workgroup -> (tile-grid workgroup id, z index = member * batches + batch, XCDs sharing the grid).
+// Grouped launches with member_xcds > 0 give each member XCDs of its own (member m owns XCDs
+// m * member_xcds ... ): its operand panels then fill 8 / ngroups L2 caches instead of all eight.
+// The hardware deals workgroups to the XCDs round robin in dispatch order (x fastest, then z here:
+// such launches have no split along y).
+__device__ __forceinline__ void place_workgroup(const GemmArgs& g, long& wg, long& z, int& nx) {
+  wg = blockIdx.x; z = blockIdx.z; nx = 8;
+  if (g.member_xcds > 0) {
+    const long linear = z * gridDim.x + wg;
+    const long xcd = linear & 7, slot = linear >> 3;
+    nx = g.member_xcds;
+    z = xcd / nx;                 // the member (one batch entry each)
+    wg = slot * nx + xcd % nx;
+  }
 }
 
 // ---- staging one operand tile: global -> registers -> LDS --------------------------------------
@@ -351,13 +369,15 @@ gemm_bf16_kernel(const GemmArgs g) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
   const long tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-  long tmi, tni;
-  tile_of_block(blockIdx.x, tiles_m, tiles_n, g.xcd_m, tmi, tni);
+  long tmi, tni, wg, zz;
+  int nx;
+  place_workgroup(g, wg, zz, nx);
+  tile_of_block(wg, tiles_m, tiles_n, g.xcd_m, nx, tmi, tni);
   const long m0 = tmi * BM, n0 = tni * BN;
   long ao, bo, co;
   const void *abase, *bbase;
   void *cbase, *c2base;
-  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase, c2base), ao, bo, co);
+  decode_batch(g, decode_group(g, zz, abase, bbase, cbase, c2base), ao, bo, co);
   const AT* A = static_cast<const AT*>(abase) + ao;
   const BT* B = static_cast<const BT*>(bbase) + bo;
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
@@ -615,13 +635,15 @@ gemm_f32_kernel(const GemmArgs g) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
   const long tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-  long tmi, tni;
-  tile_of_block(blockIdx.x, tiles_m, tiles_n, g.xcd_m, tmi, tni);
+  long tmi, tni, wg, zz;
+  int nx;
+  place_workgroup(g, wg, zz, nx);
+  tile_of_block(wg, tiles_m, tiles_n, g.xcd_m, nx, tmi, tni);
   const long m0 = tmi * BM, n0 = tni * BN;
   long ao, bo, co;
   const void *abase, *bbase;
   void *cbase, *c2base;
-  decode_batch(g, decode_group(g, blockIdx.z, abase, bbase, cbase, c2base), ao, bo, co);
+  decode_batch(g, decode_group(g, zz, abase, bbase, cbase, c2base), ao, bo, co);
   const float* A = static_cast<const float*>(abase) + ao;
   const float* B = static_cast<const float*>(bbase) + bo;
   const long lda = A_KC ? g.a_row : g.a_k, ldb = B_KC ? g.b_row : g.b_k;
@@ -867,10 +889,19 @@ hipError_t launch_gemm(const GemmDesc& d, const GemmArgs& a_in, void* workspace,
     const long tile = big ? 256 : 128;
     const long tiles_m = (d.M + tile - 1) / tile, tiles_n = (d.N + tile - 1) / tile;
     const double a_bytes = (double)d.M * prec_in_bytes(d.a.prec), b_bytes = (double)d.N * prec_in_bytes(d.b.prec);
+    // a grouped launch of 2 or 4 unbatched members without a K split: each member on 4 or 2 XCDs of
+    // its own, so that its panels are fetched into that many L2 caches instead of all eight
+    const int members = 1 + (int)d.group.size();
+    int nx = 8;
+    a.member_xcds = 0;
+    if ((members == 2 || members == 4) && d.nbatch == 0 && a.splits == 1 && (tiles_m * tiles_n) % (8 / members) == 0) {
+      nx = 8 / members;
+      a.member_xcds = nx;
+    }
     a.xcd_m = 0;
     double best = 0;
-    for (int xm = 1; xm <= 8; xm *= 2) {
-      const int xn = 8 / xm;
+    for (int xm = 1; xm <= nx; xm *= 2) {
+      const int xn = nx / xm;
       if (tiles_m % xm || tiles_n % xn) continue;
       const double cost = a_bytes * xn + b_bytes * xm;
       if (a.xcd_m == 0 || cost < best) { a.xcd_m = xm; best = cost; }

@@ -19,6 +19,7 @@ struct GemmArgs {
   int accumulate;    // beta = 1
   int c_is_bf16;
   int xcd_m;         // tile-grid rows of the XCD partition (set by launch_gemm; 0: none)
+  int member_xcds;   // > 0: every member of a grouped launch keeps to this many XCDs of its own (set by launch_gemm)
   int splits;        // split-K factor (set by launch_gemm)
   float* ws;         // split-K workspace [batch][split][M][N] (set by launch_gemm)
   // One launch may cover up to four independent contractions of identical shapes, strides and

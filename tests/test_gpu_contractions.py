@@ -167,23 +167,27 @@ def _f64(x, prec, kc):
     return v if kc else v.T
 
 
-@pytest.mark.parametrize("shape", [(256, 384, 512), (136, 72, 200), (128, 128, 4096)])
+@pytest.mark.parametrize("shape", [(256, 384, 512), (136, 72, 200), (128, 128, 4096), (512, 256, 256)])
 @pytest.mark.parametrize("layout", [(True, True), (True, False), (False, False)])
 @pytest.mark.parametrize("precs", [("bfloat16", "single", True), ("bfloat16", "bfloat16", False), ("single", "single", False)])
-def test_independent_products_of_one_shape_share_a_launch(shape, layout, precs):
-    # y_g (+)= x w_g for three weights, with a pointwise statement on an unrelated tensor in between
+@pytest.mark.parametrize("members", [2, 3, 4])
+def test_independent_products_of_one_shape_share_a_launch(shape, layout, precs, members):
+    # y_g (+)= x w_g for two to four weights, with a pointwise statement on an unrelated tensor in
+    # between.  (Two or four members whose tile count allows it each keep to XCDs of their own: the
+    # workgroup -> member / tile mapping differs from the plain one.)
     M, N, K = shape
     a_kc, b_kc = layout
     prec, c_prec, accumulate = precs
+    G = members
     L.reset_symbols(0)
     X = L.Node(1, "x", prec, (M, K) if a_kc else (K, M))
-    Ws = [L.Node(2 + g, f"w{g}", prec, (N, K) if b_kc else (K, N)) for g in range(3)]
-    Ys = [L.Node(5 + g, f"y{g}", c_prec, (M, N)) for g in range(3)]
-    U = L.Node(8, "u", "single", (64,))
+    Ws = [L.Node(2 + g, f"w{g}", prec, (N, K) if b_kc else (K, N)) for g in range(G)]
+    Ys = [L.Node(6 + g, f"y{g}", c_prec, (M, N)) for g in range(G)]
+    U = L.Node(10, "u", "single", (64,))
     i = L.fresh_symbol()
     bump = L.For(i, 0, 63, [L.Set(U, (L.It(i),), L.Binop("add", L.Get(U, (L.It(i),)), L.Const(1.0)))])
     body = []
-    for g in range(3):
+    for g in range(G):
         if not accumulate:
             body.append(L.ZeroOut(Ys[g]))
         body.append(_product_nest(X, Ws[g], Ys[g], M, N, K, a_kc, b_kc))
@@ -195,7 +199,7 @@ def test_independent_products_of_one_shape_share_a_launch(shape, layout, precs):
     init[U.id] = np.zeros(64, np.float32)
     x64 = _f64(init[X.id], prec, a_kc)
     outs = {}
-    for opts, launches in (("min_mfma_flops=1", 1), ("min_mfma_flops=1;groups=0", 3)):
+    for opts, launches in (("min_mfma_flops=1", 1), ("min_mfma_flops=1;groups=0", G)):
         hip = HipRun(r, init, opts)
         ks = hip.code.kernels()
         assert sorted(k["kind"] for k in ks) == ["generated"] + ["mfma"] * launches, ks
@@ -204,15 +208,15 @@ def test_independent_products_of_one_shape_share_a_launch(shape, layout, precs):
         assert np.array_equal(hip.get(U), np.ones(64, np.float32))
         hip.close()
     tol = 2.0 ** -8 if c_prec == "bfloat16" else 2e-6 * max(1.0, np.sqrt(K) / 8)
-    for g in range(3):
+    for g in range(G):
         want = x64 @ _f64(init[Ws[g].id], prec, b_kc).T
         if accumulate:
             want = want + W.to_float(init[Ys[g].id], c_prec).astype(np.float64)
         for got in outs.values():
             assert np.max(np.abs(got[g] - want)) <= tol * np.max(np.abs(want)), (g, layout, precs)
     # grouped and separate launches sum in the same order: identical bits
-    for g in range(3):
-        assert np.array_equal(outs[1][g], outs[3][g])
+    for g in range(G):
+        assert np.array_equal(outs[1][g], outs[G][g])
 
 
 def test_a_product_that_reads_another_products_result_is_not_grouped_with_it():
