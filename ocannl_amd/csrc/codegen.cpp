@@ -873,6 +873,21 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
       }
       pr.shadow.clear(); pr.shadow_live.clear();
       total_threads = 256;
+    } else if (!ph.parallel_members.empty()) {
+      // ---- independent phases side by side: every member owns a range of whole workgroups
+      body.push_back(ind + "const uint64_t g_ = ((uint64_t)blockIdx.y * gridDim.x + blockIdx.x) * blockDim.x + threadIdx.x;");
+      uint64_t first = 0;
+      for (auto& q : ph.parallel_members) {
+        uint64_t qt = (uint64_t)q.coop_lanes;
+        for (auto e : (q.members.empty() ? q.par_ext : q.row_outer_ext)) qt *= (uint64_t)e;
+        const uint64_t end = first + (qt + 255) / 256 * 256;
+        body.push_back(ind + (first ? "else if" : "if") + " (g_ < " + std::to_string(end) + "ull) {  /* " + q.label + " */");
+        body.push_back(ind + "  const uint64_t gtid_ = g_ - " + std::to_string(first) + "ull;");
+        emit_points(q, ind + "  ", "return");
+        body.push_back(ind + "}");
+        first = end;
+      }
+      total_threads = first;
     } else {
       body.push_back(ind + "const uint64_t gtid_ = ((uint64_t)blockIdx.y * gridDim.x + blockIdx.x) * blockDim.x + threadIdx.x;");
       total_threads = emit_points(ph, ind, "return");

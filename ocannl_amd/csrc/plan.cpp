@@ -492,6 +492,7 @@ bool phase_touches(const Phase& ph, int node) {
     for (auto& pr : ph.gemm.more) if (pr.first.node == node || pr.second.node == node) return true;
     return ph.gemm.a.node == node || ph.gemm.b.node == node || ph.gemm.c.node == node;
   }
+  if (!ph.parallel_members.empty()) { for (auto& m : ph.parallel_members) if (phase_touches(m, node)) return true; return false; }
   std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
   block_accesses(ph.inner, acc, w, f, d);
   if (w) return true;   // a Zero_out inside the nest: not tracked per node, assume the worst
@@ -1330,6 +1331,86 @@ void serialise_tiny(const Routine& r, Plan& plan) {
 
 }  // namespace
 
+// ---- independent small phases ------------------------------------------------------------------------
+// A run of consecutive small generated phases none of which touches what another writes (the updates
+// of the many small parameters of a model, the finishing touches of bias gradients) becomes one
+// kernel: each member owns a range of workgroups, so they run side by side instead of as launches of
+// a few microseconds each in a row.
+namespace {
+
+void group_independent(const Routine& r, Plan& plan) {
+  (void)r;
+  if (plan.phases.size() < 2) return;
+  struct Sets { std::set<int> reads, writes; bool ok = false; };
+  auto add_accesses = [&](const Phase& ph, Sets& s) {
+    std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+    block_accesses(ph.inner, acc, w, f, d);
+    if (w || f) return false;
+    for (auto& a : acc) {
+      (a.write ? s.writes : s.reads).insert(a.node);
+      if (a.write) { auto m = plan.mirrors.find(a.node); if (m != plan.mirrors.end()) s.writes.insert(m->second); }
+    }
+    return true;
+  };
+  auto sets_of = [&](const Phase& ph) {
+    Sets s;
+    if (ph.kind != Phase::Generic || !ph.serial_members.empty() || !ph.parallel_members.empty()) return s;
+    if (ph.bytes > (double)(32 << 20)) return s;
+    bool ok = true;
+    if (ph.members.empty()) ok = add_accesses(ph, s);
+    else for (auto& m : ph.members) ok = ok && add_accesses(m, s);
+    s.ok = ok;
+    return s;
+  };
+  auto disjoint = [](const std::set<int>& x, const std::set<int>& y) {
+    for (int v : x) if (y.count(v)) return false;
+    return true;
+  };
+  std::vector<Sets> sets;
+  for (auto& ph : plan.phases) sets.push_back(sets_of(ph));
+  std::vector<Phase> out;
+  size_t i = 0;
+  while (i < plan.phases.size()) {
+    if (!sets[i].ok) { out.push_back(std::move(plan.phases[i])); ++i; continue; }
+    size_t j = i;
+    while (j < plan.phases.size() && sets[j].ok) ++j;
+    // [i, j): a window of eligible phases.  A phase's level is one more than the highest level among
+    // the earlier phases of the window it conflicts with, so phases of one level are independent and
+    // conflicting phases keep their order when the levels run one after the other.
+    std::vector<int> level(j - i, 0);
+    int top = 0;
+    for (size_t k = i; k < j; ++k) {
+      for (size_t e = i; e < k; ++e) {
+        const bool conflict = !disjoint(sets[k].writes, sets[e].reads) || !disjoint(sets[k].writes, sets[e].writes) ||
+                              !disjoint(sets[e].writes, sets[k].reads);
+        if (conflict) level[k - i] = std::max(level[k - i], level[e - i] + 1);
+      }
+      top = std::max(top, level[k - i]);
+    }
+    for (int lv = 0; lv <= top; ++lv) {
+      std::vector<size_t> same;
+      for (size_t k = i; k < j; ++k) if (level[k - i] == lv) same.push_back(k);
+      for (size_t c = 0; c < same.size(); c += 32) {
+        const size_t n = std::min<size_t>(32, same.size() - c);
+        if (n == 1) { out.push_back(std::move(plan.phases[same[c]])); continue; }
+        Phase g;
+        g.kind = Phase::Generic;
+        g.label = std::to_string(n) + " independent phases side by side";
+        for (size_t q = c; q < c + n; ++q) {
+          g.bytes += plan.phases[same[q]].bytes;
+          g.flops += plan.phases[same[q]].flops;
+          g.parallel_members.push_back(std::move(plan.phases[same[q]]));
+        }
+        out.push_back(std::move(g));
+      }
+    }
+    i = j;
+  }
+  plan.phases = std::move(out);
+}
+
+}  // namespace
+
 // ---- bf16 copies of fp32 contraction operands -----------------------------------------------------
 // A contraction with one fp32 and one bf16 operand runs on the bf16 matrix cores: the fp32
 // operand is rounded to bf16 on the way in.  Doing that rounding once, in a pass of its own into a
@@ -1353,6 +1434,7 @@ bool phase_writes(const Phase& ph, int node) {
     return false;
   };
   if (!ph.members.empty()) { for (auto& m : ph.members) if (writes(m)) return true; return false; }
+  if (!ph.parallel_members.empty()) { for (auto& m : ph.parallel_members) if (writes(m)) return true; return false; }
   return writes(ph);
 }
 
@@ -1672,6 +1754,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
   if (opt.enable_mfma && opt.group_contractions) merge_contractions(plan, false);
   if (opt.enable_coop && opt.enable_row_groups) group_rows(r, plan);
   if (opt.enable_serial_group) serialise_tiny(r, plan);
+  if (opt.enable_coop && opt.enable_parallel_groups) group_independent(r, plan);
   return plan;
 }
 

@@ -91,6 +91,10 @@ struct Phase {
   // shadowed in LDS (node -> index of the member that makes the shadow valid): later members read
   // the shadow instead of waiting on global memory; every store still goes to global memory too.
   std::map<int, int> serial_shadows;
+  // Parallel group (kind Generic, `parallel_members` non-empty): consecutive small phases that do not
+  // depend on one another (the updates of many small parameters) run as ONE kernel in which every
+  // member owns a range of workgroups.
+  std::vector<Phase> parallel_members;
   // Fill
   int fill_node = -1;
   // Contraction
@@ -107,6 +111,7 @@ struct PlanOptions {
   bool enable_serial_group = true;   // tiny routines as one single-workgroup kernel
   bool group_contractions = true;   // independent contractions of equal shapes as one launch
   bool merge_chains = true;         // `c =+ a_i * b_i` chains of equal shapes as one launch
+  bool enable_parallel_groups = true;   // consecutive independent small phases as one launch
   bool large_models = false;        // 64-bit offsets in generated kernels even when every node is small
   bool enable_bf16_copies = true;   // keep bf16 copies of fp32 operands of mixed contractions (written by the producing kernels)
 };

@@ -115,6 +115,7 @@ PlanOptions parse_options(const char* options) {
     else if (k == "large_models") o.large_models = v != "0";
     else if (k == "groups") o.group_contractions = v != "0";
     else if (k == "chains") o.merge_chains = v != "0";
+    else if (k == "parallel") o.enable_parallel_groups = v != "0";
     else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
     else throw InvalidArgument("compile options: unknown key '" + k + "'");
   }

@@ -24,9 +24,11 @@ def test_library_exports_every_declared_symbol():
 
 def test_compile_needs_no_gpu_and_reports_kernels():
     w = W.moons_mlp()
-    code = B.compile(w.routine, "serial=0")
+    code = B.compile(w.routine, "serial=0;parallel=0")
     ks = code.kernels()
     assert len(ks) > 10 and all(k["kind"] in ("generated", "fill") for k in ks)
+    # independent small phases share launches
+    assert len(B.compile(w.routine, "serial=0").kernels()) < len(ks)
     # by default a routine of tiny phases becomes ONE single-workgroup kernel
     assert len(B.compile(w.routine).kernels()) == 1
     src = code.source()

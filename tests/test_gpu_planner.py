@@ -178,3 +178,40 @@ def test_bf16_operand_copy_follows_every_kind_of_writer():
         assert np.max(np.abs(got - want)) <= 2e-2 * np.max(np.abs(want))
     assert not hip.get(outs[2]).any() and not hip.get(G).any()
     hip.close()
+
+
+def test_independent_small_statements_run_side_by_side():
+    # p_k = p_k - lr (g_k + 0 p_k) for seven parameters of different shapes, as two statements each (the
+    # shape of an SGD step): the seven deltas do not touch one another, neither do the seven updates, and
+    # every update reads its delta -- two launches instead of fourteen
+    # (one launch when each delta / update pair has been fused into a row group first)
+    L.reset_symbols(0)
+    shapes = [(512,), (512,), (64, 48), (2048,), (7,), (300, 10), (33, 5, 3)]
+    ids = iter(range(1, 100))
+    lr = L.Node(next(ids), "lr", "single", (1,))
+    params, grads, deltas, body = [], [], [], []
+    for k, dims in enumerate(shapes):
+        p, g, d = (L.Node(next(ids), f"{n}{k}", "single", dims) for n in ("p", "g", "delta"))
+        params.append(p); grads.append(g); deltas.append(d)
+    def nest(dims, stmt):
+        syms = [L.fresh_symbol() for _ in dims]
+        b = [stmt(tuple(L.It(s) for s in syms))]
+        for s, e in reversed(list(zip(syms, dims))):
+            b = [L.For(s, 0, e - 1, b)]
+        return b
+    for p, g, d in zip(params, grads, deltas):
+        body += nest(p.dims, lambda ix: L.Set(d, ix, L.Binop("add", L.Get(g, ix), L.Binop("mul", L.Const(0.0), L.Get(p, ix)))))
+        body += nest(p.dims, lambda ix: L.Set(p, ix, L.Binop("sub", L.Get(p, ix), L.Binop("mul", L.Get(lr, (L.Fixed(0),)), L.Get(d, ix)))))
+    r = L.Routine("small_updates", body)
+    rng = np.random.default_rng(8)
+    init = {n.id: rng.standard_normal(n.dims).astype(np.float32) for n in params + grads}
+    init[lr.id] = np.array([0.1], np.float32)
+    ora = OracleRun(r, init)
+    ora.step(); ora.step()
+    for opts, launches in (("serial=0;rows=0", 2), ("serial=0;rows=0;parallel=0", 14), ("serial=0", 1)):
+        hip = HipRun(r, init, opts)
+        assert len(hip.code.kernels()) == launches, hip.code.kernels()
+        hip.step(); hip.step()
+        for n in params + deltas:     # (the host compiler may fuse the multiply into the subtraction: last bit)
+            assert rel_err(hip.get(n), ora.get(n), "single") <= 1e-6, (opts, n.ident)
+        hip.close()
