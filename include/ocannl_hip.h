@@ -113,7 +113,8 @@ int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** code);
    bf16 contraction once into scratch instead of in every kernel that reads it), serial=0|1 (a routine
    of tiny phases as one single-workgroup kernel), groups=0|1 (independent contractions of identical
    shapes share a launch), chains=0|1 (`c =+ a * b` statements into one result with identical operand
-   shapes share a launch), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
+   shapes share a launch), parallel=0|1 (consecutive small phases that do not depend on one another
+   run side by side in one launch), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
    indices and offsets in generated kernels, the `large_models` setting of c_syntax.ml:111-112; a
    routine with a node of more than 2^31 - 1 elements gets them without asking). */
 int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, ocannl_hip_code** code);
