@@ -1185,7 +1185,8 @@ void merge_contractions(Plan& plan, bool chain) {
       const std::vector<Member> mine = members_of(g);
       if (candidate && chain)
         candidate = h.accumulate && h.c_copy < 0 && h.c.node == g.c.node && h.c.offset == g.c.offset &&
-                    h.c.static_terms == g.c.static_terms && source_of(h.a.node) != g.c.node && source_of(h.b.node) != g.c.node;
+                    h.c.static_terms == g.c.static_terms && source_of(h.a.node) != g.c.node && source_of(h.b.node) != g.c.node &&
+                    (g.c_copy < 0 || (h.a.node != g.c_copy && h.b.node != g.c_copy));
       if (candidate && !chain) {
         candidate = h.accumulate == g.accumulate && (h.c_copy >= 0) == (g.c_copy >= 0);
         for (auto& x : mine) {
