@@ -493,6 +493,8 @@ bool phase_touches(const Phase& ph, int node) {
     return ph.gemm.a.node == node || ph.gemm.b.node == node || ph.gemm.c.node == node;
   }
   if (!ph.parallel_members.empty()) { for (auto& m : ph.parallel_members) if (phase_touches(m, node)) return true; return false; }
+  if (!ph.members.empty()) { for (auto& m : ph.members) if (phase_touches(m, node)) return true; return false; }
+  if (!ph.serial_members.empty()) { for (auto& m : ph.serial_members) if (phase_touches(m, node)) return true; return false; }
   std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
   block_accesses(ph.inner, acc, w, f, d);
   if (w) return true;   // a Zero_out inside the nest: not tracked per node, assume the worst
@@ -1339,6 +1341,8 @@ void serialise_tiny(const Routine& r, Plan& plan) {
 // a few microseconds each in a row.
 namespace {
 
+bool phase_writes(const Phase& ph, int node);
+
 void group_independent(const Routine& r, Plan& plan) {
   (void)r;
   if (plan.phases.size() < 2) return;
@@ -1367,6 +1371,28 @@ void group_independent(const Routine& r, Plan& plan) {
     for (int v : x) if (y.count(v)) return false;
     return true;
   };
+  // A small phase that stands at the end of its window (a phase that cannot join follows it) waits
+  // for the first later phase that conflicts with it and runs right before that one -- the second
+  // half of a split bias-gradient sum, say, joins the window of the optimiser's updates, the first
+  // thing that reads it.  (From the last phase backwards, so that positions ahead stay valid.)
+  for (size_t i = plan.phases.size(); i-- > 0;) {
+    const Sets mine = sets_of(plan.phases[i]);
+    if (!mine.ok || plan.phases[i].bytes > (double)(2 << 20) || i + 1 >= plan.phases.size()) continue;
+    if (sets_of(plan.phases[i + 1]).ok) continue;
+    size_t t = i + 1;
+    for (; t < plan.phases.size(); ++t) {
+      const Phase& q = plan.phases[t];
+      bool conflict = false;
+      for (int n : mine.writes) conflict = conflict || phase_touches(q, n);
+      for (int n : mine.reads) conflict = conflict || phase_writes(q, n);
+      if (conflict) break;
+    }
+    if (t == i + 1) continue;
+    // worth it only next to a phase it can share a launch with
+    const bool joins = (t < plan.phases.size() && sets_of(plan.phases[t]).ok) || sets_of(plan.phases[t - 1]).ok;
+    if (!joins) continue;
+    std::rotate(plan.phases.begin() + i, plan.phases.begin() + i + 1, plan.phases.begin() + t);
+  }
   std::vector<Sets> sets;
   for (auto& ph : plan.phases) sets.push_back(sets_of(ph));
   std::vector<Phase> out;
@@ -1435,7 +1461,8 @@ bool phase_writes(const Phase& ph, int node) {
     return false;
   };
   if (!ph.members.empty()) { for (auto& m : ph.members) if (writes(m)) return true; return false; }
-  if (!ph.parallel_members.empty()) { for (auto& m : ph.parallel_members) if (writes(m)) return true; return false; }
+  if (!ph.parallel_members.empty()) { for (auto& m : ph.parallel_members) if (phase_writes(m, node)) return true; return false; }
+  if (!ph.serial_members.empty()) { for (auto& m : ph.serial_members) if (phase_writes(m, node)) return true; return false; }
   return writes(ph);
 }
 
