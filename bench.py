@@ -21,7 +21,6 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 import numpy as np  # noqa: E402
 
@@ -67,14 +66,18 @@ def cpu_baseline(name: str):
     in process) timed on a bounded sample of the same workload, scaled to steps/s of the full
     configuration.  Reported next to the GPU number; it is not a target."""
     from ocannl_amd import workloads as W
-    from parity import OracleRun
+    from oracle import cc_oracle   # the checker, used here as the reported CPU baseline only
 
     def time_steps(w, n, statics=None):
-        o = OracleRun(w.routine, w.init)
-        o.step(statics)   # first call: page in
+        lib = cc_oracle.CompiledOracle([w.routine])
+        bufs = {}
+        for nd in w.routine.param_nodes():
+            bufs[nd.id] = (np.ascontiguousarray(np.array(w.init[nd.id], copy=True)) if nd.id in w.init
+                           else cc_oracle.host_array(nd))
+        lib.run(w.routine.name, bufs, statics or {})   # first call: page in
         t = time.perf_counter()
         for _ in range(n):
-            o.step(statics)
+            lib.run(w.routine.name, bufs, statics or {})
         return (time.perf_counter() - t) / n
 
     if name == "transformer":
@@ -121,7 +124,7 @@ def main():
         raise SystemExit("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)")
 
     from ocannl_amd import backend as B
-    from parity import HipRun
+    from ocannl_amd.backend import HipRun
 
     w, metric, unit, dtype = build_workload(args.workload)
     t_c = time.perf_counter()

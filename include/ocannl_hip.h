@@ -34,6 +34,9 @@ extern "C" {
 #define OCANNL_HIP_E_INVALID (-2)  /* Invalid_argument: misuse of the interface, malformed IR      */
 #define OCANNL_HIP_E_RUNTIME (-3)  /* Failure: HIP / hiprtc error                                  */
 
+/* Size of the library's static device scratch array (see ocannl_hip_routine_run_static_scratch). */
+#define OCANNL_HIP_STATIC_SCRATCH_BYTES (32ull << 20)
+
 typedef struct ocannl_hip_device ocannl_hip_device;    /* (dev, runner) of one ordinal            */
 typedef struct ocannl_hip_event ocannl_hip_event;      /* Lowered_backend.event                   */
 typedef struct ocannl_hip_code ocannl_hip_code;        /* Lowered_backend.code / code_batch       */
@@ -118,6 +121,8 @@ int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** code);
    indices and offsets in generated kernels, the `large_models` setting of c_syntax.ml:111-112; a
    routine with a node of more than 2^31 - 1 elements gets them without asking). */
 int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, ocannl_hip_code** code);
+/* Drops the caller's reference.  Routines linked from the code keep what they need alive (the launch
+   closure's context_lifetime, cuda_backend.ml:1046-1051), so code_free before routine_free is fine. */
 void ocannl_hip_code_free(ocannl_hip_code* code);
 int ocannl_hip_code_num_routines(ocannl_hip_code* code, int* n);
 int ocannl_hip_code_routine_name(ocannl_hip_code* code, int index, char* buf, size_t cap);
@@ -141,6 +146,18 @@ int ocannl_hip_routine_set_static(ocannl_hip_routine* routine, int symbol, int64
    is now, :1009-1011; E_USER when no transfer has filled it or it is smaller than the merge node),
    then enqueues the routine's kernels on the device stream. */
 int ocannl_hip_routine_run(ocannl_hip_routine* routine);
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP
+   graph capture, tight serving loops, harnesses that forbid hipMalloc): ocannl_hip_routine_run with
+   the routine's scratch memory -- `Local` nodes, tensors the planner materialises, the split-K
+   workspace of the MFMA kernels -- taken from a static device array of
+   OCANNL_HIP_STATIC_SCRATCH_BYTES that belongs to the loaded library (one copy per GPU, held until
+   the process ends) instead of the arena that link allocated.  Inputs and outputs are the context
+   nodes the routine was linked against, as for routine_run.  Calls no hipMalloc / hipFree / event or
+   other allocating routine; zero fills run as kernels, not memsets.  A routine whose scratch needs
+   exceed the array is refused with E_USER.  Every call on a GPU shares that GPU's array, which keeps
+   the previous call's contents (nothing in it needs to start at zero: every routine fills what it
+   reads); calls that overlap on one GPU -- other than in order on the device's one stream -- race. */
+int ocannl_hip_routine_run_static_scratch(ocannl_hip_routine* routine);
 /* Same, bracketing every kernel with HIP events on the device stream; synchronises and writes the
    per-kernel milliseconds (cap >= number of kernels).  For measurement only. */
 int ocannl_hip_routine_run_timed(ocannl_hip_routine* routine, float* kernel_ms, int cap);

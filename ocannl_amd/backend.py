@@ -75,7 +75,8 @@ EXPORTS = (
     "ocannl_hip_code_routine_name", "ocannl_hip_code_kparams", "ocannl_hip_code_source",
     "ocannl_hip_code_num_kernels", "ocannl_hip_code_kernel_info", "ocannl_hip_link",
     "ocannl_hip_routine_free", "ocannl_hip_routine_set_static", "ocannl_hip_routine_run",
-    "ocannl_hip_routine_run_timed", "ocannl_hip_routine_profile_kernel", "ocannl_hip_routine_profile_read",
+    "ocannl_hip_routine_run_static_scratch", "ocannl_hip_routine_run_timed",
+    "ocannl_hip_routine_profile_kernel", "ocannl_hip_routine_profile_read",
 )
 
 _lib = None
@@ -127,6 +128,7 @@ def load_library() -> ctypes.CDLL:
         "ocannl_hip_routine_free": (None, [vp]),
         "ocannl_hip_routine_set_static": (i32, [vp, i32, i64]),
         "ocannl_hip_routine_run": (i32, [vp]),
+        "ocannl_hip_routine_run_static_scratch": (i32, [vp]),
         "ocannl_hip_routine_run_timed": (i32, [vp, P(ctypes.c_float), i32]),
         "ocannl_hip_routine_profile_kernel": (i32, [vp, i32]),
         "ocannl_hip_routine_profile_read": (i32, [vp, P(ctypes.c_double), P(i64)]),
@@ -350,6 +352,11 @@ class Routine:
         """``Task.run``: checks static indices, enqueues the kernels; asynchronous."""
         _check(load_library().ocannl_hip_routine_run(self._h))
 
+    def run_static_scratch(self) -> None:
+        """``run`` with the routine's scratch memory taken from the library's static device array:
+        allocates nothing; refuses (``User_error``) a routine whose scratch needs exceed it."""
+        _check(load_library().ocannl_hip_routine_run_static_scratch(self._h))
+
     def profile_kernel(self, kernel_index: int) -> None:
         _check(load_library().ocannl_hip_routine_profile_kernel(self._h, kernel_index))
 
@@ -468,3 +475,34 @@ class Context:
             free_pool(self.dev, pool_id=p)
         self.pools = []
         self.ctx_buffers = {}
+
+
+class HipRun:
+    """One routine compiled, given a context of its own with the given initial values, and linked:
+    what a test or a benchmark steps (``Train.to_routine`` + ``Context.run``, lib/train.ml:108-170)."""
+
+    def __init__(self, routine: L.Routine, init: Mapping[int, np.ndarray], options: Optional[str] = None):
+        self.routine = routine
+        self.code = compile(routine, options)
+        self.ctx = Context()
+        self.ctx.allocate(routine.param_nodes())
+        for n in routine.param_nodes():
+            if n.id in init:
+                self.ctx.set_values(n, init[n.id])
+        self.rt = self.ctx.link(self.code)
+
+    def step(self, static: Optional[Mapping[int, int]] = None, static_scratch: bool = False):
+        for sym, v in (static or {}).items():
+            self.rt.set_static(sym, v)
+        if static_scratch:
+            self.rt.run_static_scratch()
+        else:
+            self.rt.run()
+
+    def get(self, node: L.Node) -> np.ndarray:
+        return self.ctx.get_values(node)
+
+    def close(self):
+        await_(self.ctx.dev)
+        del self.rt
+        self.ctx.free()

@@ -918,12 +918,8 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     }
     for (auto& s : r.statics) {
       if (!pr.used_statics.count(s.sym)) continue;
-      if (plan.large_index) {   // widen before any offset arithmetic
-        decls.push_back("const uint32_t " + sym_ident(s.sym) + "_arg");
-        body.insert(body.begin(), "  const uint64_t " + sym_ident(s.sym) + " = " + sym_ident(s.sym) + "_arg;");
-      } else {
-        decls.push_back("const uint32_t " + sym_ident(s.sym));
-      }
+      // integer arguments are 64 bits wide under large_models (c_syntax.ml:111-112 `arg_int_prefix`)
+      decls.push_back(std::string(plan.large_index ? "const uint64_t " : "const uint32_t ") + sym_ident(s.sym));
       gk.params.push_back({KernelParam::StaticIdx, s.sym});
     }
     src << "/* phase " << pi << ": " << ph.label << " */\n";

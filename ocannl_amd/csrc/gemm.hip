@@ -11,10 +11,11 @@
 //
 // Kernel structure (bf16 compute, fp32 accumulate):
 //   * 256 threads = 4 wavefronts in a 2x2 grid; block tile BM x BN, K step 64;
-//   * global -> registers (16-byte loads) -> LDS, double buffered, one barrier per K step;
-//     row-contiguous operands are transposed 8x8 in registers on the way so that LDS always holds
-//     [row][k] with k contiguous; rows are padded by 16 bytes so that ds_read_b128 of 16 rows hits
-//     distinct banks; fp32 sources are rounded to bf16 (RNE) on the way;
+//   * global -> registers (16-byte loads) -> LDS, double buffered, one barrier per K step; a
+//     K-contiguous operand is held [row][k] (rows padded by 16 bytes: ds_read_b128 of 16 rows hits
+//     distinct banks), a row-contiguous operand stays [k][row] as it lies in memory and its MFMA
+//     fragments are read with ds_read_b64_tr_b16 -- no transposition anywhere; fp32 sources are
+//     rounded to bf16 (RNE) on the way to LDS;
 //   * v_mfma_f32_32x32x16_bf16, each wavefront owns a (BM/2) x (BN/2) sub-tile;
 //   * workgroup ids are remapped so that each XCD (ids are dealt round-robin over 8 XCDs) works on
 //     a compact band of tiles and shares B/A panels through its own L2.
@@ -47,20 +48,6 @@ template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl<N>(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
 }
-
-// Phase timestamps for kernel tuning (compiled in only with -DOCANNL_GEMM_TIMING): workgroup w
-// writes the 100 MHz wall clock at stamp i to g_gemm_stamps[8 * w + i].
-#ifdef OCANNL_GEMM_TIMING
-__device__ int g_probe_skip;   // bit 0: no global loads / LDS stores in the main loop; bit 1: no LDS fragment reads
-#define OCANNL_PROBE_SKIP(bit) (g_probe_skip & (bit))
-__device__ long long g_gemm_stamps[8 * 4096];
-#define OCANNL_STAMP(i) \
-  do { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && blockIdx.x < 4096) g_gemm_stamps[8 * blockIdx.x + (i)] = wall_clock64(); } while (0)
-#else
-#define OCANNL_STAMP(i) do { } while (0)
-#define OCANNL_PROBE_SKIP(bit) 0
-#endif
-
 
 constexpr int kThreads = 256;
 constexpr int kBK = 64;        // K elements per stage (bf16 compute)
@@ -364,8 +351,6 @@ gemm_bf16_kernel(const GemmArgs g) {
   extern __shared__ __align__(16) unsigned short smem[];
   unsigned short* const As0 = smem;
   unsigned short* const Bs0 = smem + 2 * kAT;
-
-  OCANNL_STAMP(0);
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
   const long tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
@@ -428,7 +413,6 @@ gemm_bf16_kernel(const GemmArgs g) {
   sa[0].store(As0, tid);
   sb[0].store(Bs0, tid);
   __syncthreads();
-  OCANNL_STAMP(1);
 
   // one K step; `par` = ks % kPF is a compile-time constant so that the register sets are
   // addressed statically
@@ -436,7 +420,7 @@ gemm_bf16_kernel(const GemmArgs g) {
     constexpr int par = decltype(par_c)::value;
     const int cur = ks & 1;
     // register set `par` held tile ks (already in LDS): refill it with tile ks + kPF
-    if (ks + kPF < ksteps && !OCANNL_PROBE_SKIP(1)) {
+    if (ks + kPF < ksteps) {
       sa[par].load(A, lda, m0, kbeg + (ks + kPF) * kBK, g.M, kend, tid);
       sb[par].load(B, ldb, n0, kbeg + (ks + kPF) * kBK, g.N, kend, tid);
     }
@@ -461,7 +445,7 @@ gemm_bf16_kernel(const GemmArgs g) {
     static_for<kBK / 16>([&](auto kkc) OCN_LAMBDA_INLINE {
       constexpr int kk = decltype(kkc)::value, fb = kk & 1;
       if constexpr (kk + 1 < kBK / 16) {
-        if (!OCANNL_PROBE_SKIP(2)) read_frags(std::integral_constant<int, kk + 1>{});
+        read_frags(std::integral_constant<int, kk + 1>{});
         __builtin_amdgcn_sched_barrier(0);
       }
       static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
@@ -473,7 +457,7 @@ gemm_bf16_kernel(const GemmArgs g) {
     });
     __builtin_amdgcn_sched_barrier(0);
     // tile ks + 1 sits in the other register set (or, with one set, in the one just refilled)
-    if (ks + 1 < ksteps && !OCANNL_PROBE_SKIP(1)) {
+    if (ks + 1 < ksteps) {
       constexpr int nxt = (par + 1) % kPF;
       sa[nxt].store(As0 + (cur ^ 1) * kAT, tid);
       sb[nxt].store(Bs0 + (cur ^ 1) * kBT, tid);
@@ -573,10 +557,8 @@ gemm_bf16_kernel(const GemmArgs g) {
   } else {
     pipeline();
   }
-  OCANNL_STAMP(2);
 
   epilogue<TM, TN>(g, cbase, c2base, acc, m0 + wm0, n0 + wn0, co, lane);
-  OCANNL_STAMP(3);
 }
 
 // ---- fp32 compute -------------------------------------------------------------------------------
@@ -761,9 +743,6 @@ long batch_count(const GemmDesc& d) {
   return nb;
 }
 
-#ifdef OCANNL_GEMM_TIMING
-int g_force_tile = 0, g_force_splits = 0, g_force_prefetch = 0;   // tuning overrides of the probe build
-#endif
 
 // Tile size and split-K factor, from a measured sweep on MI355X (bf16 operands).  256x256 tiles
 // (one workgroup per CU) win only when the output alone gives >= 256 of them and K runs at least
@@ -791,17 +770,10 @@ TileConfig tile_config(const GemmDesc& d) {
     }
     c.splits = (int)s;
   }
-#ifdef OCANNL_GEMM_TIMING
-  if (g_force_tile) c.big = g_force_tile == 256;
-  if (g_force_splits) c.splits = g_force_splits;
-#endif
   // two stages of global loads in flight when the launch puts at most one workgroup on a CU and
   // each runs at least 8 K stages (measured: 8192x512x2048 bf16 595 -> 738 TFLOP/s)
   c.prefetch = (!c.big && bf16_sources && t128 * c.splits <= 256 && d.K / c.splits >= 512) ? 2 : 1;
   if (!d.more.empty()) c.prefetch = 2;   // the only variant built for chains
-#ifdef OCANNL_GEMM_TIMING
-  if (g_force_prefetch) c.prefetch = (!c.big && bf16_sources) ? g_force_prefetch : 1;
-#endif
   return c;
 }
 

@@ -234,6 +234,20 @@ bool match_contraction(const Routine& r, Phase& ph, const PlanOptions& opt) {
   while (ms.size() > 1) { batch.push_back(ms.front()); ms.erase(ms.begin()); }
   while (ns.size() > 1) { batch.push_back(ns.front()); ns.erase(ns.begin()); }
   if (ks.size() > 1 || batch.size() > 3) return false;
+  // The kernels store (or read-add-write) every (batch, m, n) cell from its own lane with no atomics:
+  // distinct cells must be distinct elements of C.  An accumulation through overlapping windows
+  // (the input gradient of a convolution: x_grad[stride * o + k] with stride < window) is not that,
+  // and stays a generated kernel, which has the same one-to-one test per axis.
+  {
+    std::vector<std::pair<int64_t, int64_t>> cells;   // (C stride, extent)
+    for (auto* v : {&batch, &ms, &ns}) for (auto& s : *v) cells.push_back({s.c, s.ext});
+    std::sort(cells.begin(), cells.end());
+    int64_t reach = 0;
+    for (auto& c : cells) {
+      if (c.first <= reach) return false;
+      reach += c.first * (c.second - 1);
+    }
+  }
 
   GemmDesc g;
   g.M = ms.empty() ? 1 : ms[0].ext;
@@ -1487,7 +1501,10 @@ bool writes_whole_node(const Routine& r, const Phase& ph, int node) {
 
 struct Bf16Copies {
   std::map<int, int> copy_of;       // fp32 node -> its bf16 scratch copy
-  std::map<int, size_t> made_at;    // fp32 node -> plan.phases.size() when the copy was planned
+  std::map<int, size_t> made_at;    // fp32 node -> position in plan.phases from which writers make the copy stale
+  // positions move when the planner erases a folded fill or inserts a fill for a copy
+  void erased(size_t at) { for (auto& kv : made_at) if (kv.second > at) --kv.second; }
+  void inserted(size_t at) { for (auto& kv : made_at) if (kv.second >= at) ++kv.second; }
 };
 
 void use_bf16_copies(Routine& r, Plan& plan, Phase& ph, Bf16Copies& copies, int* next_sym) {
@@ -1548,6 +1565,7 @@ void use_bf16_copies(Routine& r, Plan& plan, Phase& ph, Bf16Copies& copies, int*
         f.kind = Phase::Fill; f.label = "zero bf16 copy of " + src.ident; f.fill_node = t.id;
         f.bytes = (double)t.size_in_bytes();
         plan.phases.insert(plan.phases.begin() + fills[k] + 1, std::move(f));
+        copies.inserted(fills[k] + 1);
       }
       op.node = t.id;
       op.prec = Prec::Bfloat16;
@@ -1748,7 +1766,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
             if (ph.par_syms[i] == a.sym) full = ph.par_from[i] == 0 && ph.par_ext[i] == n.dims[p];
         } else full = false;
       }
-      if (full) { ph.fused_zero_init = true; plan.phases.erase(plan.phases.begin() + fill_at); }
+      if (full) { ph.fused_zero_init = true; plan.phases.erase(plan.phases.begin() + fill_at); copies.erased((size_t)fill_at); }
     }
     // a dead fill: the nest stores to every element of a tensor without reading it, and nothing has
     // touched the tensor since its Zero_out
@@ -1761,7 +1779,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
       if (!reads_target && writes_whole_node(r, ph, target)) {
         for (int q = (int)plan.phases.size() - 1; q >= 0; --q) {
           const Phase& prev = plan.phases[q];
-          if (prev.kind == Phase::Fill && prev.fill_node == target) { plan.phases.erase(plan.phases.begin() + q); break; }
+          if (prev.kind == Phase::Fill && prev.fill_node == target) { plan.phases.erase(plan.phases.begin() + q); copies.erased((size_t)q); break; }
           if (phase_touches(prev, target)) break;
         }
       }

@@ -31,11 +31,25 @@ void hip_check(hipError_t e, const char* what) {
   if (e != hipSuccess) throw RuntimeError(std::string(what) + ": " + hipGetErrorString(e));
 }
 
+// Scratch memory for ocannl_hip_routine_run_static_scratch, the entry point that may not allocate:
+// device memory that belongs to the loaded library itself.  Every GPU holds its own copy at its own
+// address until the process ends; host code reaches it only through the pointer that
+// hipGetSymbolAddress returns (ocannl_hip_device::static_scratch), never through this name.
+constexpr uint64_t kStaticScratchBytes = OCANNL_HIP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Zero fill as a kernel (16-byte stores), for the path that callers may record into a HIP graph.
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint4* p, uint64_t n16) {
+  const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n16) p[i] = uint4{0, 0, 0, 0};
+}
+
 }  // namespace
 
 struct ocannl_hip_device {
   int ordinal = 0;
   hipStream_t stream = nullptr;
+  void* static_scratch = nullptr;   // this device's copy of `scratch` (hipGetSymbolAddress at device set-up)
   std::map<int, std::pair<void*, uint64_t>> pools;   // pool_id -> (base, size)
   uint64_t used = 0;
   uint64_t scratch_used = 0;
@@ -46,7 +60,7 @@ struct ocannl_hip_device {
   void* resolve(int pool_id, uint64_t offset, uint64_t bytes, const char* what) const {
     auto it = pools.find(pool_id);
     if (it == pools.end()) throw InvalidArgument(std::string(what) + ": unknown pool_id " + std::to_string(pool_id));
-    if (offset + bytes > it->second.second)
+    if (offset > it->second.second || bytes > it->second.second - offset)
       throw InvalidArgument(std::string(what) + ": range [" + std::to_string(offset) + ", +" + std::to_string(bytes) +
                             ") exceeds pool " + std::to_string(pool_id) + " of " + std::to_string(it->second.second) + " bytes");
     return static_cast<char*>(it->second.first) + offset;
@@ -124,30 +138,36 @@ PlanOptions parse_options(const char* options) {
 
 }  // namespace
 
+// The compiled routines are shared between the caller's handle and every routine linked from it:
+// ocannl_hip_code_free only drops the caller's reference (context_lifetime, cuda_backend.ml:1046-1051).
 struct ocannl_hip_code {
-  std::vector<CompiledRoutine> routines;
+  std::shared_ptr<std::vector<CompiledRoutine>> routines = std::make_shared<std::vector<CompiledRoutine>>();
 };
 
 struct ocannl_hip_routine {
   ocannl_hip_device* dev = nullptr;
   const CompiledRoutine* code = nullptr;
-  std::shared_ptr<void> keep_code;   // context_lifetime: keeps module + code alive (cuda_backend.ml:1046-1051)
+  std::shared_ptr<std::vector<CompiledRoutine>> keep_code;   // owns what `code` points into
   hipModule_t module = nullptr;
-  void* scratch = nullptr;
+  void* scratch = nullptr;           // the routine's own arena: local nodes, planner scratch, split-K workspace
   uint64_t scratch_bytes = 0;
-  void* gemm_ws = nullptr;           // split-K workspace inside the scratch arena
-  std::map<int, void*> node_ptr;
+  bool counted = false;              // included in the device's live_routines
+  // Everything that names arena memory exists twice: [0] bound to the routine's own arena, [1] bound to
+  // the library's static scratch array (valid when static_ok).
+  bool static_ok = false;
+  void* gemm_ws[2] = {nullptr, nullptr};   // split-K workspace
+  std::map<int, void*> node_ptr[2];
   std::map<int, int64_t> statics;    // symbol -> current value
   struct Launch {
-    int phase;
+    int phase = 0;
     hipFunction_t fn = nullptr;
-    std::vector<void*> ptr_vals;       // storage for pointer arguments
-    std::vector<uint32_t> idx_vals;    // storage for static-index arguments
+    std::vector<void*> ptr_vals[2];    // storage for pointer arguments
+    std::vector<uint64_t> idx_vals;    // storage for static-index arguments (a 32-bit parameter reads the low half)
     std::vector<int> idx_syms;
     int merge_slot = -1;               // index in ptr_vals of the merge-buffer argument, bound at launch
-    std::vector<void*> args;
+    std::vector<void*> args[2];
     unsigned grid = 1, grid_y = 1, block = 256;
-    void* fill_ptr = nullptr; uint64_t fill_bytes = 0;
+    void* fill_ptr[2] = {nullptr, nullptr}; uint64_t fill_bytes = 0;
   };
   std::vector<Launch> launches;
   std::vector<hipEvent_t> timing_events;
@@ -175,7 +195,21 @@ void copy_out(const std::string& s, char* buf, size_t cap) {
   buf[n] = '\0';
 }
 
-void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
+void destroy_routine(ocannl_hip_routine* rt) {
+  if (!rt) return;
+  (void)hipSetDevice(rt->dev->ordinal);
+  (void)hipStreamSynchronize(rt->dev->stream);
+  for (auto e : rt->timing_events) (void)hipEventDestroy(e);
+  for (auto e : rt->profile_events) (void)hipEventDestroy(e);
+  if (rt->module) (void)hipModuleUnload(rt->module);
+  if (rt->scratch) { (void)hipFree(rt->scratch); rt->dev->scratch_used -= rt->scratch_bytes; }
+  if (rt->counted) rt->dev->live_routines--;
+  delete rt;
+}
+
+// `v` = 0: the routine's own arena; 1: the library's static scratch array, with fills as kernels
+// and no call that allocates (no events: kernel_ms must be null and bracketing is off).
+void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0) {
   ocannl_hip_device& dev = *rt.dev;
   dev.make_current();
   const Routine& r = rt.code->r;
@@ -187,6 +221,10 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
     if (s.range >= 0 && v >= s.range)
       throw UserError("hip backend: static index " + sym_ident(s.sym) + " is too big: " + std::to_string(v) +
                       " (range 0.." + std::to_string(s.range - 1) + ")");
+    // generated kernels take 32-bit static indices unless the routine was planned with 64-bit offsets
+    if (!rt.code->plan.large_index && v > (int64_t)0xFFFFFFFFll)
+      throw UserError("hip backend: static index " + sym_ident(s.sym) + " = " + std::to_string(v) +
+                      " needs 64-bit indices: compile with large_models=1");
   }
   // the merge buffer is bound when the routine is scheduled, not when it is linked: it may have been
   // regrown since (cuda_backend.ml:1009-1011, :130-134)
@@ -212,7 +250,7 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
   for (size_t li = 0; li < rt.launches.size(); ++li) {
     auto& l = rt.launches[li];
     const Phase& ph = rt.code->plan.phases[l.phase];
-    const bool bracket = !timed && li < rt.profile_mask.size() && rt.profile_mask[li];
+    const bool bracket = v == 0 && !timed && li < rt.profile_mask.size() && rt.profile_mask[li];
     if (bracket) {
       while (rt.profile_events.size() < rt.profile_used + 2) {
         hipEvent_t e;
@@ -222,18 +260,26 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
       hip_check(hipEventRecord(rt.profile_events[rt.profile_used], dev.stream), "hipEventRecord");
     }
     if (ph.kind == Phase::Fill) {
-      hip_check(hipMemsetAsync(l.fill_ptr, 0, l.fill_bytes, dev.stream), "hipMemsetAsync");
+      if (v == 0) {
+        hip_check(hipMemsetAsync(l.fill_ptr[0], 0, l.fill_bytes, dev.stream), "hipMemsetAsync");
+      } else {
+        // local nodes sit at 256-byte offsets and are padded to 256 bytes: whole 16-byte stores
+        const uint64_t n16 = (l.fill_bytes + 15) / 16;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, dev.stream,
+                           static_cast<uint4*>(l.fill_ptr[1]), n16);
+        hip_check(hipGetLastError(), "fill_zero_kernel");
+      }
     } else if (ph.kind == Phase::Generic) {
-      for (size_t i = 0; i < l.idx_syms.size(); ++i) l.idx_vals[i] = (uint32_t)rt.statics[l.idx_syms[i]];
-      if (l.merge_slot >= 0) l.ptr_vals[l.merge_slot] = merge_base;
-      hip_check(hipModuleLaunchKernel(l.fn, l.grid, l.grid_y, 1, l.block, 1, 1, 0, dev.stream, l.args.data(), nullptr),
+      for (size_t i = 0; i < l.idx_syms.size(); ++i) l.idx_vals[i] = (uint64_t)rt.statics[l.idx_syms[i]];
+      if (l.merge_slot >= 0) l.ptr_vals[v][l.merge_slot] = merge_base;
+      hip_check(hipModuleLaunchKernel(l.fn, l.grid, l.grid_y, 1, l.block, 1, 1, 0, dev.stream, l.args[v].data(), nullptr),
                 "hipModuleLaunchKernel");
     } else {
       const GemmDesc& g = ph.gemm;
       auto base = [&](const GemmOperand& o) -> char* {
         int64_t off = o.offset;
         for (auto& t : o.static_terms) off += rt.statics[t.first] * t.second;
-        return static_cast<char*>(rt.node_ptr.at(o.node)) + off * prec_in_bytes(o.prec);
+        return static_cast<char*>(rt.node_ptr[v].at(o.node)) + off * prec_in_bytes(o.prec);
       };
       GemmArgs a{};
       a.a = base(g.a); a.b = base(g.b); a.c = base(g.c);
@@ -246,16 +292,16 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap) {
       }
       a.accumulate = g.accumulate ? 1 : 0;
       a.c_is_bf16 = g.c.prec == Prec::Bfloat16;
-      a.c2 = g.c_copy >= 0 ? rt.node_ptr.at(g.c_copy) : nullptr;
+      a.c2 = g.c_copy >= 0 ? rt.node_ptr[v].at(g.c_copy) : nullptr;
       a.npairs = 1 + (int)g.more.size();
       for (size_t p = 0; p < g.more.size(); ++p) { a.a_more[p] = base(g.more[p].first); a.b_more[p] = base(g.more[p].second); }
       a.ngroups = 1 + (int)g.group.size();
       for (size_t m = 0; m < g.group.size(); ++m) {
         a.a_more[m] = base(g.group[m].a); a.b_more[m] = base(g.group[m].b); a.c_more[m] = base(g.group[m].c);
-        a.c2_more[m] = g.group[m].c_copy >= 0 ? rt.node_ptr.at(g.group[m].c_copy) : nullptr;
+        a.c2_more[m] = g.group[m].c_copy >= 0 ? rt.node_ptr[v].at(g.group[m].c_copy) : nullptr;
       }
       // a bracketed contraction is timed without its split-K reduction (a kernel of its own)
-      hip_check(launch_gemm(g, a, rt.gemm_ws, dev.stream, bracket ? rt.profile_events[rt.profile_used + 1] : nullptr),
+      hip_check(launch_gemm(g, a, rt.gemm_ws[v], dev.stream, bracket ? rt.profile_events[rt.profile_used + 1] : nullptr),
                 "launch_gemm");
     }
     if (timed) hip_check(hipEventRecord(rt.timing_events[li + 1], dev.stream), "hipEventRecord");
@@ -315,6 +361,8 @@ int ocannl_hip_get_device(int ordinal, ocannl_hip_device** out) {
       if (std::string(d->props.gcnArchName).rfind("gfx950", 0) != 0)
         throw RuntimeError(std::string("hip backend: device is ") + d->props.gcnArchName + ", this library is built for gfx950 only");
       hip_check(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+      // this device's address of the library's static scratch array (the device is current here)
+      hip_check(hipGetSymbolAddress(&d->static_scratch, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
       g_devices[ordinal] = std::move(d);
     }
     *out = g_devices[ordinal].get();
@@ -525,7 +573,7 @@ int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, o
       cr.plan = make_plan(cr.r, opt);
       cr.mod = generate_module(cr.r, cr.plan);
       if (!cr.mod.kernels.empty()) cr.binary = hiprtc_compile(cr.mod.source, cr.r.name);
-      code->routines.push_back(std::move(cr));
+      code->routines->push_back(std::move(cr));
     }
     *out = code.release();
   });
@@ -539,12 +587,12 @@ void ocannl_hip_code_free(ocannl_hip_code* code) { delete code; }
 
 static const CompiledRoutine& routine_at(ocannl_hip_code* code, int index) {
   if (!code) throw InvalidArgument("null code");
-  if (index < 0 || index >= (int)code->routines.size()) throw InvalidArgument("routine index out of range");
-  return code->routines[index];
+  if (index < 0 || index >= (int)code->routines->size()) throw InvalidArgument("routine index out of range");
+  return (*code->routines)[index];
 }
 
 int ocannl_hip_code_num_routines(ocannl_hip_code* code, int* n) {
-  return guarded([&] { if (!code || !n) throw InvalidArgument("null argument"); *n = (int)code->routines.size(); });
+  return guarded([&] { if (!code || !n) throw InvalidArgument("null argument"); *n = (int)code->routines->size(); });
 }
 
 int ocannl_hip_code_routine_name(ocannl_hip_code* code, int index, char* buf, size_t cap) {
@@ -573,7 +621,7 @@ int ocannl_hip_code_source(ocannl_hip_code* code, char* buf, size_t cap, size_t*
   return guarded([&] {
     if (!code) throw InvalidArgument("null code");
     std::string all;
-    for (auto& cr : code->routines) all += cr.mod.source;
+    for (auto& cr : *code->routines) all += cr.mod.source;
     if (needed) *needed = all.size() + 1;
     if (buf) copy_out(all, buf, cap);
   });
@@ -616,12 +664,36 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
     const CompiledRoutine& cr = routine_at(code, index);
     if (n_locs > 0 && !locs) throw InvalidArgument("link: null locs");
     dev->make_current();
-    auto rt = std::make_unique<ocannl_hip_routine>();
+    // anything that fails below releases what the routine holds so far
+    std::unique_ptr<ocannl_hip_routine, void (*)(ocannl_hip_routine*)> rt(new ocannl_hip_routine, destroy_routine);
     rt->dev = dev;
     rt->code = &cr;
-    // ctx nodes from the caller's table
+    rt->keep_code = code->routines;
+    // ctx nodes from the caller's table: checked before anything is allocated
     std::map<int, const ocannl_hip_node_loc*> by_id;
     for (int i = 0; i < n_locs; ++i) by_id[locs[i].node_id] = &locs[i];
+    std::map<int, void*> ctx_ptr;
+    for (auto& kv : cr.r.nodes) {
+      const Node& n = kv.second;
+      if (n.mode != Mode::Ctx) continue;
+      auto it = by_id.find(n.id);
+      if (it == by_id.end())
+        throw UserError("hip backend link: node " + n.ident + " (id " + std::to_string(n.id) + ") missing from context");
+      ctx_ptr[n.id] = dev->resolve(it->second->pool_id, it->second->offset, (uint64_t)n.size_in_bytes(), "link");
+    }
+    // the MFMA kernels read 16-byte chunks relative to the node base (local nodes sit at 256-byte offsets)
+    for (auto& ph : cr.plan.phases) {
+      if (ph.kind != Phase::Contraction) continue;
+      std::vector<const GemmOperand*> ops{&ph.gemm.a, &ph.gemm.b, &ph.gemm.c};
+      for (auto& m : ph.gemm.group) { ops.push_back(&m.a); ops.push_back(&m.b); ops.push_back(&m.c); }
+      for (auto& pr : ph.gemm.more) { ops.push_back(&pr.first); ops.push_back(&pr.second); }
+      for (const GemmOperand* op : ops) {
+        auto it = ctx_ptr.find(op->node);
+        if (it != ctx_ptr.end() && reinterpret_cast<uintptr_t>(it->second) % 16 != 0)
+          throw UserError("hip backend link: node " + cr.r.node(op->node).ident +
+                          " feeds a matrix-core contraction and must sit at a 16-byte aligned pool offset");
+      }
+    }
     // local nodes (and planner scratch): one private arena, 256-byte aligned sub-buffers
     uint64_t arena = 0;
     std::map<int, uint64_t> local_off;
@@ -636,42 +708,32 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
       if (ph.kind == Phase::Contraction) ws_bytes = std::max<uint64_t>(ws_bytes, gemm_workspace_bytes(ph.gemm));
     const uint64_t ws_off = arena;
     arena += (ws_bytes + 255) / 256 * 256;
+    rt->scratch_bytes = arena;
     if (arena) {
       hip_check(hipMalloc(&rt->scratch, arena), "hipMalloc(scratch)");
-      if (ws_bytes) rt->gemm_ws = static_cast<char*>(rt->scratch) + ws_off;
-      rt->scratch_bytes = arena;
       dev->scratch_used += arena;
     }
-    for (auto& kv : cr.r.nodes) {
-      const Node& n = kv.second;
-      if (n.mode == Mode::Virtual) continue;
-      if (n.mode == Mode::Local) { rt->node_ptr[n.id] = static_cast<char*>(rt->scratch) + local_off[n.id]; continue; }
-      auto it = by_id.find(n.id);
-      if (it == by_id.end())
-        throw UserError("hip backend link: node " + n.ident + " (id " + std::to_string(n.id) + ") missing from context");
-      rt->node_ptr[n.id] = dev->resolve(it->second->pool_id, it->second->offset, (uint64_t)n.size_in_bytes(), "link");
-    }
-    // the MFMA kernels read 16-byte chunks relative to the node base
-    for (auto& ph : cr.plan.phases) {
-      if (ph.kind != Phase::Contraction) continue;
-      std::vector<const GemmOperand*> ops{&ph.gemm.a, &ph.gemm.b, &ph.gemm.c};
-      for (auto& m : ph.gemm.group) { ops.push_back(&m.a); ops.push_back(&m.b); ops.push_back(&m.c); }
-      for (auto& pr : ph.gemm.more) { ops.push_back(&pr.first); ops.push_back(&pr.second); }
-      for (const GemmOperand* op : ops)
-        if (reinterpret_cast<uintptr_t>(rt->node_ptr.at(op->node)) % 16 != 0)
-          throw UserError("hip backend link: node " + cr.r.node(op->node).ident +
-                          " feeds a matrix-core contraction and must sit at a 16-byte aligned pool offset");
+    // Two bindings of the same kernel list: [0] over the routine's own arena, [1] over the library's
+    // static scratch array (only when the arena fits into it).
+    char* const bases[2] = {static_cast<char*>(rt->scratch), static_cast<char*>(dev->static_scratch)};
+    rt->static_ok = arena <= kStaticScratchBytes && dev->static_scratch != nullptr;
+    for (int v = 0; v < 2; ++v) {
+      if (v == 1 && !rt->static_ok) break;
+      rt->node_ptr[v] = ctx_ptr;
+      for (auto& kv : local_off) rt->node_ptr[v][kv.first] = bases[v] + kv.second;
+      rt->gemm_ws[v] = ws_bytes ? bases[v] + ws_off : nullptr;
     }
     for (auto& s : cr.r.statics) rt->statics[s.sym] = 0;
     if (!cr.binary.empty()) hip_check(hipModuleLoadData(&rt->module, cr.binary.data()), "hipModuleLoadData");
     // launch records
     size_t next_generic = 0;
+    rt->launches.resize(cr.plan.phases.size());
     for (size_t pi = 0; pi < cr.plan.phases.size(); ++pi) {
       const Phase& ph = cr.plan.phases[pi];
-      ocannl_hip_routine::Launch l;
+      ocannl_hip_routine::Launch& l = rt->launches[pi];
       l.phase = (int)pi;
       if (ph.kind == Phase::Fill) {
-        l.fill_ptr = rt->node_ptr.at(ph.fill_node);
+        for (int v = 0; v < (rt->static_ok ? 2 : 1); ++v) l.fill_ptr[v] = rt->node_ptr[v].at(ph.fill_node);
         l.fill_bytes = (uint64_t)cr.r.node(ph.fill_node).size_in_bytes();
       } else if (ph.kind == Phase::Generic) {
         const GeneratedKernel& gk = cr.mod.kernels.at(next_generic++);
@@ -686,44 +748,28 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
         l.block = (unsigned)gk.block;
         size_t np = 0, ni = 0;
         for (auto& p : gk.params) (p.kind != KernelParam::StaticIdx ? np : ni)++;
-        l.ptr_vals.reserve(np); l.idx_vals.reserve(ni);
-        for (auto& p : gk.params) {
-          if (p.kind == KernelParam::NodePtr) { l.ptr_vals.push_back(rt->node_ptr.at(p.id)); }
-          else if (p.kind == KernelParam::MergeBuffer) { l.merge_slot = (int)l.ptr_vals.size(); l.ptr_vals.push_back(nullptr); }
-          else { l.idx_vals.push_back(0); l.idx_syms.push_back(p.id); }
-        }
-        size_t ip = 0, ii = 0;
-        for (auto& p : gk.params) {
-          if (p.kind != KernelParam::StaticIdx) l.args.push_back(&l.ptr_vals[ip++]);
-          else l.args.push_back(&l.idx_vals[ii++]);
+        // (sized once: the argument arrays below point into these vectors)
+        l.idx_vals.assign(ni, 0);
+        for (auto& p : gk.params) if (p.kind == KernelParam::StaticIdx) l.idx_syms.push_back(p.id);
+        for (int v = 0; v < (rt->static_ok ? 2 : 1); ++v) {
+          l.ptr_vals[v].assign(np, nullptr);
+          size_t ip = 0, ii = 0;
+          for (auto& p : gk.params) {
+            if (p.kind == KernelParam::StaticIdx) { l.args[v].push_back(&l.idx_vals[ii++]); continue; }
+            if (p.kind == KernelParam::NodePtr) l.ptr_vals[v][ip] = rt->node_ptr[v].at(p.id);
+            else l.merge_slot = (int)ip;
+            l.args[v].push_back(&l.ptr_vals[v][ip++]);
+          }
         }
       }
-      rt->launches.push_back(std::move(l));
-    }
-    // argument storage moved with the Launch objects: rebuild the pointers into it
-    for (auto& l : rt->launches) {
-      if (l.args.empty()) continue;
-      const GeneratedKernel* gk = nullptr;
-      for (auto& k : cr.mod.kernels) if (k.phase_index == l.phase) gk = &k;
-      size_t ip = 0, ii = 0, ai = 0;
-      for (auto& p : gk->params) l.args[ai++] = p.kind != KernelParam::StaticIdx ? (void*)&l.ptr_vals[ip++] : (void*)&l.idx_vals[ii++];
     }
     dev->live_routines++;
+    rt->counted = true;
     *out = rt.release();
   });
 }
 
-void ocannl_hip_routine_free(ocannl_hip_routine* rt) {
-  if (!rt) return;
-  (void)hipSetDevice(rt->dev->ordinal);
-  (void)hipStreamSynchronize(rt->dev->stream);
-  for (auto e : rt->timing_events) (void)hipEventDestroy(e);
-  for (auto e : rt->profile_events) (void)hipEventDestroy(e);
-  if (rt->module) (void)hipModuleUnload(rt->module);
-  if (rt->scratch) { (void)hipFree(rt->scratch); rt->dev->scratch_used -= rt->scratch_bytes; }
-  rt->dev->live_routines--;
-  delete rt;
-}
+void ocannl_hip_routine_free(ocannl_hip_routine* rt) { destroy_routine(rt); }
 
 int ocannl_hip_routine_set_static(ocannl_hip_routine* rt, int symbol, int64_t value) {
   return guarded([&] {
@@ -738,6 +784,18 @@ int ocannl_hip_routine_run(ocannl_hip_routine* rt) {
   return guarded([&] {
     if (!rt) throw InvalidArgument("run: null routine");
     enqueue(*rt, nullptr, 0);
+  });
+}
+
+int ocannl_hip_routine_run_static_scratch(ocannl_hip_routine* rt) {
+  return guarded([&] {
+    if (!rt) throw InvalidArgument("run_static_scratch: null routine");
+    if (rt->scratch_bytes > kStaticScratchBytes)
+      throw UserError("hip backend: routine " + rt->code->r.name + " needs " + std::to_string(rt->scratch_bytes) +
+                      " bytes of scratch memory, above the " + std::to_string(kStaticScratchBytes) +
+                      " bytes of the library's static scratch array: use ocannl_hip_routine_run");
+    if (!rt->static_ok) throw RuntimeError("run_static_scratch: the device's static scratch array was not set up");
+    enqueue(*rt, nullptr, 0, 1);
   });
 }
 

@@ -132,3 +132,93 @@ def test_padding_region_loops_visit_exactly_the_margin():
         want = np.ones(dims, int)
         want[tuple(slice(l, d - r) for d, (l, r) in zip(dims, padding))] = 0
         assert np.array_equal(visits, want), (dims, padding)
+
+
+def _conv_input_gradient(stride, ksz, b=8, oh=32, ow=32, ic=64, oc=64):
+    """x_grad[b, stride*o1+k1, stride*o2+k2, i] += y_grad[b, o1, o2, c] * w[c, k1, k2, i]
+    (the input gradient of lib/nn_blocks.ml:418-428's convolution)."""
+    L.reset_symbols(0)
+    ih, iw = stride * (oh - 1) + ksz, stride * (ow - 1) + ksz
+    w = L.Node(2, "w", "single", (oc, ksz, ksz, ic)); dy = L.Node(4, "y_grad", "single", (b, oh, ow, oc))
+    dx = L.Node(5, "x_grad", "single", (b, ih, iw, ic))
+    s = [L.fresh_symbol() for _ in range(7)]
+    bb, o1, o2, c, k1, k2, i = s
+    xi = (L.It(bb), L.Affine(((stride, o1), (1, k1)), 0), L.Affine(((stride, o2), (1, k2)), 0), L.It(i))
+    yi = (L.It(bb), L.It(o1), L.It(o2), L.It(c))
+    wi = (L.It(c), L.It(k1), L.It(k2), L.It(i))
+    body = [L.Set(dx, xi, L.Ternop("fma", L.Get(dy, yi), L.Get(w, wi), L.Get(dx, xi)))]
+    for sym, ext in reversed(list(zip(s, (b, oh, ow, oc, ksz, ksz, ic)))):
+        body = [L.For(sym, 0, ext - 1, body)]
+    return L.Routine(f"conv_dx_s{stride}_k{ksz}", [L.ZeroOut(dx)] + body), dict(w=w, dy=dy, dx=dx)
+
+
+def test_overlapping_window_accumulation_is_not_a_matrix_core_contraction():
+    # stride 1, window 3: different (o, k) meet on one element of x_grad, which the contraction kernels'
+    # plain read-add-write epilogue would lose; such a nest stays a generated kernel.  With
+    # stride = window the map is one-to-one and the matrix cores may take it.
+    r, _ = _conv_input_gradient(1, 3)
+    assert all(k["kind"] != "mfma" for k in B.compile(r, "min_mfma_flops=0").kernels())
+    r, _ = _conv_input_gradient(3, 3)
+    assert any(k["kind"] == "mfma" for k in B.compile(r, "min_mfma_flops=0").kernels())
+
+
+def _stale_copy_routine(n=256):
+    """zero_out y1; zero_out y2; c1 = x * w; x := 2 x; y1 += ..; y2 += ..; c2 = x * w with x fp32 and w
+    bf16: the second product must not reuse the bf16 copy of x made for the first."""
+    L.reset_symbols(0)
+    x = L.Node(1, "x", "single", (n, n)); w = L.Node(2, "w", "bfloat16", (n, n))
+    c1 = L.Node(3, "c1", "single", (n, n)); c2 = L.Node(4, "c2", "single", (n, n))
+    y1 = L.Node(5, "y1", "single", (n,)); y2 = L.Node(6, "y2", "single", (n,))
+    u = L.Node(7, "u", "single", (n, n))
+
+    def matmul(c):
+        i, j, k = L.fresh_symbol(), L.fresh_symbol(), L.fresh_symbol()
+        return [L.ZeroOut(c), L.For(i, 0, n - 1, [L.For(j, 0, n - 1, [L.For(k, 0, n - 1, [L.Set(
+            c, (L.It(i), L.It(j)), L.Ternop("fma", L.Get(x, (L.It(i), L.It(k))), L.Get(w, (L.It(j), L.It(k))),
+                                            L.Get(c, (L.It(i), L.It(j)))))])])])]
+
+    def rowsum(y):
+        i, k = L.fresh_symbol(), L.fresh_symbol()
+        return [L.For(i, 0, n - 1, [L.For(k, 0, n - 1, [L.Set(y, (L.It(i),), L.Binop(
+            "add", L.Get(y, (L.It(i),)), L.Get(u, (L.It(i), L.It(k)))))])])]
+
+    i, j = L.fresh_symbol(), L.fresh_symbol()
+    scale = [L.For(i, 0, n - 1, [L.For(j, 0, n - 1, [L.Set(x, (L.It(i), L.It(j)), L.Binop(
+        "mul", L.Const(2.0), L.Get(x, (L.It(i), L.It(j)))))])])]
+    body = [L.ZeroOut(y1), L.ZeroOut(y2)] + matmul(c1) + scale + rowsum(y1) + rowsum(y2) + matmul(c2)
+    return L.Routine("stale_copy", body), dict(x=x, w=w, c1=c1, c2=c2, y1=y1, y2=y2, u=u)
+
+
+def test_bf16_copy_of_an_operand_rewritten_between_two_products_is_refreshed():
+    # zero fills grouped ahead of their sums (as zero_grads-then-backprop orders them) are folded away
+    # after the copy was planned; the second product still has to see the rewritten operand
+    r, _ = _stale_copy_routine()
+    code = B.compile(r, "min_mfma_flops=0")
+    src = code.source()
+    # two distinct bf16 copies of x: one converted before x is rewritten, one kept by the kernel that rewrites it
+    copies = set(re.findall(r"\b(bf\d+_x)\[[^\]]*\] = ", src))
+    assert len(copies) >= 2, src
+
+
+def test_compile_batch_holds_every_routine():
+    # Lowered_backend.compile_batch (arrayjit/lib/backend_impl.ml:349-353): several routines, one code
+    w1 = W.dense_contraction(b=64, i=64, o=64, prec="single", which=("fwd",))
+    r1 = w1.routine
+    a = r1.param_nodes()[0]
+    L.reset_symbols(100)
+    i = L.fresh_symbol()
+    out = L.Node(900, "rowsum", "single", (a.dims[0],))
+    j = L.fresh_symbol()
+    r2 = L.Routine("second_routine", [L.ZeroOut(out), L.For(i, 0, a.dims[0] - 1, [L.For(j, 0, a.dims[1] - 1, [L.Set(
+        out, (L.It(i),), L.Binop("add", L.Get(out, (L.It(i),)), L.Get(a, (L.It(i), L.It(j)))))])])])
+    code = B.compile_batch([r1, r2])
+    lib = B.load_library()
+    n = ctypes.c_int()
+    assert lib.ocannl_hip_code_num_routines(code._h, ctypes.byref(n)) == 0 and n.value == 2
+    buf = ctypes.create_string_buffer(64)
+    assert lib.ocannl_hip_code_routine_name(code._h, 1, buf, 64) == 0 and buf.value.decode() == "second_routine"
+    assert code.index_of("second_routine") == 1
+    assert {i for k, i, _ in code.kparams(1) if k == "ptr"} == {a.id, out.id}
+    assert len(code.kernels(0)) >= 1 and len(code.kernels(1)) >= 1
+    assert "second_routine_k0" in code.source()
+    assert lib.ocannl_hip_code_routine_name(code._h, 2, buf, 64) == -2

@@ -117,3 +117,91 @@ def test_link_rejects_misaligned_contraction_operand(dev):
     with pytest.raises(B.User_error, match="16-byte"):
         B.link(dev, code, bad)
     B.free_pool(dev, pool_id=905)
+
+
+def test_compile_batch_links_and_runs_each_routine(dev):
+    # Lowered_backend.compile_batch + link per routine (arrayjit/lib/backend_impl.ml:349-355;
+    # cuda_backend.ml:930-974): two routines that share nodes, one code object, one context
+    from ocannl_amd import workloads as W
+    from parity import OracleRun
+    w1 = W.dense_contraction(b=128, i=64, o=96, prec="single", which=("fwd",))
+    r1 = w1.routine
+    x = r1.param_nodes()[0]
+    L.reset_symbols(100)
+    i, j = L.fresh_symbol(), L.fresh_symbol()
+    out = L.Node(900, "rowsum", "single", (x.dims[0],))
+    r2 = L.Routine("second_routine", [L.ZeroOut(out), L.For(i, 0, x.dims[0] - 1, [L.For(j, 0, x.dims[1] - 1, [L.Set(
+        out, (L.It(i),), L.Binop("add", L.Get(out, (L.It(i),)), L.Get(x, (L.It(i), L.It(j)))))])])])
+    code = B.compile_batch([r1, r2], "min_mfma_flops=0")
+    ctx = B.Context(dev)
+    for n in r1.param_nodes():
+        if n.id in w1.init:
+            ctx.set_values(n, w1.init[n.id])
+    rt0, rt1 = ctx.link(code, 0), ctx.link(code, 1)
+    rt1.run(); rt0.run()
+    o1, o2 = OracleRun(r1, w1.init), OracleRun(r2, {x.id: w1.init[x.id]})
+    o1.step(); o2.step()
+    y = [n for n in r1.param_nodes() if n.id not in w1.init][0]
+    assert np.allclose(ctx.get_values(y), o1.get(y), rtol=1e-4, atol=1e-5)
+    assert np.allclose(ctx.get_values(out), o2.get(out), rtol=1e-5, atol=1e-5)
+    del rt0, rt1
+    ctx.free()
+
+
+def test_routine_outlives_its_code_handle(dev):
+    # the launch closure keeps what it needs alive (context_lifetime, cuda_backend.ml:1046-1051):
+    # freeing the code handle first, as a finaliser may, leaves the linked routine usable
+    L.reset_symbols(0)
+    a = L.Node(1, "a", "single", (64,)); b = L.Node(2, "b", "single", (64,))
+    st = L.StaticSymbol(L.fresh_symbol(), 4)
+    i = L.fresh_symbol()
+    r = L.Routine("scaled", [L.For(i, 0, 63, [L.Set(b, (L.It(i),), L.Binop(
+        "mul", L.Get(a, (L.It(i),)), L.EmbedIndex(L.It(st.sym))))])], static_indices=[st])
+    code = B.compile(r)
+    ctx = B.Context(dev)
+    ctx.set_values(a, np.arange(64, dtype=np.float32))
+    rt = ctx.link(code)
+    B.load_library().ocannl_hip_code_free(code._h)
+    code._h = None
+    garbage = [B.compile(r) for _ in range(4)]   # churn the allocator where the code object lived
+    rt.set_static(st.sym, 3)
+    rt.run()
+    assert np.array_equal(ctx.get_values(b), 3.0 * np.arange(64, dtype=np.float32))
+    with pytest.raises(B.User_error):
+        rt.set_static(st.sym, 4)
+        rt.run()
+    del rt, garbage
+    ctx.free()
+
+
+def test_failed_link_releases_what_it_allocated(dev):
+    from ocannl_amd import workloads as W
+    w = W.moons_mlp()                      # has routine-local nodes: link allocates an arena
+    code = B.compile(w.routine)
+    before = B.get_used_memory(dev)
+    info = B.get_debug_info(dev)
+    with pytest.raises(B.User_error):
+        B.link(dev, code, {})              # every context node missing
+    assert B.get_used_memory(dev) == before and B.get_debug_info(dev) == info
+
+
+def test_static_indices_travel_as_64_bit_under_large_models(dev):
+    # c_syntax.ml:111-112: with large_models static indices are uint64_t arguments
+    L.reset_symbols(0)
+    a = L.Node(1, "a", "single", (5, 7)); b = L.Node(2, "b", "single", (7,))
+    st = L.StaticSymbol(L.fresh_symbol(), 5)
+    j = L.fresh_symbol()
+    r = L.Routine("row_of", [L.For(j, 0, 6, [L.Set(b, (L.It(j),), L.Binop(
+        "add", L.Get(a, (L.It(st.sym), L.It(j))), L.EmbedIndex(L.It(j))))])], static_indices=[st])
+    av = np.arange(35, dtype=np.float32).reshape(5, 7)
+    for opts, typ in ((None, "const uint32_t "), ("large_models=1", "const uint64_t ")):
+        code = B.compile(r, opts)
+        assert typ + L.sym_ident(st.sym) in code.source()
+        ctx = B.Context(dev)
+        ctx.set_values(a, av)
+        rt = ctx.link(code)
+        rt.set_static(st.sym, 3)
+        rt.run()
+        assert np.array_equal(ctx.get_values(b), av[3] + np.arange(7))
+        del rt
+        ctx.free()

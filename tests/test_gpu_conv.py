@@ -139,3 +139,21 @@ def test_padded_node_margins_are_reset_before_a_same_convolution(neutral, option
     if neutral == 0.0:
         assert np.allclose(hip.get(y), ora.get(y), rtol=1e-5, atol=1e-5)
     hip.close()
+
+
+def test_input_gradient_at_matrix_core_size_with_overlapping_windows():
+    # x_grad[b, o1+k1, o2+k2, i] += y_grad * w at a size the matrix-core kernels would take (M, N >= 16,
+    # min_mfma_flops=0): the overlapping windows keep it a generated kernel, and the result is the
+    # checker's; the one-to-one case (stride = window) may go to the matrix cores and has to agree too
+    from test_capi_cpu import _conv_input_gradient
+    for stride, ksz in ((1, 3), (3, 3)):
+        r, n = _conv_input_gradient(stride, ksz, b=2, oh=8, ow=8, ic=32, oc=32)
+        rng = np.random.default_rng(stride)
+        init = {n[k].id: rng.uniform(-1, 1, n[k].dims).astype(np.float32) for k in ("w", "dy")}
+        ora = OracleRun(r, init)
+        ora.step()
+        for opts in ("min_mfma_flops=0", "min_mfma_flops=0;mfma=0;coop=0"):
+            hip = HipRun(r, init, opts)
+            hip.step()
+            assert np.allclose(hip.get(n["dx"]), ora.get(n["dx"]), rtol=1e-4, atol=1e-4), (stride, opts)
+            hip.close()

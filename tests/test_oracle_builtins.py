@@ -218,3 +218,87 @@ def test_half_roundtrip_exhaustive(lib):
         else:
             assert got == w
             assert lib.ocn_x_single_to_half_bits(w) == b or (w == 0.0)
+
+
+# ---- the restatement against the reference's own C, in bulk -------------------------------------------
+
+@pytest.fixture(scope="module")
+def ref_lib(reference_root):
+    """The reference's builtins.c (its plain-C part) compiled unchanged by `make -C oracle ref`."""
+    subprocess.run(["make", "-C", os.path.join(ROOT, "oracle"), "ref"], check=True, capture_output=True)
+    return ctypes.CDLL(os.path.join(ROOT, "oracle", "_ref", "builtins_ref.so"))
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+@pytest.mark.parametrize("crypto", [0, 1], ids=["light", "crypto"])
+def test_threefry_bit_identical_to_reference_c(lib, ref_lib, crypto):
+    # builtins.c:195-323, both variants: 20 000 random (key, counter) pairs plus structured ones
+    # (zero key, zero counter, all ones, single bits) that a wrong rotation or key-schedule index shows
+    rng = np.random.default_rng(7 + crypto)
+    n = 20000
+    keys = rng.integers(0, 2**32, (n, 4), dtype=np.uint64).astype(np.uint32)
+    ctrs = rng.integers(0, 2**32, (n, 4), dtype=np.uint64).astype(np.uint32)
+    keys[:64] = 0; ctrs[64:128] = 0; keys[128:160] = 0xFFFFFFFF; ctrs[160:192] = 0xFFFFFFFF
+    for b in range(128):
+        keys[200 + b] = 0; keys[200 + b, b // 32] = 1 << (b % 32)
+        ctrs[400 + b] = 0; ctrs[400 + b, b // 32] = 1 << (b % 32)
+    keys, ctrs = np.ascontiguousarray(keys), np.ascontiguousarray(ctrs)
+    mine, theirs = np.zeros((n, 4), np.uint32), np.ones((n, 4), np.uint32)
+    lib.ocn_x_batch_threefry(crypto, _p(keys), _p(ctrs), _p(mine), n)
+    ref_lib.ocn_x_batch_threefry(crypto, _p(keys), _p(ctrs), _p(theirs), n)
+    assert np.array_equal(mine, theirs)
+    # and the two variants are different functions of their input
+    other = np.zeros((n, 4), np.uint32)
+    lib.ocn_x_batch_threefry(1 - crypto, _p(keys), _p(ctrs), _p(other), n)
+    assert not np.array_equal(mine, other)
+
+
+def test_uniform_converters_bit_identical_to_reference_c(lib, ref_lib):
+    # builtins.c:345-528: every uint4x32 -> uniform converter, vector and scalar forms
+    rng = np.random.default_rng(11)
+    n = 20000
+    xs = rng.integers(0, 2**32, (n, 4), dtype=np.uint64).astype(np.uint32)
+    xs[:8] = 0; xs[8:16] = 0xFFFFFFFF; xs[16:24] = 0x00FFFFFF; xs[24:32] = 0x80000000
+    xs = np.ascontiguousarray(xs)
+
+    def run(l):
+        f4, d2 = np.zeros((n, 4), np.float32), np.zeros((n, 2), np.float64)
+        b8, h8 = np.zeros((n, 8), np.uint16), np.zeros((n, 8), np.float32)
+        f1, d1, b1 = np.zeros(n, np.float32), np.zeros(n, np.float64), np.zeros(n, np.uint16)
+        l.ocn_x_batch_uniform(_p(xs), _p(f4), _p(d2), _p(b8), _p(h8), _p(f1), _p(d1), _p(b1), n)
+        return f4, d2, b8, h8, f1, d1, b1
+
+    for name, a, b in zip(("single_vec", "double_vec", "bf16_vec", "half_vec", "single", "double", "bf16"), run(lib), run(ref_lib)):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), name
+
+
+def test_conversions_and_spreading_bit_identical_to_reference_c(lib, ref_lib):
+    # builtins.c:531-606 (X -> uint4x32) and :611-743 (bf16, fp8): random bit patterns of every float
+    # class (normals, subnormals, infinities, NaNs, both zeros) plus values near the fp8 range edges
+    rng = np.random.default_rng(13)
+    n = 40000
+    bits = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+    bits[:6] = [0, 0x80000000, 0x7F800000, 0xFF800000, 0x7FC00000, 0x00000001]
+    xs = bits.view(np.float32).copy()
+    xs[100:2100] = rng.uniform(-70000, 70000, 2000).astype(np.float32)
+    xs[2100:4100] = (rng.standard_normal(2000) * 1e-5).astype(np.float32)
+
+    def conv(l):
+        bf, f8 = np.zeros(n, np.uint16), np.zeros(n, np.uint8)
+        bfb, f8b = np.zeros(n, np.float32), np.zeros(n, np.float32)
+        l.ocn_x_batch_convert(_p(xs), _p(bf), _p(f8), _p(bfb), _p(f8b), n)
+        return bf, f8, bfb.view(np.uint32), f8b.view(np.uint32)
+
+    for name, a, b in zip(("single_to_bf16", "single_to_fp8", "bf16_to_single", "fp8_to_single"), conv(lib), conv(ref_lib)):
+        assert np.array_equal(a, b), name
+
+    def spread(l):
+        a, b, c = (np.zeros((n, 4), np.uint32) for _ in range(3))
+        l.ocn_x_batch_spread(_p(bits), _p(a), _p(b), _p(c), n)
+        return a, b, c
+
+    for name, a, b in zip(("uint32", "int64", "single"), spread(lib), spread(ref_lib)):
+        assert np.array_equal(a, b), name + "_to_uint4x32"
