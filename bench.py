@@ -110,25 +110,17 @@ def cpu_baseline(name: str):
     return {"value": 1.0 / t, "unit": "steps/s", "cores": 1, "kind": "port", "sample": "20000 full steps"}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="transformer")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--options", default=None, help="compile options for the library, e.g. 'rows=0;bf16_copies=0'")
-    ap.add_argument("--kernel-table", action="store_true", help="print per-kernel times to stderr")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        raise SystemExit("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)")
-
+def measure(workload: str, steps: int, warmup: int, options=None, kernel_table: bool = False):
+    """Runs `steps` timed steps of one workload (after `warmup` untimed ones) and returns the
+    measurements: whole-routine rate, the dominant kernel's roofline (its launches bracketed with HIP
+    events on the device stream inside the timed region), contraction TFLOP/s and generated-kernel GB/s
+    on algorithmic work."""
     from ocannl_amd import backend as B
     from ocannl_amd.backend import HipRun
 
-    w, metric, unit, dtype = build_workload(args.workload)
+    w, metric, unit, dtype = build_workload(workload)
     t_c = time.perf_counter()
-    hip = HipRun(w.routine, w.init, args.options)
+    hip = HipRun(w.routine, w.init, options)
     compile_s = time.perf_counter() - t_c
     kernels = hip.code.kernels()
     statics = {s.sym: 0 for s in w.statics.values()}
@@ -137,7 +129,7 @@ def main():
     def step(i):
         hip.step({sym: i % nb for sym in statics} if statics else None)
 
-    for i in range(max(args.warmup, 1)):
+    for i in range(max(warmup, 1)):
         step(i)
     B.await_(hip.ctx.dev)
 
@@ -168,8 +160,8 @@ def main():
         dom_idx = [longest_gen[1]]
         dom_name = kernels[longest_gen[1]]["name"]
         bound = "hbm"
-    if args.kernel_table:
-        for k, ms in sorted(zip(kernels, per), key=lambda x: -x[1])[:40]:
+    if kernel_table:
+        for k, ms in sorted(zip(kernels, per), key=lambda x: -x[1])[:60]:
             print(f"{ms*1e3:9.1f} us  {k['kind']:9s} {k['name'][:70]:70s} flops={k['flops']:.3g} bytes={k['bytes']:.3g} "
                   f"mnk={k['m']}x{k['n']}x{k['k']}x{k['batch']} coop={k['coop_lanes']}", file=sys.stderr)
 
@@ -181,7 +173,7 @@ def main():
     hip.rt.profile_read()
     B.await_(hip.ctx.dev)
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         step(i)
     B.await_(hip.ctx.dev)
     dt = time.perf_counter() - t0
@@ -199,22 +191,21 @@ def main():
         f32 = "gemm_f32" in dom_name
         peak = PEAKS["mfma_f32"] if f32 else PEAKS["mfma_bf16"]
         roof = {"bound": "mfma", "kernel": dom_name, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                "frac": achieved / peak, "traffic": measured_traffic(args.workload, dom_name),
+                "frac": achieved / peak, "traffic": measured_traffic(workload, dom_name),
                 "launches_per_step": len(dom_idx),
                 "avg_launch_ms": avg_ms, "flops_per_launch": per_launch}
     else:
         per_launch = kernels[dom_idx[0]]["bytes"]
         achieved = per_launch / (avg_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "kernel": dom_name, "achieved": achieved, "peak": PEAKS["hbm"], "unit": "GB/s",
-                "frac": achieved / PEAKS["hbm"], "traffic": measured_traffic(args.workload, dom_name),
+                "frac": achieved / PEAKS["hbm"], "traffic": measured_traffic(workload, dom_name),
                 "launches_per_step": 1, "avg_launch_ms": avg_ms,
                 "bytes_per_launch": per_launch}
-
-    out = {
-        "metric": metric, "value": args.steps / dt, "unit": unit, "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {w.description}", "routine": w.routine.name,
+    hip.close()
+    return {
+        "metric": metric, "value": steps / dt, "unit": unit, "steps": steps, "warmup": warmup,
+        "ms_per_step": dt / steps * 1e3, "dtype": dtype,
+        "config": {"workload": f"{workload}: {w.description}", "routine": w.routine.name,
                    "kernels_per_step": len(kernels), "compile_s": round(compile_s, 2)},
         "roofline": roof,
         "einsum_tflops": (mfma_fl / (mfma_ms * 1e-3) / 1e12) if mfma_ms > 0 else None,
@@ -223,7 +214,44 @@ def main():
         "pointwise_ms_per_step": gen_ms,
         "final_loss": loss,
     }
-    hip.close()
+
+
+# the other benchmark configurations, measured after the headline one: (workload, steps, warm-up)
+OTHER_CONFIGS = (("dense_bf16", 10, 2), ("dense_f32", 5, 1), ("attention", 10, 2), ("char_mlp", 500, 20), ("moons", 500, 20))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="transformer")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="measure only --workload (by default the headline run also times the other configurations)")
+    ap.add_argument("--options", default=None, help="compile options for the library, e.g. 'rows=0;bf16_copies=0'")
+    ap.add_argument("--kernel-table", action="store_true", help="print per-kernel times to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)")
+
+    m = measure(args.workload, args.steps, args.warmup, args.options, args.kernel_table)
+    out = {
+        "metric": m["metric"], "value": m["value"], "unit": m["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": m["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": m["dtype"], "data": "synthetic", "config": m["config"],
+        "roofline": m["roofline"], "einsum_tflops": m["einsum_tflops"], "einsum_ms_per_step": m["einsum_ms_per_step"],
+        "pointwise_gbps": m["pointwise_gbps"], "pointwise_ms_per_step": m["pointwise_ms_per_step"],
+        "final_loss": m["final_loss"],
+    }
+    if args.workload == "transformer" and not args.no_other_configs:
+        # every other configuration, a few steps each, in the same process: the same measurements,
+        # keyed by workload (each with its own roofline for its own dominant kernel)
+        out["configs"] = {}
+        for name, k, wu in OTHER_CONFIGS:
+            c = measure(name, k, wu, args.options)
+            out["configs"][name] = {key: c[key] for key in ("ms_per_step", "value", "unit", "steps", "warmup", "dtype", "roofline",
+                                                            "einsum_tflops", "pointwise_gbps", "config")}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.workload)
     print(json.dumps(out))

@@ -482,6 +482,8 @@ class HipRun:
     what a test or a benchmark steps (``Train.to_routine`` + ``Context.run``, lib/train.ml:108-170)."""
 
     def __init__(self, routine: L.Routine, init: Mapping[int, np.ndarray], options: Optional[str] = None):
+        import sys
+        self.B = sys.modules[__name__]   # the backend module, for callers that hold only the run
         self.routine = routine
         self.code = compile(routine, options)
         self.ctx = Context()

@@ -126,7 +126,7 @@ def test_compile_batch_links_and_runs_each_routine(dev):
     from parity import OracleRun
     w1 = W.dense_contraction(b=128, i=64, o=96, prec="single", which=("fwd",))
     r1 = w1.routine
-    x = r1.param_nodes()[0]
+    x = w1.nodes["x"]
     L.reset_symbols(100)
     i, j = L.fresh_symbol(), L.fresh_symbol()
     out = L.Node(900, "rowsum", "single", (x.dims[0],))
@@ -141,7 +141,7 @@ def test_compile_batch_links_and_runs_each_routine(dev):
     rt1.run(); rt0.run()
     o1, o2 = OracleRun(r1, w1.init), OracleRun(r2, {x.id: w1.init[x.id]})
     o1.step(); o2.step()
-    y = [n for n in r1.param_nodes() if n.id not in w1.init][0]
+    y = w1.nodes["y"]
     assert np.allclose(ctx.get_values(y), o1.get(y), rtol=1e-4, atol=1e-5)
     assert np.allclose(ctx.get_values(out), o2.get(out), rtol=1e-5, atol=1e-5)
     del rt0, rt1

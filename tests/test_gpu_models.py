@@ -144,3 +144,90 @@ def test_full_size_attention_against_torch_autograd():
     sums = W.to_float(hip.get(w.nodes["attn"]), w.nodes["attn"].prec).reshape(-1, 1024)[::997].sum(axis=1)
     assert np.all(np.abs(sums - 1.0) < 2e-2), (sums.min(), sums.max())
     hip.close()
+
+
+def _torch_transformer_steps(w, kw, steps, dev):
+    """The architecture of benchmark configuration 4 in plain PyTorch, fp32, on `dev`: embedding by a
+    one-hot product + positions, post-norm blocks (lib/nn_blocks.ml:222-285: masked soft-max attention,
+    layer norm whose "mean" is the plain sum as written there, relu feed-forward), soft-max cross
+    entropy averaged over tokens, SGD.  Returns the losses and the updated parameters."""
+    layers, dk = kw["layers"], kw["d_model"] // kw["heads"]
+    by_ident = {n.ident.rsplit("_", 1)[0]: n for n in w.routine.param_nodes()}
+    t32 = lambda n: torch.tensor(W.to_float(w.init[n.id], n.prec).astype(np.float32), device=dev)
+    x_in, target, mask = (t32(by_ident[k]) for k in ("input_batch", "target_batch", "mask"))
+    P = {label: t32(node).requires_grad_(True) for label, node in w.nodes.items() if label not in ("loss", "logits")}
+
+    def layer_norm(x, gamma, beta, eps=1e-5):
+        d = x.shape[-1]
+        centered = (x - x.sum(-1, keepdim=True)) / d
+        return gamma * (centered / torch.sqrt((centered * centered).sum(-1, keepdim=True) + eps)) + beta
+
+    losses = []
+    for _ in range(steps):
+        for p in P.values():
+            p.grad = None
+        x = torch.einsum("mv,bsv->bsm", P["w_embed"], x_in) + P["pos_encoding"]
+        for li in range(layers):
+            lb = f"l{li}"
+            q = torch.einsum("hdm,bsm->bshd", P[f"w_q_{lb}"], x)
+            k = torch.einsum("hdm,btm->bthd", P[f"w_k_{lb}"], x)
+            v = torch.einsum("hem,btm->bthe", P[f"w_v_{lb}"], x)
+            scores = torch.einsum("bshd,bthd->bsht", q, k) / float(np.sqrt(dk))
+            attn = torch.softmax(torch.where(mask[None, :, None, :] != 0, scores, torch.tensor(-1e9, device=dev)), dim=-1)
+            mha = torch.einsum("mhe,bshe->bsm", P[f"w_o_{lb}"], torch.einsum("bsht,bthe->bshe", attn, v))
+            x1 = layer_norm(x + mha, P[f"gamma_ln1_{lb}"], P[f"beta_ln1_{lb}"])
+            hid = torch.relu(torch.einsum("fm,bsm->bsf", P[f"w_ffn1_{lb}"], x1) + P[f"b_ffn1_{lb}"])
+            x = layer_norm(x1 + torch.einsum("mf,bsf->bsm", P[f"w_ffn2_{lb}"], hid), P[f"gamma_ln2_{lb}"], P[f"beta_ln2_{lb}"])
+        logits = torch.einsum("vm,bsm->bsv", P["w_out"], x)
+        loss = -(torch.log_softmax(logits, dim=-1) * target).sum() / (x_in.shape[0] * x_in.shape[1])
+        loss.backward()
+        losses.append(float(loss.detach()))
+        with torch.no_grad():
+            for p in P.values():
+                p -= kw["lr"] * p.grad
+    return losses, {k: p.detach() for k, p in P.items()}
+
+
+def test_full_size_transformer_step_against_torch_autograd():
+    # benchmark configuration 4 at its real size (4 blocks, d_model 512, 8 heads, d_ff 2048, seq 256,
+    # batch 32, vocabulary 4096; bf16 values, fp32 gradients) against the same architecture in plain
+    # PyTorch fp32 on the same device: the loss after each of three steps and the updated parameters
+    # (every stored bf16 intermediate carries a 2^-9 rounding: the bar for bf16 routines, 2e-2, applies
+    # to the loss relative to its size and to the parameter UPDATES in the Frobenius norm)
+    import inspect
+    kw = {k: v.default for k, v in inspect.signature(W.transformer).parameters.items() if v.default is not inspect.Parameter.empty}
+    w = W.transformer()
+    hip = HipRun(w.routine, w.init)
+    dev = torch.device("cuda:0")
+    steps = 3
+    want, P = _torch_transformer_steps(w, kw, steps, dev)
+    got = []
+    for _ in range(steps):
+        hip.step()
+        got.append(float(W.to_float(hip.get(w.nodes["loss"]), w.nodes["loss"].prec)[0]))
+    assert np.all(np.abs(np.array(got) - np.array(want)) <= 2e-2 * np.maximum(np.abs(want), 1.0)), (got, want)
+    errs = {}
+    for name in ("w_q_l0", "w_ffn2_l3", "w_out", "gamma_ln1_l0", "w_embed", "b_ffn1_l2"):
+        n = w.nodes[name]
+        start = W.to_float(w.init[n.id], n.prec).astype(np.float64)
+        mine = W.to_float(hip.get(n), n.prec).astype(np.float64)
+        ref = P[name].cpu().numpy().astype(np.float64)
+        errs[name] = (float(np.linalg.norm(mine - ref) / np.linalg.norm(ref)),
+                      float(np.linalg.norm((mine - start) - (ref - start)) / max(np.linalg.norm(ref - start), 1e-30)))
+    print("full-size transformer vs torch: losses", got, want, "errors (value, update)", errs)
+    assert all(e[0] <= 2e-2 for e in errs.values()), errs
+    hip.close()
+
+
+def test_small_transformer_loss_curve_100_steps():
+    # the north star's wording for fp32: loss curves over 100 steps within 1e-3 of the `cc` semantics
+    kw = dict(batch=2, seq=16, d_model=32, heads=2, d_ff=64, layers=2, vocab=64, grad_prec="single", lr=0.05)
+    w = W.transformer(prec="single", **kw)
+    hip, ora = HipRun(w.routine, w.init, "min_mfma_flops=100000"), OracleRun(w.routine, w.init)
+    lh, lo = [], []
+    for _ in range(100):
+        hip.step(); ora.step()
+        lh.append(float(hip.get(w.nodes["loss"])[0])); lo.append(float(ora.get(w.nodes["loss"])[0]))
+    assert lo[-1] < 0.5 * lo[0]
+    assert np.max(np.abs(np.array(lh) - np.array(lo))) <= 1e-3, float(np.max(np.abs(np.array(lh) - np.array(lo))))
+    hip.close()
