@@ -292,11 +292,65 @@ __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, 
   });
 }
 
+// The same row of tiles through LDS, for full tiles whose rows start on 16-byte boundaries: the
+// accumulators go to this wave's staging area as fp32 [32][TN * 32] (ds_write_b32, a half-wave per
+// 128-byte row piece), come back row-wise as 16-byte chunks, and every lane stores 16 bytes (four
+// fp32 or eight bf16 results) next to its neighbours' -- an eighth (a quarter) of the store
+// instructions of the direct form, each covering whole cache lines.  `stage` holds 32 * (TN * 32 + 4)
+// floats of this wave's own; LDS operations of one wave complete in order, so no barrier is needed.
+template <int TN, int OUT, bool ACC>
+__device__ __forceinline__ void store_tile_row_wide(f32x16 (&acc)[TN], float* stage, void* origin, long ld, int lane,
+                                                    void* origin2 = nullptr) {
+  constexpr int CW = TN * 32, LS = CW + 4;
+  static_assert(TN == 2 || TN == 4, "tile rows of 2 or 4 tiles");
+  asm volatile("" : "+a"(acc[0]), "+a"(acc[1]));
+  if constexpr (TN == 4) asm volatile("" : "+a"(acc[2]), "+a"(acc[3]));
+  float* const wr = stage + ((lane >> 5) * 4) * LS + (lane & 31);
+  static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
+    static_for<16>([&](auto ec) OCN_LAMBDA_INLINE {
+      constexpr int j = decltype(jc)::value, e = decltype(ec)::value, r = (e >> 2) * 8 + (e & 3);
+      wr[r * LS + j * 32] = acc[j][e];
+    });
+  });
+  constexpr int VEC = OUT == kOutBf16 ? 8 : 4;     // results per lane
+  constexpr int LPR = CW / VEC, RPP = 64 / LPR;    // lanes per row, rows per pass
+  const int rr = lane / LPR, cc = (lane % LPR) * VEC;
+  const float* const rd = stage + rr * LS + cc;
+  const unsigned goff = (unsigned)rr * (unsigned)ld + (unsigned)cc;
+  static_for<32 / RPP>([&](auto pc) OCN_LAMBDA_INLINE {
+    constexpr int p = decltype(pc)::value;
+    const long row_off = (long)(p * RPP) * ld;     // uniform
+    f32x4 v0 = *reinterpret_cast<const f32x4*>(rd + p * RPP * LS);
+    if constexpr (OUT == kOutBf16) {
+      f32x4 v1 = *reinterpret_cast<const f32x4*>(rd + p * RPP * LS + 4);
+      u32x4* const dst = reinterpret_cast<u32x4*>(static_cast<unsigned short*>(origin) + row_off + goff);
+      if (ACC) {
+        const u32x4 o = *dst;
+        v0 += f32x4{__uint_as_float(o.x << 16), __uint_as_float(o.x & 0xFFFF0000u), __uint_as_float(o.y << 16), __uint_as_float(o.y & 0xFFFF0000u)};
+        v1 += f32x4{__uint_as_float(o.z << 16), __uint_as_float(o.z & 0xFFFF0000u), __uint_as_float(o.w << 16), __uint_as_float(o.w & 0xFFFF0000u)};
+      }
+      *dst = u32x4{pack2(v0.x, v0.y), pack2(v0.z, v0.w), pack2(v1.x, v1.y), pack2(v1.z, v1.w)};
+    } else {
+      f32x4* const dst = reinterpret_cast<f32x4*>(static_cast<float*>(origin) + row_off + goff);
+      if (ACC) v0 += *dst;
+      *dst = v0;
+      if constexpr (OUT == kOutF32Copy) {
+        typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+        *reinterpret_cast<u32x2*>(static_cast<unsigned short*>(origin2) + row_off + goff) = u32x2{pack2(v0.x, v0.y), pack2(v0.z, v0.w)};
+      }
+    }
+  });
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 // (m, n) is the origin of the wave's block.  The variant is picked per row of tiles with a
 // wave-uniform switch: that bounds what the compiler can hoist above the branch to one row's
 // registers (hoisting all 256 accumulator reads above one up-front branch spills them).
+// `stage`: this wave's own LDS area of at least 32 * (TN * 32 + 4) floats, free once the main loop
+// has passed its last barrier.
 template <int TM, int TN>
-__device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, void* c2base, f32x16 (&acc)[TM][TN], long m, long n, long co, int lane) {
+__device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, void* c2base, f32x16 (&acc)[TM][TN], long m, long n, long co, int lane,
+                                         float* stage) {
   const long rows_left = g.M - m, cols_left = g.N - n;
   if (rows_left <= 0 || cols_left <= 0) return;
   const bool full = rows_left >= TM * 32 && cols_left >= TN * 32;
@@ -307,7 +361,14 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, void* c
   char* const origin = (to_ws ? reinterpret_cast<char*>(g.ws) : static_cast<char*>(cbase)) + first * (bf ? 2 : 4);
   const bool copy = !to_ws && !bf && c2base != nullptr;   // (with split-K the reduction pass writes the copy)
   char* const origin2 = copy ? static_cast<char*>(c2base) + first * 2 : nullptr;
-  const int variant = (copy ? 8 : bf ? 4 : 0) + ((!to_ws && g.accumulate) ? 2 : 0) + (full ? 0 : 1);
+  // 16-byte stores need rows that start on 16-byte boundaries (and 8-byte ones for the bf16 copy)
+  const bool wide = full && ((reinterpret_cast<unsigned long>(origin) | (unsigned long)(ld * (bf ? 2 : 4))) & 15) == 0 &&
+                    (!copy || ((reinterpret_cast<unsigned long>(origin2) | (unsigned long)(ld * 2)) & 7) == 0) &&
+                    (unsigned long)ld * 32 < 0x100000000ul;
+  // fp32 results already leave as 128-byte row pieces per half-wave and go out directly (measured:
+  // staging them gains nothing, the burst of a tile's results is bound by the memory system); bf16
+  // results and bf16 copies would leave as 2-byte elements and take the staged form
+  const int variant = (copy ? 8 : bf ? 4 : 0) + ((!to_ws && g.accumulate) ? 2 : 0) + ((copy || bf) ? (wide ? 0 : 1) : (full ? 0 : 1));
   static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
     constexpr int i = decltype(ic)::value;
     void* o = origin + (long)i * 32 * ld * (bf ? 2 : 4);
@@ -318,13 +379,13 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, void* c
       case 1: store_tile_row<TN, kOutF32, false, true>(acc[i], o, ld, lane, rl, cols_left); break;
       case 2: store_tile_row<TN, kOutF32, true, false>(acc[i], o, ld, lane, rl, cols_left); break;
       case 3: store_tile_row<TN, kOutF32, true, true>(acc[i], o, ld, lane, rl, cols_left); break;
-      case 4: store_tile_row<TN, kOutBf16, false, false>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 4: store_tile_row_wide<TN, kOutBf16, false>(acc[i], stage, o, ld, lane); break;
       case 5: store_tile_row<TN, kOutBf16, false, true>(acc[i], o, ld, lane, rl, cols_left); break;
-      case 6: store_tile_row<TN, kOutBf16, true, false>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 6: store_tile_row_wide<TN, kOutBf16, true>(acc[i], stage, o, ld, lane); break;
       case 7: store_tile_row<TN, kOutBf16, true, true>(acc[i], o, ld, lane, rl, cols_left); break;
-      case 8: store_tile_row<TN, kOutF32Copy, false, false>(acc[i], o, ld, lane, rl, cols_left, o2); break;
+      case 8: store_tile_row_wide<TN, kOutF32Copy, false>(acc[i], stage, o, ld, lane, o2); break;
       case 9: store_tile_row<TN, kOutF32Copy, false, true>(acc[i], o, ld, lane, rl, cols_left, o2); break;
-      case 10: store_tile_row<TN, kOutF32Copy, true, false>(acc[i], o, ld, lane, rl, cols_left, o2); break;
+      case 10: store_tile_row_wide<TN, kOutF32Copy, true>(acc[i], stage, o, ld, lane, o2); break;
       default: store_tile_row<TN, kOutF32Copy, true, true>(acc[i], o, ld, lane, rl, cols_left, o2); break;
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -558,7 +619,9 @@ gemm_bf16_kernel(const GemmArgs g) {
     pipeline();
   }
 
-  epilogue<TM, TN>(g, cbase, c2base, acc, m0 + wm0, n0 + wn0, co, lane);
+  // (every wave has passed the last barrier of the main loop: the operand stages are free)
+  epilogue<TM, TN>(g, cbase, c2base, acc, m0 + wm0, n0 + wn0, co, lane,
+                   reinterpret_cast<float*>(smem) + wave * ((kAT + kBT) / 4));
 }
 
 // ---- fp32 compute -------------------------------------------------------------------------------
@@ -695,7 +758,7 @@ gemm_f32_kernel(const GemmArgs g) {
     __syncthreads();
   }
 
-  epilogue<TM, TN>(g, cbase, c2base, acc, m0 + wm0, n0 + wn0, co, lane);
+  epilogue<TM, TN>(g, cbase, c2base, acc, m0 + wm0, n0 + wn0, co, lane, fsm + wave * ((kAT + kBT) / 2));
 }
 
 template <int BM, int BN, bool A_KC, bool B_KC>
