@@ -66,6 +66,9 @@ typedef struct {
                               sharing the launch count as batch entries, a chain of operand pairs into
                               one result as a longer k                                                 */
   char name[96];
+  int32_t queue;           /* 0 = the device's main queue; 1 = its side queue: a contraction off the critical
+                              path that runs beside the kernels that follow it (compile option side_queue=0|1) */
+  int32_t reserved;
 } ocannl_hip_kernel_info;
 
 const char* ocannl_hip_last_error(void);
@@ -117,7 +120,13 @@ int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** code);
    of tiny phases as one single-workgroup kernel), groups=0|1 (independent contractions of identical
    shapes share a launch), chains=0|1 (`c =+ a * b` statements into one result with identical operand
    shapes share a launch), parallel=0|1 (consecutive small phases that do not depend on one another
-   run side by side in one launch), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
+   run side by side in one launch), debug_log=0|1 (in-routine logging, see
+   ocannl_hip_routine_log_id; the wire form then carries every Set's text), side_queue=0|1 (contractions
+   whose results nothing needs for a while -- weight gradients -- run on a second queue of the device, beside
+   the kernels that follow), fused=0|1|2 (a short-K contraction whose only reader is the row-wise
+   kernel that follows -- attention scores ahead of the soft-max chain -- runs on the matrix cores as that
+   kernel's prologue, into LDS, instead of as a launch of its own; 2: also when its result is a context
+   node that has to be stored anyway), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
    indices and offsets in generated kernels, the `large_models` setting of c_syntax.ml:111-112; a
    routine with a node of more than 2^31 - 1 elements gets them without asking). */
 int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, ocannl_hip_code** code);
@@ -158,6 +167,14 @@ int ocannl_hip_routine_run(ocannl_hip_routine* routine);
    the previous call's contents (nothing in it needs to start at zero: every routine fills what it
    reads); calls that overlap on one GPU -- other than in order on the device's one stream -- race. */
 int ocannl_hip_routine_run_static_scratch(ocannl_hip_routine* routine);
+/* debug_log_from_routines (arrayjit/lib/utils.ml:591; c_syntax.ml:493-535; cuda_backend.ml:871-893,992-1041):
+   a routine compiled with the option debug_log=1 prints, from the device, what every statement
+   computes: `<log id>: # <statement>$` and `<log id>: lhs[offset]{=old} = new = expression{=values}$`
+   (`$` stands for a newline, as in the CUDA backend), comments as `<log id>: COMMENT: text$`, in program
+   order -- such a routine runs every top-level statement as ONE thread.  The lines go to the process's
+   standard output when the device is next synchronised; this returns the id of the routine's latest
+   run, the prefix by which the host picks its lines out (Utils.add_log_processor ~prefix). */
+int ocannl_hip_routine_log_id(ocannl_hip_routine* routine, int* log_id);
 /* Same, bracketing every kernel with HIP events on the device stream; synchronises and writes the
    per-kernel milliseconds (cap >= number of kernels).  For measurement only. */
 int ocannl_hip_routine_run_timed(ocannl_hip_routine* routine, float* kernel_ms, int cap);

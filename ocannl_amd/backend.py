@@ -53,14 +53,15 @@ class _Kparam(ctypes.Structure):
 class KernelInfo(ctypes.Structure):
     _fields_ = [("kind", ctypes.c_int32), ("coop_lanes", ctypes.c_int32), ("flops", ctypes.c_double),
                 ("bytes", ctypes.c_double), ("m", ctypes.c_int64), ("n", ctypes.c_int64),
-                ("k", ctypes.c_int64), ("batch", ctypes.c_int64), ("name", ctypes.c_char * 96)]
+                ("k", ctypes.c_int64), ("batch", ctypes.c_int64), ("name", ctypes.c_char * 96),
+                ("queue", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
     KINDS = ("generated", "fill", "mfma")
 
     def as_dict(self):
         return {"kind": self.KINDS[self.kind], "coop_lanes": self.coop_lanes, "flops": self.flops,
                 "bytes": self.bytes, "m": self.m, "n": self.n, "k": self.k, "batch": self.batch,
-                "name": self.name.decode()}
+                "name": self.name.decode(), "queue": self.queue}
 
 
 # every symbol include/ocannl_hip.h declares
@@ -75,7 +76,7 @@ EXPORTS = (
     "ocannl_hip_code_routine_name", "ocannl_hip_code_kparams", "ocannl_hip_code_source",
     "ocannl_hip_code_num_kernels", "ocannl_hip_code_kernel_info", "ocannl_hip_link",
     "ocannl_hip_routine_free", "ocannl_hip_routine_set_static", "ocannl_hip_routine_run",
-    "ocannl_hip_routine_run_static_scratch", "ocannl_hip_routine_run_timed",
+    "ocannl_hip_routine_run_static_scratch", "ocannl_hip_routine_log_id", "ocannl_hip_routine_run_timed",
     "ocannl_hip_routine_profile_kernel", "ocannl_hip_routine_profile_read",
 )
 
@@ -129,6 +130,7 @@ def load_library() -> ctypes.CDLL:
         "ocannl_hip_routine_set_static": (i32, [vp, i32, i64]),
         "ocannl_hip_routine_run": (i32, [vp]),
         "ocannl_hip_routine_run_static_scratch": (i32, [vp]),
+        "ocannl_hip_routine_log_id": (i32, [vp, P(i32)]),
         "ocannl_hip_routine_run_timed": (i32, [vp, P(ctypes.c_float), i32]),
         "ocannl_hip_routine_profile_kernel": (i32, [vp, i32]),
         "ocannl_hip_routine_profile_read": (i32, [vp, P(ctypes.c_double), P(i64)]),
@@ -320,7 +322,9 @@ def compile(routine: L.Routine, options: Optional[str] = None) -> Code:  # noqa:
 
 def compile_batch(routines: Sequence[L.Routine], options: Optional[str] = None) -> Code:
     """``Lowered_backend.compile_batch`` (backend_impl.ml:349-353)."""
-    text = "".join(L.to_wire(r) for r in routines).encode()
+    # with debug_log=1 every Set carries its text, as Low_level.Set's `debug` field does
+    debug = options is not None and "debug_log=1" in options.replace(" ", "")
+    text = "".join(L.to_wire(r, debug=debug) for r in routines).encode()
     h = ctypes.c_void_p()
     lib = load_library()
     if options is None:
@@ -356,6 +360,12 @@ class Routine:
         """``run`` with the routine's scratch memory taken from the library's static device array:
         allocates nothing; refuses (``User_error``) a routine whose scratch needs exceed it."""
         _check(load_library().ocannl_hip_routine_run_static_scratch(self._h))
+
+    def log_id(self) -> int:
+        """The prefix of the log lines of this routine's latest run (``debug_log=1``)."""
+        v = ctypes.c_int()
+        _check(load_library().ocannl_hip_routine_log_id(self._h, ctypes.byref(v)))
+        return v.value
 
     def profile_kernel(self, kernel_index: int) -> None:
         _check(load_library().ocannl_hip_routine_profile_kernel(self._h, kernel_index))
@@ -508,3 +518,15 @@ class HipRun:
         await_(self.ctx.dev)
         del self.rt
         self.ctx.free()
+
+
+def routine_log_lines(stdout_text: str, log_id: int) -> List[str]:
+    """The log of one run out of captured standard output: the lines that start with ``<log_id>: ``,
+    prefix removed, ``$`` turned back into line ends (``Utils.log_debug_routine_logs``)."""
+    prefix = f"{log_id}: "
+    out: List[str] = []
+    for chunk in stdout_text.split("$"):
+        chunk = chunk.rsplit("\n", 1)[-1]   # (other output of the process may sit between two log lines)
+        if chunk.startswith(prefix):
+            out.append(chunk[len(prefix):])
+    return out

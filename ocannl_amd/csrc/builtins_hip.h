@@ -184,3 +184,47 @@ OCN_DEV uint4x32_t fp8_to_uint4x32(unsigned char x) { return ocn_u4(x, 0u, 0u, 0
 // ---- lane-group combine used by cooperative reductions ------------------------------------------
 OCN_DEV float ocn_xshfl(float v, int m) { return __shfl_xor(v, m, 64); }
 OCN_DEV double ocn_xshfl(double v, int m) { return __shfl_xor(v, m, 64); }
+
+// ---- a contraction as the prologue of a row-wise kernel ---------------------------------------------
+// xs[32][T] = A[32][K] * B[T][K]^T for a workgroup of NW waves: bf16 operands, both unit-stride
+// along K, fp32 accumulation on the matrix cores (v_mfma_f32_32x32x16_bf16), results rounded to XT
+// (bf16 bits or float) in LDS.  The workgroup's NW waves take the T / 32 column tiles in turn.  The MFMA
+// fragments come straight from memory: a lane supplies row (lane % 32) of its operand at
+// k = 8 * (lane / 32) .. + 7 of each 16-k sub-step (16 bytes), and receives column (lane % 32) of the
+// 32 x 32 result at rows 8 * (e / 4) + 4 * (lane / 32) + e % 4.
+typedef __bf16 ocn_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float ocn_f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int ocn_u32x4 __attribute__((ext_vector_type(4)));
+
+OCN_DEV void ocn_rowtile_put(unsigned short* p, float v) { *p = single_to_bfloat16(v); }
+OCN_DEV void ocn_rowtile_put(float* p, float v) { *p = v; }
+
+template <int T, int K, int NW, typename XT>
+__device__ __forceinline__ void ocn_rowtile_contract(const unsigned short* __restrict__ a, long long a_row,
+                                                     const unsigned short* __restrict__ b, long long b_row, XT* xs) {
+  static_assert(T % 32 == 0 && K % 16 == 0 && K <= 128, "row tile: T in steps of 32, K in steps of 16 up to 128");
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;   // NW waves share the T / 32 column tiles
+  constexpr int KS = K / 16;
+  if (wave >= T / 32) return;
+  ocn_bf16x8 af[KS];
+  const unsigned short* ap = a + (long long)(lane & 31) * a_row + (lane >> 5) * 8;
+#pragma unroll
+  for (int kk = 0; kk < KS; ++kk) af[kk] = __builtin_bit_cast(ocn_bf16x8, *reinterpret_cast<const ocn_u32x4*>(ap + kk * 16));
+#pragma unroll
+  for (int t = 0; t < (T / 32 + NW - 1) / NW; ++t) {
+    const int n0 = (wave + t * NW) * 32;
+    if (n0 >= T) break;
+    const unsigned short* bp = b + (long long)(n0 + (lane & 31)) * b_row + (lane >> 5) * 8;
+    ocn_bf16x8 bf[KS];
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) bf[kk] = __builtin_bit_cast(ocn_bf16x8, *reinterpret_cast<const ocn_u32x4*>(bp + kk * 16));
+    ocn_f32x16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk], bf[kk], acc, 0, 0, 0);
+    XT* out = xs + ((lane >> 5) * 4) * T + n0 + (lane & 31);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) ocn_rowtile_put(out + ((e >> 2) * 8 + (e & 3)) * T, acc[e]);
+  }
+}

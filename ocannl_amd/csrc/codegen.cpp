@@ -368,6 +368,97 @@ struct Printer {
     return ind + "for (" + idx_t + " " + sym + " = " + std::to_string(from) + " + lane_; " + sym + " <= " + std::to_string(to) +
            "; " + sym + " += " + std::to_string(lanes) + ") {";
   }
+  // row group with a contraction prologue: reads of this node come from the LDS tile `xs_` that the
+  // kernel computed itself: [row of the tile][row position]
+  int lds_node = -1;
+  std::string lds_row;
+  int64_t lds_ld = 0;
+  // ---- debug logging (debug_log_from_routines; c_syntax.ml:493-535 and debug_float, :857-) ----------
+  // A statement prints `# <its text>` and `<lhs>[<offset>]{=<old value>} = <new value> = <expression
+  // with the value of every read in braces>`, as the reference's generated code does; every line starts
+  // with the run's log id and ends in `$` for a newline (cuda_backend.ml:874-893), for the host to split.
+  bool debug_log = false;
+  struct Dbg { std::string fmt; std::vector<std::string> args; };
+  static std::string lit(const std::string& t) {   // text inside a C string literal that is a printf format
+    std::string o;
+    for (char ch : t) {
+      if (ch == '%') o += "%%";
+      else if (ch == '"') o += "\\\"";
+      else if (ch == '\\') o += "\\\\";
+      else if (ch == '\n') o += "$";
+      else o += ch;
+    }
+    return o;
+  }
+  static bool loggable(Prec p) { return p != Prec::Uint4x32 && p != Prec::Void; }
+  std::string as_double(Prec from, const std::string& e) { Pair c = convert_precision(from, Prec::Double); return c.first + e + c.second; }
+  // op syntax around already-formatted sub-expressions: print it around placeholders, escape, put them back
+  std::string wrap_fmt(const std::string& with_marks, const std::vector<std::string>& subs) {
+    std::string o = lit(with_marks);
+    for (size_t i = 0; i < subs.size(); ++i) {
+      const std::string mark = std::string("\001") + (char)('A' + i) + "\001";
+      for (size_t at = o.find(mark); at != std::string::npos; at = o.find(mark, at + subs[i].size())) o.replace(at, mark.size(), subs[i]);
+    }
+    return o;
+  }
+  Dbg dbg(Prec prec, const Scalar& s) {
+    Dbg d;
+    switch (s.kind) {
+      case Scalar::LocalScope: case Scalar::GetLocal: {
+        const Prec sp = r.node(s.scope.node).prec;
+        Pair c = convert_precision(sp, prec);
+        const std::string v = c.first + scope_name(s.scope) + c.second;
+        d.fmt = lit(v) + "{=%g}";
+        d.args.push_back(loggable(prec) ? as_double(prec, v) : "0.0");
+        return d;
+      }
+      case Scalar::Get: case Scalar::GetMerge: {
+        const Node& n = r.node(s.node);
+        Pair c = convert_precision(n.prec, prec);
+        const std::string name = s.kind == Scalar::GetMerge ? "merge_buffer" : n.ident;
+        const std::string off = offset_str(s.idcs, n.dims);
+        d.fmt = lit(c.first + name) + "[%u]" + lit(c.second) + "{=%g}";
+        d.args.push_back("(unsigned)(" + off + ")");
+        d.args.push_back(loggable(prec) && loggable(n.prec) ? as_double(prec, c.first + name + "[" + off + "]" + c.second) : "0.0");
+        return d;
+      }
+      case Scalar::GetDyn: {   // the table is not dereferenced in the log: the index value is what is shown
+        std::vector<Def> defs;
+        d.fmt = lit(r.node(s.node).ident + "@dyn_idx") + "{=%g}";
+        d.args.push_back(as_double(s.arg_prec, scalar(s.arg_prec, *s.a, "", defs)));
+        return d;
+      }
+      case Scalar::Const: { Pair c = convert_precision(Prec::Double, prec); d.fmt = lit(c.first + const_str(s.cst) + c.second); return d; }
+      case Scalar::Bits: { Pair c = convert_precision(Prec::Int64, prec); d.fmt = lit(c.first + std::to_string((long long)s.bits) + "LL" + c.second); return d; }
+      case Scalar::Index: d.fmt = lit(axis_str(s.index)); return d;
+      case Scalar::Un: {
+        Dbg a = dbg(s.un == Unop::Uniform1 ? s.arg_prec : prec, *s.a);
+        d.fmt = wrap_fmt(emit_unop(prec, s.un, "\001A\001"), {a.fmt});
+        d.args = a.args;
+        return d;
+      }
+      case Scalar::Bin: {
+        if (s.bin == Binop::Arg1) return dbg(prec, *s.a);
+        if (s.bin == Binop::Arg2) return dbg(prec, *s.b);
+        Dbg a = dbg(prec, *s.a), b = dbg(prec, *s.b);
+        d.fmt = wrap_fmt(emit_binop(prec, s.bin, "\001A\001", "\001B\001"), {a.fmt, b.fmt});
+        d.args = a.args; d.args.insert(d.args.end(), b.args.begin(), b.args.end());
+        return d;
+      }
+      case Scalar::Tern: {
+        Dbg a = dbg(s.tern == Ternop::Where ? s.arg_prec : prec, *s.a), b = dbg(prec, *s.b), c = dbg(prec, *s.c);
+        d.fmt = wrap_fmt(emit_ternop(prec, s.tern, "\001A\001", "\001B\001", "\001C\001"), {a.fmt, b.fmt, c.fmt});
+        d.args = a.args; d.args.insert(d.args.end(), b.args.begin(), b.args.end()); d.args.insert(d.args.end(), c.args.begin(), c.args.end());
+        return d;
+      }
+    }
+    return d;
+  }
+  std::string log_call(const std::string& fmt, const std::vector<std::string>& args) {
+    std::string c = "printf(\"%d: " + fmt + "$\", log_id";
+    for (auto& a : args) c += ", " + a;
+    return c + ");";
+  }
   // when set, a read of exactly this (node, indices) prints as `self_name`
   const Stmt* self_set = nullptr;
   std::string self_name;
@@ -418,6 +509,10 @@ struct Printer {
         const Node& n = r.node(s.node);
         Pair c = convert_precision(n.prec, prec);
         if (self_set && s.node == self_set->node && s.idcs == self_set->idcs) return c.first + self_name + c.second;
+        if (s.node == lds_node) {
+          note_idx(s.idcs.back());
+          return c.first + "xs_[" + lds_row + " * " + std::to_string(lds_ld) + "u + " + axis_str(s.idcs.back()) + "]" + c.second;
+        }
         if (cache_defined.count(s.node)) return c.first + cache_name.at(s.node) + c.second;
         note(s.node, s.idcs);
         if (shadow_live.count(s.node)) return c.first + shadow.at(s.node) + "[" + offset_str(s.idcs, n.dims) + "]" + c.second;
@@ -541,7 +636,10 @@ struct Printer {
 
   void stmt(const Stmt& c, const std::string& ind, std::vector<std::string>& out) {
     switch (c.kind) {
-      case Stmt::Comment: out.push_back(ind + "/* " + c.text + " */"); break;
+      case Stmt::Comment:
+        if (debug_log) out.push_back(ind + log_call("COMMENT: " + lit(c.text), {}));
+        else out.push_back(ind + "/* " + c.text + " */");
+        break;
       case Stmt::For: {
         const std::string s = sym_ident(c.sym);
         out.push_back(ind + "for (" + idx_t + " " + s + " = " + std::to_string(c.from) + "; " + s + " <= " +
@@ -565,6 +663,20 @@ struct Printer {
         note(c.node, c.idcs);
         std::vector<Def> defs;
         std::string v = scalar(n.prec, *c.value, ind + "  ", defs);
+        if (debug_log && loggable(n.prec)) {
+          // { T new_set_v = value; log "# text"; log "lhs[off]{=old} = new = expression{=values}"; lhs[off] = new_set_v; }
+          const std::string off = offset_str(c.idcs, n.dims), lhs = n.ident + "[" + off + "]";
+          Dbg d = dbg(n.prec, *c.value);
+          std::vector<std::string> args{"(unsigned)(" + off + ")", as_double(n.prec, lhs), as_double(n.prec, "new_set_v")};
+          args.insert(args.end(), d.args.begin(), d.args.end());
+          std::vector<std::string> lines{std::string(c_typ(n.prec)) + " new_set_v = " + v + ";"};
+          if (!c.text.empty()) lines.push_back(log_call("# " + lit(c.text), {}));
+          lines.push_back(log_call(lit(n.ident) + "[%u]{=%g} = %g = " + d.fmt, args));
+          lines.push_back(store_line(c.node, lhs, "new_set_v", store_guard));
+          if (defs.empty()) { out.push_back(ind + "{"); for (auto& l : lines) out.push_back(ind + "  " + l); out.push_back(ind + "}"); }
+          else with_defs(defs, lines, ind, out);
+          break;
+        }
         with_defs(defs, {store_line(c.node, n.ident + "[" + offset_str(c.idcs, n.dims) + "]", v, store_guard)}, ind, out);
         break;
       }
@@ -597,7 +709,20 @@ struct Printer {
       }
       case Stmt::SetLocal: {
         std::vector<Def> defs;
-        std::string v = scalar(r.node(c.scope.node).prec, *c.value, ind + "  ", defs);
+        const Prec sp = r.node(c.scope.node).prec;
+        std::string v = scalar(sp, *c.value, ind + "  ", defs);
+        if (debug_log && loggable(sp)) {
+          const std::string name = scope_name(c.scope);
+          Dbg d = dbg(sp, *c.value);
+          std::vector<std::string> args{as_double(sp, name), as_double(sp, "new_set_v")};
+          args.insert(args.end(), d.args.begin(), d.args.end());
+          std::vector<std::string> lines{std::string(c_typ(sp)) + " new_set_v = " + v + ";",
+                                         log_call("# local " + lit(name + " := " + v), {}),
+                                         log_call(lit(name) + "{=%g} = %g = " + d.fmt, args), name + " = new_set_v;"};
+          if (defs.empty()) { out.push_back(ind + "{"); for (auto& l : lines) out.push_back(ind + "  " + l); out.push_back(ind + "}"); }
+          else with_defs(defs, lines, ind, out);
+          break;
+        }
         with_defs(defs, {scope_name(c.scope) + " = " + v + ";"}, ind, out);
         break;
       }
@@ -754,9 +879,11 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     Printer pr(r);
     if (plan.large_index) pr.idx_t = "uint64_t";
     pr.mirrors = &plan.mirrors;
+    pr.debug_log = plan.debug_log;
     std::vector<std::string> body;
     const std::string ind = "  ";
 
+    int fused_block = 0;   // > 0: the kernel is a row group with a contraction prologue and wants this workgroup size
     // one phase for the thread (or loop iteration) identified by gtid_; `skip` leaves it
     auto emit_points = [&](const Phase& q, const std::string& pind, const std::string& skip) {
       const int QG = q.coop_lanes;
@@ -766,6 +893,98 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
         body.push_back(pind + "uint64_t pt_ = gtid_ / " + std::to_string(QG) + "u;");
       } else {
         body.push_back(pind + "uint64_t pt_ = gtid_;");
+      }
+      if (!q.members.empty() && q.fused_x >= 0) {
+        // ---- row group with a contraction prologue: a workgroup owns 32 rows (consecutive along outer
+        //      axis fused_m_axis); it computes their part of x into LDS on the matrix cores, then each of
+        //      its four waves runs the members over eight of the rows
+        const Node& xn = r.node(q.fused_x);
+        const size_t n = q.row_outer_ext.size();
+        const int ma = q.fused_m_axis;
+        QP = 1;
+        for (size_t k = 0; k < n; ++k) QP *= (uint64_t)(k == (size_t)ma ? q.row_outer_ext[k] / 32 : q.row_outer_ext[k]);
+        // 16 waves of two rows each for short rows; long rows keep more of what they produce in
+        // registers and take 8 waves of four rows
+        const int NW = q.row_len <= 512 ? 16 : 8, RPW = 32 / NW;
+        fused_block = NW * 64;
+        body.pop_back(); body.pop_back();   // (lane_ / pt_ as laid out for lane groups: redone per workgroup)
+        body.push_back(pind + "const uint32_t lane_ = threadIdx.x & 63u, wave_ = threadIdx.x >> 6;");
+        body.push_back(pind + "uint64_t pt_ = gtid_ / " + std::to_string(fused_block) + "u;");
+        body.push_back(pind + "if (pt_ >= " + std::to_string(QP) + "ull) " + skip + ";");
+        for (int k = (int)n - 1; k >= 0; --k) {
+          const std::string ext = std::to_string(k == ma ? q.row_outer_ext[k] / 32 : q.row_outer_ext[k]) + "ull";
+          std::string line = pind + "const " + pr.idx_t + " t" + std::to_string(k) + "_ = (" + pr.idx_t + ")(";
+          if (k == 0) line += "pt_);";
+          else line += "pt_ % " + ext + "); pt_ /= " + ext + ";";
+          body.push_back(line);
+        }
+        const std::string xt = c_typ(xn.prec);
+        body.push_back(pind + "__shared__ __attribute__((aligned(16))) " + xt + " xs_[" + std::to_string(32 * q.row_len) + "];");
+        {
+          pr.used_nodes.insert(q.fused_a.node); pr.used_nodes.insert(q.fused_b.node);
+          std::string ao = std::to_string(q.fused_a.offset) + "ull", bo = std::to_string(q.fused_b.offset) + "ull";
+          for (size_t k = 0; k < n; ++k) {
+            const std::string tk = "(uint64_t)t" + std::to_string(k) + "_" + (k == (size_t)ma ? " * 32ull" : "");
+            if (q.fused_a_stride[k]) ao += " + " + tk + " * " + std::to_string(q.fused_a_stride[k]) + "ull";
+            if (q.fused_b_stride[k]) bo += " + " + tk + " * " + std::to_string(q.fused_b_stride[k]) + "ull";
+          }
+          body.push_back(pind + "ocn_rowtile_contract<" + std::to_string(q.row_len) + ", " + std::to_string(q.fused_k) + ", " +
+                         std::to_string(NW) + ", " + xt + ">(" +
+                         r.node(q.fused_a.node).ident + " + (" + ao + "), " + std::to_string(q.fused_a_stride[ma]) + "ll, " +
+                         r.node(q.fused_b.node).ident + " + (" + bo + "), " + std::to_string(q.fused_b_row) + "ll, xs_);");
+        }
+        body.push_back(pind + "__syncthreads();");
+        if (q.row_len % 64 != 0 || q.row_len / 64 > 16 || QG != 64) throw InvalidArgument("planner: fused row group of a shape the kernel does not take");
+        pr.row_iters = (int)(q.row_len / 64);
+        for (auto& m : q.members) {
+          const Stmt& st = *m.inner[0];
+          if (pr.cache_name.count(st.node)) continue;
+          const Node& wn = r.node(st.node);
+          bool per_position = false;
+          for (auto& ix : st.idcs) if (ix.kind == AxisIndex::Iter && ix.sym == m.row_sym && m.row_role == Phase::RowPointwise) per_position = true;
+          const std::string base = "c" + std::to_string(st.node) + "_";
+          if (per_position) {
+            body.push_back(pind + c_typ(wn.prec) + " " + base + "[" + std::to_string(pr.row_iters) + "];");
+            pr.cache_name[st.node] = base + "[it_]";
+          } else {
+            body.push_back(pind + c_typ(wn.prec) + " " + base + ";");
+            pr.cache_name[st.node] = base;
+          }
+        }
+        body.push_back(pind + "for (uint32_t rl_ = 0; rl_ < " + std::to_string(RPW) + "u; ++rl_) {");
+        const std::string rind = pind + "  ";
+        for (size_t k = 0; k < n; ++k)
+          body.push_back(rind + "const " + pr.idx_t + " row" + std::to_string(k) + "_ = t" + std::to_string(k) + "_" +
+                         (k == (size_t)ma ? " * 32u + wave_ * " + std::to_string(RPW) + "u + rl_;" : ";"));
+        pr.lds_node = q.fused_x; pr.lds_row = "(wave_ * " + std::to_string(RPW) + "u + rl_)"; pr.lds_ld = q.row_len;
+        if (q.fused_x_store) {
+          // x is visible outside the kernel: its rows go to memory as well (adjacent lanes adjacent elements)
+          pr.used_nodes.insert(q.fused_x);
+          std::string off;
+          for (size_t k = 0; k < n; ++k) off = k == 0 ? "(uint64_t)row0_" : "(" + off + ") * " + std::to_string(q.row_outer_ext[k]) + "ull + row" + std::to_string(k) + "_";
+          body.push_back(rind + "_Pragma(\"unroll\") for (uint32_t it_ = 0; it_ < " + std::to_string(pr.row_iters) + "; ++it_) " + xn.ident +
+                         "[(" + off + ") * " + std::to_string(q.row_len) + "ull + lane_ + it_ * 64u] = xs_[" + pr.lds_row + " * " +
+                         std::to_string(q.row_len) + "u + lane_ + it_ * 64u];");
+        }
+        for (size_t mi = 0; mi < q.members.size(); ++mi) {
+          const Phase& m = q.members[mi];
+          body.push_back(rind + "{  /* " + m.label + " */");
+          const std::string mi_ind = rind + "  ";
+          for (size_t k = 0; k < m.row_outer_syms.size(); ++k)
+            body.push_back(mi_ind + "const " + pr.idx_t + " " + sym_ident(m.row_outer_syms[k]) + " = row" + std::to_string(k) + "_;");
+          if (m.row_role == Phase::RowPointwise) {
+            body.push_back(pr.row_loop(sym_ident(m.row_sym), 0, q.row_len - 1, QG, mi_ind));
+            emit_phase_statements(r, pr, m, 1, false, mi_ind + "  ", body);
+            body.push_back(mi_ind + "}");
+          } else {
+            emit_phase_statements(r, pr, m, QG, true, mi_ind, body);
+          }
+          body.push_back(rind + "}");
+        }
+        body.push_back(pind + "}");
+        pr.lds_node = -1;
+        pr.row_iters = 0; pr.cache_name.clear(); pr.cache_defined.clear();
+        return (uint64_t)(QP * (uint64_t)fused_block);
       }
       if (!q.members.empty()) {
         // ---- row group: a lane group owns one row and runs the member phases in order
@@ -893,11 +1112,21 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
       total_threads = emit_points(ph, ind, "return");
     }
 
+    if (plan.debug_log) {
+      // one thread runs the phase (the planner kept every loop sequential); the routine's top-level
+      // comments since the previous phase come first, those after the last phase at the very end
+      std::vector<std::string> head;
+      for (auto& t : ph.comments_before) head.push_back(ind + "if (gtid_ == 0) " + pr.log_call("COMMENT: " + Printer::lit(t), {}));
+      body.insert(body.begin() + 1, head.begin(), head.end());   // (after the line that defines gtid_)
+      bool last_generic = true;
+      for (size_t q = pi + 1; q < plan.phases.size(); ++q) last_generic = last_generic && plan.phases[q].kind != Phase::Generic;
+      if (last_generic) for (auto& t : plan.trailing_comments) body.push_back(ind + pr.log_call("COMMENT: " + Printer::lit(t), {}));
+    }
     GeneratedKernel gk;
     gk.name = r.name + "_k" + std::to_string(kidx++);
     gk.phase_index = (int)pi;
     gk.threads = total_threads;
-    gk.block = 256;
+    gk.block = fused_block > 0 ? fused_block : 256;
     std::vector<std::string> decls;
     for (int id : r.node_order) {
       if (!pr.used_nodes.count(id)) continue;
@@ -922,8 +1151,9 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
       decls.push_back(std::string(plan.large_index ? "const uint64_t " : "const uint32_t ") + sym_ident(s.sym));
       gk.params.push_back({KernelParam::StaticIdx, s.sym});
     }
+    if (plan.debug_log) { decls.push_back("const int log_id"); gk.params.push_back({KernelParam::LogId, 0}); }
     src << "/* phase " << pi << ": " << ph.label << " */\n";
-    src << "extern \"C\" __global__ void __launch_bounds__(256) " << gk.name << "(";
+    src << "extern \"C\" __global__ void __launch_bounds__(" << gk.block << ") " << gk.name << "(";
     for (size_t i = 0; i < decls.size(); ++i) src << (i ? ", " : "") << decls[i];
     src << ") {\n";
     for (auto& l : body) src << l << "\n";

@@ -16,7 +16,7 @@
 namespace ocannl {
 
 struct KernelParam {
-  enum Kind { NodePtr, StaticIdx, MergeBuffer } kind;
+  enum Kind { NodePtr, StaticIdx, MergeBuffer, LogId } kind;   // LogId: `int log_id`, the prefix of the run's log lines
   int id;   // node id (NodePtr; MergeBuffer: the node whose layout the buffer has) or static symbol
 };
 

@@ -172,6 +172,7 @@ StmtP parse_stmt(const Sx& x) {
   else if (h == "set") {
     s->kind = Stmt::Set; s->node = (int)to_int(x.at(1)); s->idcs = parse_indices(x.at(2));
     s->value = parse_scalar(x.at(3));
+    if (x.kids.size() > 4) s->text = x.at(4).s;   // Low_level.Set's `debug` field: the statement as text
   } else if (h == "set_vec") {
     s->kind = Stmt::SetVec; s->node = (int)to_int(x.at(1)); s->idcs = parse_indices(x.at(2));
     s->length = (int)to_int(x.at(3));

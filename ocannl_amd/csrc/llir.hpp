@@ -93,7 +93,7 @@ struct Scalar {
 
 struct Stmt {
   enum Kind : uint8_t { Comment, For, ZeroOut, Set, SetVec, SetLocal, DeclareLocal } kind;
-  std::string text;          // Comment
+  std::string text;          // Comment; Set: its `debug` text when the routine was serialised with one
   int sym = 0; int64_t from = 0, to = 0;  // For (inclusive bounds, c_syntax.ml:450-456)
   Block body;                // For
   int node = 0;              // ZeroOut / Set / SetVec

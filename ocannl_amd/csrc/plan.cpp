@@ -507,6 +507,7 @@ bool phase_touches(const Phase& ph, int node) {
     return ph.gemm.a.node == node || ph.gemm.b.node == node || ph.gemm.c.node == node;
   }
   if (!ph.parallel_members.empty()) { for (auto& m : ph.parallel_members) if (phase_touches(m, node)) return true; return false; }
+  if (ph.fused_x >= 0 && (ph.fused_x == node || ph.fused_a.node == node || ph.fused_b.node == node)) return true;
   if (!ph.members.empty()) { for (auto& m : ph.members) if (phase_touches(m, node)) return true; return false; }
   if (!ph.serial_members.empty()) { for (auto& m : ph.serial_members) if (phase_touches(m, node)) return true; return false; }
   std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
@@ -526,6 +527,9 @@ Block strip_comments(const Block& b, std::string* last_comment) {
 }
 
 }  // namespace
+
+// debug logging: every loop of a statement stays inside one thread, in program order
+static thread_local bool g_all_sequential = false;
 
 // Chain/inner split and parallel classification of one top-level statement.
 // Returns false when the statement runs nothing (a zero-trip loop).
@@ -567,7 +571,7 @@ static bool analyze_nest(const Routine& r, const StmtP& sp, Phase& ph) {
   inner_loops(inner);
   for (const Stmt* l : chain) {
     const int64_t ext = l->to - l->from + 1;
-    const bool par = !whole && !foreign && symbol_is_parallel(l->sym, acc, extents);
+    const bool par = !g_all_sequential && !whole && !foreign && symbol_is_parallel(l->sym, acc, extents);
     if (par) { ph.par_syms.push_back(l->sym); ph.par_from.push_back(l->from); ph.par_ext.push_back(ext); }
     else { ph.seq_syms.push_back(l->sym); ph.seq_from.push_back(l->from); ph.seq_to.push_back(l->to); }
   }
@@ -1144,7 +1148,7 @@ bool same_layout(const GemmOperand& x, const GemmOperand& y) {
   return true;
 }
 
-void merge_contractions(Plan& plan, bool chain) {
+void merge_contractions(Plan& plan, bool chain, int window = 1 << 30) {
   std::map<int, int> mirror_source;   // bf16 copy -> the tensor whose stores keep it in step
   for (auto& kv : plan.mirrors) mirror_source[kv.second] = kv.first;
   auto source_of = [&](int node) { auto m = mirror_source.find(node); return m == mirror_source.end() ? node : m->second; };
@@ -1193,6 +1197,7 @@ void merge_contractions(Plan& plan, bool chain) {
       Phase& p = plan.phases[i];
       GemmDesc& g = p.gemm;
       if (g.group.size() + g.more.size() >= 3) break;
+      if (!chain && (long)j - (long)i > (long)window) break;
       Phase& q = plan.phases[j];
       const GemmDesc& h = q.gemm;
       bool candidate = q.kind == Phase::Contraction && h.group.empty() && h.more.empty() && h.M == g.M && h.N == g.N &&
@@ -1373,7 +1378,7 @@ void group_independent(const Routine& r, Plan& plan) {
   };
   auto sets_of = [&](const Phase& ph) {
     Sets s;
-    if (ph.kind != Phase::Generic || !ph.serial_members.empty() || !ph.parallel_members.empty()) return s;
+    if (ph.kind != Phase::Generic || !ph.serial_members.empty() || !ph.parallel_members.empty() || ph.fused_x >= 0) return s;
     if (ph.bytes > (double)(32 << 20)) return s;
     bool ok = true;
     if (ph.members.empty()) ok = add_accesses(ph, s);
@@ -1474,6 +1479,7 @@ bool phase_writes(const Phase& ph, int node) {
     for (auto& a : acc) if (a.write && a.node == node) return true;
     return false;
   };
+  if (ph.fused_x == node && ph.fused_x_store) return true;
   if (!ph.members.empty()) { for (auto& m : ph.members) if (writes(m)) return true; return false; }
   if (!ph.parallel_members.empty()) { for (auto& m : ph.parallel_members) if (phase_writes(m, node)) return true; return false; }
   if (!ph.serial_members.empty()) { for (auto& m : ph.serial_members) if (phase_writes(m, node)) return true; return false; }
@@ -1695,24 +1701,206 @@ void lift_routine_locals(Routine& r, Plan& plan) {
 
 }  // namespace
 
+// ---- a contraction as the prologue of the row group that consumes it ------------------------------------
+// `x[o.., t] = sum_k a[..] * b[..]` with a short K (both operands unit-stride along it) whose only
+// reader is the row group that follows -- Q K^T ahead of the soft-max chain, dOut V^T ahead of its
+// backward chain -- is taken out of the plan: the group's kernel computes 32 rows of x at a time on
+// the matrix cores into LDS and its members read them there.  Saves a launch, the write of x when it
+// is planner scratch, and its read in either case.
+namespace {
+
+void fuse_row_contractions(Routine& r, Plan& plan, bool also_stored) {
+  std::map<int, int> mirror_source;
+  for (auto& kv : plan.mirrors) mirror_source[kv.second] = kv.first;
+  for (size_t j = 0; j < plan.phases.size(); ++j) {
+    Phase& G = plan.phases[j];
+    if (G.kind != Phase::Generic || G.members.empty() || G.fused_x >= 0) continue;
+    if (G.coop_lanes != 64 || G.row_len % 128 != 0 || G.row_len / 64 > 16 || G.row_outer_ext.empty()) continue;
+    // tensors the members read without having written them, through the identity signature only
+    std::set<int> written, bad;
+    std::vector<int> cands;
+    const size_t n_outer = G.row_outer_ext.size();
+    std::string identity;
+    for (size_t k = 0; k < n_outer; ++k) identity += "o" + std::to_string(k) + ",";
+    identity += "r,";
+    for (auto& m : G.members) {
+      std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+      block_accesses(m.inner, acc, w, f, d);
+      for (auto& a : acc) {
+        if (a.write) { written.insert(a.node); continue; }
+        if (written.count(a.node)) continue;
+        if (row_signature(m, *a.idcs) != identity) { bad.insert(a.node); continue; }
+        if (std::find(cands.begin(), cands.end(), a.node) == cands.end()) cands.push_back(a.node);
+      }
+    }
+    for (int X : cands) {
+      if (bad.count(X) || written.count(X)) continue;
+      const Node& xn = r.node(X);
+      if (xn.dims.size() != n_outer + 1 || xn.dims.back() != G.row_len) continue;
+      bool dims_ok = true;
+      for (size_t k = 0; k < n_outer; ++k) dims_ok = dims_ok && xn.dims[k] == G.row_outer_ext[k];
+      if (!dims_ok || !(xn.prec == Prec::Bfloat16 || xn.prec == Prec::Single)) continue;
+      if ((int64_t)32 * G.row_len * prec_in_bytes(xn.prec) > 65536) continue;   // the rows live in static LDS
+      // the producer: the latest earlier phase that writes x
+      int i = -1;
+      for (int q = (int)j - 1; q >= 0; --q) if (phase_writes(plan.phases[q], X)) { i = q; break; }
+      if (i < 0) continue;
+      const Phase& P = plan.phases[i];
+      const GemmDesc& g = P.gemm;
+      if (P.kind != Phase::Contraction || g.c.node != X || g.accumulate || !g.group.empty() || !g.more.empty() || g.c_copy >= 0) continue;
+      if (g.a.prec != Prec::Bfloat16 || g.b.prec != Prec::Bfloat16 || g.a.s_k != 1 || g.b.s_k != 1) continue;
+      if (g.K % 16 != 0 || g.K > 128 || g.N != G.row_len) continue;
+      if (!g.a.static_terms.empty() || !g.b.static_terms.empty() || !g.c.static_terms.empty() || g.c.offset != 0) continue;
+      if (P.inner.size() != 1 || P.inner[0]->kind != Stmt::Set) continue;
+      const Stmt& set = *P.inner[0];
+      const Scalar& v = *set.value;
+      if (!(v.kind == Scalar::Tern && v.tern == Ternop::Fma && v.a->kind == Scalar::Get && v.b->kind == Scalar::Get)) continue;
+      // x must be written through plain iterators, one per axis
+      std::vector<int> xsym;   // (-1: an axis of extent 1 written at position 0)
+      bool plain = set.idcs.size() == xn.dims.size();
+      std::set<int> distinct;
+      for (size_t p = 0; p < set.idcs.size() && plain; ++p) {
+        const AxisIndex& ix = set.idcs[p];
+        if (ix.kind == AxisIndex::Fixed && ix.fixed == 0 && xn.dims[p] == 1) { xsym.push_back(-1); continue; }
+        plain = ix.kind == AxisIndex::Iter && !r.is_static(ix.sym) && distinct.insert(ix.sym).second;
+        xsym.push_back(ix.sym);
+      }
+      if (!plain || xsym.back() < 0) continue;
+      Strides s1 = strides_of(r, v.a->node, v.a->idcs), s2 = strides_of(r, v.b->node, v.b->idcs);
+      const int nsym = xsym.back();
+      const bool first_is_a = get_stride(s1, nsym) == 0 && get_stride(s2, nsym) != 0;
+      const bool second_is_a = get_stride(s2, nsym) == 0 && get_stride(s1, nsym) != 0;
+      if (!first_is_a && !second_is_a) continue;
+      const Strides& sa = first_is_a ? s1 : s2;
+      const Strides& sb = first_is_a ? s2 : s1;
+      // the one remaining loop symbol is K: unit stride in both operands
+      std::vector<int> ksyms;
+      auto all_syms = P.par_syms; all_syms.insert(all_syms.end(), P.seq_syms.begin(), P.seq_syms.end());
+      for (int sy : all_syms) if (std::find(xsym.begin(), xsym.end(), sy) == xsym.end()) ksyms.push_back(sy);
+      if (ksyms.size() != 1 || get_stride(sa, ksyms[0]) != 1 || get_stride(sb, ksyms[0]) != 1) continue;
+      if (!sa.statics.empty() || !sb.statics.empty()) continue;
+      Phase F;   // the fields, filled in before G is touched
+      F.fused_a = g.a; F.fused_b = g.b;
+      F.fused_a.offset = sa.offset; F.fused_b.offset = sb.offset;
+      F.fused_k = g.K;
+      F.fused_b_row = get_stride(sb, nsym);
+      bool aligned = F.fused_b_row % 8 == 0 && sa.offset % 8 == 0 && sb.offset % 8 == 0;
+      int m_axis = -1;
+      for (size_t k = 0; k < n_outer; ++k) {
+        const int64_t ak = xsym[k] < 0 ? 0 : get_stride(sa, xsym[k]), bk = xsym[k] < 0 ? 0 : get_stride(sb, xsym[k]);
+        F.fused_a_stride.push_back(ak); F.fused_b_stride.push_back(bk);
+        aligned = aligned && ak % 8 == 0 && bk % 8 == 0 && ak >= 0 && bk >= 0;
+        if (bk == 0 && ak != 0 && G.row_outer_ext[k] % 32 == 0 && (m_axis < 0 || G.row_outer_ext[k] > G.row_outer_ext[m_axis])) m_axis = (int)k;
+      }
+      if (!aligned || m_axis < 0) continue;
+      // nothing between the contraction and the group may touch x or write the operands; nothing else
+      // before the group may read x; a later reader means the rows have to be stored
+      auto source_of = [&](int node) { auto m = mirror_source.find(node); return m == mirror_source.end() ? node : m->second; };
+      bool free_to_move = true;
+      for (size_t q = (size_t)i + 1; q < j && free_to_move; ++q) {
+        const Phase& mid = plan.phases[q];
+        free_to_move = !phase_touches(mid, X) && !phase_writes(mid, g.a.node) && !phase_writes(mid, g.b.node) &&
+                       !phase_writes(mid, source_of(g.a.node)) && !phase_writes(mid, source_of(g.b.node));
+      }
+      if (!free_to_move) continue;
+      bool later_reader = false;
+      for (size_t q = j + 1; q < plan.phases.size(); ++q) later_reader = later_reader || phase_touches(plan.phases[q], X);
+      // When the rows have to be stored anyway the separate launches were measured faster (the
+      // transformer step's backward soft-max chain: 112 us apart, 150 us as one kernel).
+      if ((xn.mode == Mode::Ctx || later_reader) && !also_stored) continue;
+      G.fused_x = X;
+      G.fused_x_store = xn.mode == Mode::Ctx || later_reader;
+      G.fused_a = F.fused_a; G.fused_b = F.fused_b;
+      G.fused_a_stride = F.fused_a_stride; G.fused_b_stride = F.fused_b_stride;
+      G.fused_b_row = F.fused_b_row; G.fused_k = F.fused_k; G.fused_m_axis = m_axis;
+      G.flops = P.flops;
+      const double x_bytes = (double)xn.size_in_bytes();
+      G.bytes += P.bytes - 2.0 * x_bytes + (G.fused_x_store ? x_bytes : 0.0);   // x is neither written (unless stored) nor read
+      G.label = P.label + " -> " + G.label;
+      if (!G.fused_x_store) r.nodes.at(X).mode = Mode::Virtual;   // no memory behind it any more
+      plan.phases.erase(plan.phases.begin() + i);
+      --j;
+      break;
+    }
+  }
+}
+
+}  // namespace
+
+// ---- contractions off the critical path ---------------------------------------------------------------
+// A weight gradient `dW += dY^T X` is needed only when the optimiser runs, dozens of phases later, while
+// the kernels that follow it form a chain in which each waits for the one before and few fill the
+// chip.  Such a contraction is put on the device's second queue: it starts once the main queue has
+// reached its position and runs beside the phases that follow; the first phase that touches its result
+// or rewrites one of its operands waits for it.  Same kernels, same operands, same bits.
+namespace {
+
+void assign_side_queue(Plan& plan) {
+  std::map<int, int> mirror_source;
+  for (auto& kv : plan.mirrors) mirror_source[kv.second] = kv.first;
+  auto source_of = [&](int node) { auto m = mirror_source.find(node); return m == mirror_source.end() ? node : m->second; };
+  struct Sets { std::vector<int> outs, ins; };
+  auto sets_of = [&](const Phase& ph) {
+    Sets s;
+    const GemmDesc& g = ph.gemm;
+    s.outs = {g.c.node}; s.ins = {g.a.node, g.b.node};
+    if (g.c_copy >= 0) s.outs.push_back(g.c_copy);
+    for (auto& m : g.group) { s.outs.push_back(m.c.node); if (m.c_copy >= 0) s.outs.push_back(m.c_copy); s.ins.push_back(m.a.node); s.ins.push_back(m.b.node); }
+    for (auto& pr : g.more) { s.ins.push_back(pr.first.node); s.ins.push_back(pr.second.node); }
+    for (int o : std::vector<int>(s.outs)) { auto m = plan.mirrors.find(o); if (m != plan.mirrors.end()) s.outs.push_back(m->second); }
+    return s;
+  };
+  auto conflicts = [&](const Sets& s, const Phase& later) {
+    for (int o : s.outs) if (phase_touches(later, o)) return true;
+    for (int i : s.ins) if (phase_writes(later, i) || phase_writes(later, source_of(i))) return true;
+    return false;
+  };
+  constexpr size_t kMinSlack = 4;   // phases that must lie between the contraction and its first dependant
+  for (size_t p = 0; p < plan.phases.size(); ++p) {
+    Phase& ph = plan.phases[p];
+    if (ph.kind != Phase::Contraction || ph.flops < 4e9) continue;
+    const Sets s = sets_of(ph);
+    size_t q = p + 1;
+    while (q < plan.phases.size() && !conflicts(s, plan.phases[q])) ++q;
+    if (q - p > kMinSlack) ph.stream = 1;
+  }
+  // every phase of the main queue waits for the side-queue phases before it that it conflicts with
+  // (side-queue phases among themselves run in order)
+  for (size_t p = 0; p < plan.phases.size(); ++p) {
+    if (plan.phases[p].stream != 1) continue;
+    const Sets s = sets_of(plan.phases[p]);
+    for (size_t q = p + 1; q < plan.phases.size(); ++q)
+      if (plan.phases[q].stream == 0 && conflicts(s, plan.phases[q])) plan.phases[q].wait_for.push_back((int)p);
+  }
+}
+
+}  // namespace
+
 Plan make_plan(Routine& r, const PlanOptions& requested) {
   PlanOptions opt = requested;
   if (r.merge_node >= 0) {
     // routines that read the merge buffer are short pointwise accumulations (cuda_backend.ml:1009-1011
     // binds the buffer at launch): plain one-kernel-per-statement plans, no fusing rewrites
-    opt.enable_mfma = opt.enable_row_groups = opt.enable_serial_group = opt.enable_bf16_copies = false;
+    opt.enable_mfma = opt.enable_row_groups = opt.enable_serial_group = opt.enable_bf16_copies = opt.fuse_row_contractions = false;
   }
+  if (opt.debug_log) {
+    opt.enable_mfma = opt.enable_coop = opt.enable_row_groups = opt.enable_serial_group = opt.enable_parallel_groups = false;
+    opt.enable_bf16_copies = opt.fuse_row_contractions = opt.side_queue = false;
+  }
+  struct SeqGuard { bool old; SeqGuard(bool v) : old(g_all_sequential) { g_all_sequential = v; } ~SeqGuard() { g_all_sequential = old; } } seq_guard(opt.debug_log);
   Plan plan;
+  plan.debug_log = opt.debug_log;
   plan.large_index = opt.large_models;
   for (auto& kv : r.nodes) if (kv.second.num_elems() > (int64_t)0x7FFFFFFF) plan.large_index = true;
   std::string label;
   int next_sym = 0;
   Bf16Copies copies;
   lift_routine_locals(r, plan);
+  std::vector<std::string> pending_comments;
   Block top = r.body;
   for (size_t ti = 0; ti < top.size(); ++ti) {
     StmtP sp = top[ti];
-    if (sp->kind == Stmt::Comment) { label = sp->text; continue; }
+    if (sp->kind == Stmt::Comment) { label = sp->text; if (opt.debug_log) pending_comments.push_back(sp->text); continue; }
     Phase ph;
     ph.label = label;
     ph.stmt = sp;
@@ -1744,7 +1932,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     // the nest overwrites all of it: every axis is a full-range parallel iterator or has extent 1.
     Binop accum;
     int fill_at = -1;
-    if (!devirt && reduction_shape(r, ph, &accum) && accum == Binop::Add) {
+    if (!devirt && !opt.debug_log && reduction_shape(r, ph, &accum) && accum == Binop::Add) {
       // the latest Zero_out of the target with nothing touching the target in between
       const int target = ph.inner[0]->node;
       for (int q = (int)plan.phases.size() - 1; q >= 0; --q) {
@@ -1770,7 +1958,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     }
     // a dead fill: the nest stores to every element of a tensor without reading it, and nothing has
     // touched the tensor since its Zero_out
-    if (!devirt && fill_at < 0 && ph.seq_syms.empty() && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set) {
+    if (!devirt && !opt.debug_log && fill_at < 0 && ph.seq_syms.empty() && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set) {
       const int target = ph.inner[0]->node;
       std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
       block_accesses(ph.inner, acc, w, f, d);
@@ -1794,13 +1982,17 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
       set_contraction_bytes(ph);
       if (opt.enable_bf16_copies) use_bf16_copies(r, plan, ph, copies, &next_sym);
     }
+    ph.comments_before.swap(pending_comments);
     plan.phases.push_back(std::move(ph));
   }
+  plan.trailing_comments.swap(pending_comments);
   if (opt.enable_mfma && opt.merge_chains) merge_contractions(plan, true);
-  if (opt.enable_mfma && opt.group_contractions) merge_contractions(plan, false);
+  if (opt.enable_mfma && opt.group_contractions) merge_contractions(plan, false, opt.group_window);
   if (opt.enable_coop && opt.enable_row_groups) group_rows(r, plan);
+  if (opt.enable_mfma && opt.enable_coop && opt.enable_row_groups && opt.fuse_row_contractions) fuse_row_contractions(r, plan, opt.fuse_stored_rows);
   if (opt.enable_serial_group) serialise_tiny(r, plan);
   if (opt.enable_coop && opt.enable_parallel_groups) group_independent(r, plan);
+  if (opt.enable_mfma && opt.side_queue && r.merge_node < 0) assign_side_queue(plan);
   return plan;
 }
 

@@ -95,10 +95,31 @@ struct Phase {
   // depend on one another (the updates of many small parameters) run as ONE kernel in which every
   // member owns a range of workgroups.
   std::vector<Phase> parallel_members;
+  // Row group with a contraction prologue (members non-empty, fused_x >= 0): the tensor `fused_x` that
+  // the members read row by row -- the result of a `+*` contraction with a short K (attention scores
+  // Q K^T, their gradient dOut V^T) -- is not read from memory: the kernel computes 32 rows of it on
+  // the matrix cores into LDS (a workgroup owns 32 consecutive positions of outer axis `fused_m_axis`,
+  // the other outer axes fixed), then its four waves run the members over eight rows each.  When the
+  // tensor is a context node, or something later reads it, the rows are stored as well.
+  int fused_x = -1;
+  bool fused_x_store = false;
+  GemmOperand fused_a, fused_b;                       // node, precision, constant offset (strides below)
+  std::vector<int64_t> fused_a_stride, fused_b_stride;   // element stride per outer axis of the group
+  int64_t fused_b_row = 0;                            // stride of B along the row position
+  int64_t fused_k = 0;                                // contracted extent (unit stride in both operands)
+  int fused_m_axis = -1;
   // Fill
   int fill_node = -1;
   // Contraction
   GemmDesc gemm;
+  // Launch order across the device's two queues.  stream 1: this contraction is off the critical path
+  // (nothing reads its result or rewrites its operands for a while: weight gradients wait for the
+  // optimiser) and runs on the side queue, next to the phases that follow it on the main one.
+  // wait_for: phases of the side queue that this phase must see finished before it starts.
+  int stream = 0;
+  std::vector<int> wait_for;
+  // debug logging: the routine's top-level comments since the previous phase, logged ahead of this one
+  std::vector<std::string> comments_before;
   // accounting (algorithmic): distinct elements read + written, and flops
   double bytes = 0, flops = 0;
 };
@@ -113,6 +134,15 @@ struct PlanOptions {
   bool merge_chains = true;         // `c =+ a_i * b_i` chains of equal shapes as one launch
   bool enable_parallel_groups = true;   // consecutive independent small phases as one launch
   bool large_models = false;        // 64-bit offsets in generated kernels even when every node is small
+  // debug_log_from_routines (arrayjit/lib/utils.ml:591, c_syntax.ml:493-535): every statement logs what
+  // it computes.  The reference runs a routine as one thread, so its log is in program order; here
+  // every top-level statement becomes a kernel of ONE thread that walks its loops in order, and none
+  // of the fusing rewrites applies.
+  bool debug_log = false;
+  int group_window = 1 << 30;        // contractions share a launch only when at most this many phases apart
+  bool side_queue = true;            // contractions off the critical path run on a second queue beside the rest
+  bool fuse_row_contractions = true; // a short-K contraction feeding a row group runs as that kernel's prologue ...
+  bool fuse_stored_rows = false;     // ... also when its result has to be stored anyway (a context node): measured slower
   bool enable_bf16_copies = true;   // keep bf16 copies of fp32 operands of mixed contractions (written by the producing kernels)
 };
 
@@ -123,6 +153,8 @@ struct Plan {
   // the node also stores the rounded value to the copy): the copy feeds bf16 contractions
   std::map<int, int> mirrors;
   bool large_index = false;    // generated kernels compute offsets in 64 bits
+  bool debug_log = false;      // generated kernels print what they compute (and take an `int log_id` argument)
+  std::vector<std::string> trailing_comments;   // debug logging: comments after the last phase
 };
 
 Plan make_plan(Routine& r, const PlanOptions& opt);

@@ -49,6 +49,7 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(uint4* p, uint64_t n16) 
 struct ocannl_hip_device {
   int ordinal = 0;
   hipStream_t stream = nullptr;
+  hipStream_t side_stream = nullptr;   // second queue for contractions off the critical path (Phase::stream == 1)
   void* static_scratch = nullptr;   // this device's copy of `scratch` (hipGetSymbolAddress at device set-up)
   std::map<int, std::pair<void*, uint64_t>> pools;   // pool_id -> (base, size)
   uint64_t used = 0;
@@ -129,6 +130,10 @@ PlanOptions parse_options(const char* options) {
     else if (k == "large_models") o.large_models = v != "0";
     else if (k == "groups") o.group_contractions = v != "0";
     else if (k == "chains") o.merge_chains = v != "0";
+    else if (k == "side_queue") o.side_queue = v != "0";
+    else if (k == "debug_log") o.debug_log = v != "0";
+    else if (k == "group_window") o.group_window = std::stoi(v);
+    else if (k == "fused") { o.fuse_row_contractions = v != "0"; o.fuse_stored_rows = v == "2"; }
     else if (k == "parallel") o.enable_parallel_groups = v != "0";
     else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
     else throw InvalidArgument("compile options: unknown key '" + k + "'");
@@ -152,10 +157,15 @@ struct ocannl_hip_routine {
   void* scratch = nullptr;           // the routine's own arena: local nodes, planner scratch, split-K workspace
   uint64_t scratch_bytes = 0;
   bool counted = false;              // included in the device's live_routines
+  int log_id = 0;                    // debug logging: prefix of this run's log lines (cuda_backend.ml:992-993)
   // Everything that names arena memory exists twice: [0] bound to the routine's own arena, [1] bound to
   // the library's static scratch array (valid when static_ok).
   bool static_ok = false;
   void* gemm_ws[2] = {nullptr, nullptr};   // split-K workspace
+  void* gemm_ws_side = nullptr;            // ... of the contractions on the side queue (own arena only)
+  // side queue: per side-queue phase an event the side queue waits for (recorded on the main queue at
+  // the phase's position) and one recorded when the phase has finished; created at link time
+  std::map<int, std::pair<hipEvent_t, hipEvent_t>> side_events;
   std::map<int, void*> node_ptr[2];
   std::map<int, int64_t> statics;    // symbol -> current value
   struct Launch {
@@ -200,6 +210,11 @@ void destroy_routine(ocannl_hip_routine* rt) {
   (void)hipSetDevice(rt->dev->ordinal);
   (void)hipStreamSynchronize(rt->dev->stream);
   for (auto e : rt->timing_events) (void)hipEventDestroy(e);
+  for (auto& kv : rt->side_events) {
+    if (kv.second.first) (void)hipEventDestroy(kv.second.first);
+    if (kv.second.second) (void)hipEventDestroy(kv.second.second);
+  }
+  if (!rt->side_events.empty()) (void)hipStreamSynchronize(rt->dev->side_stream);
   for (auto e : rt->profile_events) (void)hipEventDestroy(e);
   if (rt->module) (void)hipModuleUnload(rt->module);
   if (rt->scratch) { (void)hipFree(rt->scratch); rt->dev->scratch_used -= rt->scratch_bytes; }
@@ -237,6 +252,10 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0) {
                       " but no transfer has filled it (device_to_device ~into_merge_buffer first)");
     merge_base = it->second.first;
   }
+  if (rt.code->plan.debug_log) {
+    static int g_run_id = 0;   // get_global_run_id
+    rt.log_id = ++g_run_id;
+  }
   const bool timed = kernel_ms != nullptr;
   if (timed) {
     if (cap < (int)rt.launches.size()) throw InvalidArgument("run_timed: kernel_ms too small");
@@ -247,9 +266,27 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0) {
     }
     hip_check(hipEventRecord(rt.timing_events[0], dev.stream), "hipEventRecord");
   }
+  // The side queue is used by plain runs over the routine's own arena; per-kernel timing and the
+  // static-scratch variant keep everything in order on the main queue.
+  const bool two_queues = v == 0 && !timed && !rt.side_events.empty();
+  int joined = -1, last_side = -1;   // latest side-queue phase the main queue has waited for / that was launched
   for (size_t li = 0; li < rt.launches.size(); ++li) {
     auto& l = rt.launches[li];
     const Phase& ph = rt.code->plan.phases[l.phase];
+    const bool on_side = two_queues && ph.stream == 1;
+    hipStream_t stream = on_side ? dev.side_stream : dev.stream;
+    if (on_side) {
+      auto& ev = rt.side_events.at((int)li);
+      hip_check(hipEventRecord(ev.first, dev.stream), "hipEventRecord");
+      hip_check(hipStreamWaitEvent(dev.side_stream, ev.first, 0), "hipStreamWaitEvent");
+    } else if (two_queues) {
+      int need = -1;
+      for (int p : ph.wait_for) need = std::max(need, p);
+      if (need > joined) {   // (the side queue runs in order: its latest phase stands for the earlier ones)
+        hip_check(hipStreamWaitEvent(dev.stream, rt.side_events.at(need).second, 0), "hipStreamWaitEvent");
+        joined = need;
+      }
+    }
     const bool bracket = v == 0 && !timed && li < rt.profile_mask.size() && rt.profile_mask[li];
     if (bracket) {
       while (rt.profile_events.size() < rt.profile_used + 2) {
@@ -257,7 +294,7 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0) {
         hip_check(hipEventCreate(&e), "hipEventCreate");
         rt.profile_events.push_back(e);
       }
-      hip_check(hipEventRecord(rt.profile_events[rt.profile_used], dev.stream), "hipEventRecord");
+      hip_check(hipEventRecord(rt.profile_events[rt.profile_used], stream), "hipEventRecord");
     }
     if (ph.kind == Phase::Fill) {
       if (v == 0) {
@@ -301,8 +338,12 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0) {
         a.c2_more[m] = g.group[m].c_copy >= 0 ? rt.node_ptr[v].at(g.group[m].c_copy) : nullptr;
       }
       // a bracketed contraction is timed without its split-K reduction (a kernel of its own)
-      hip_check(launch_gemm(g, a, rt.gemm_ws[v], dev.stream, bracket ? rt.profile_events[rt.profile_used + 1] : nullptr),
+      hip_check(launch_gemm(g, a, on_side ? rt.gemm_ws_side : rt.gemm_ws[v], stream, bracket ? rt.profile_events[rt.profile_used + 1] : nullptr),
                 "launch_gemm");
+      if (on_side) {
+        hip_check(hipEventRecord(rt.side_events.at((int)li).second, dev.side_stream), "hipEventRecord");
+        last_side = (int)li;
+      }
     }
     if (timed) hip_check(hipEventRecord(rt.timing_events[li + 1], dev.stream), "hipEventRecord");
     if (bracket) {
@@ -311,6 +352,8 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0) {
       rt.profile_used += 2;
     }
   }
+  // whatever follows on the main queue (the caller's copies, the next run) comes after the side queue's work
+  if (last_side > joined) hip_check(hipStreamWaitEvent(dev.stream, rt.side_events.at(last_side).second, 0), "hipStreamWaitEvent");
   if (timed) {
     hip_check(hipStreamSynchronize(dev.stream), "hipStreamSynchronize");
     for (size_t li = 0; li < rt.launches.size(); ++li)
@@ -361,6 +404,7 @@ int ocannl_hip_get_device(int ordinal, ocannl_hip_device** out) {
       if (std::string(d->props.gcnArchName).rfind("gfx950", 0) != 0)
         throw RuntimeError(std::string("hip backend: device is ") + d->props.gcnArchName + ", this library is built for gfx950 only");
       hip_check(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+      hip_check(hipStreamCreateWithFlags(&d->side_stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
       // this device's address of the library's static scratch array (the device is current here)
       hip_check(hipGetSymbolAddress(&d->static_scratch, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
       g_devices[ordinal] = std::move(d);
@@ -641,6 +685,7 @@ int ocannl_hip_code_kernel_info(ocannl_hip_code* code, int index, int kernel, oc
     info->coop_lanes = ph.coop_lanes;
     info->flops = ph.flops;
     info->bytes = ph.bytes;
+    info->queue = ph.stream;
     std::string name;
     if (ph.kind == Phase::Contraction) {
       // grouped contractions read as more batch entries, a chain of operand pairs as a longer K
@@ -703,11 +748,16 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
       local_off[n.id] = arena;
       arena += ((uint64_t)n.size_in_bytes() + 255) / 256 * 256;
     }
-    uint64_t ws_bytes = 0;
+    uint64_t ws_bytes = 0, ws_side_bytes = 0;
     for (auto& ph : cr.plan.phases)
-      if (ph.kind == Phase::Contraction) ws_bytes = std::max<uint64_t>(ws_bytes, gemm_workspace_bytes(ph.gemm));
+      if (ph.kind == Phase::Contraction) {
+        ws_bytes = std::max<uint64_t>(ws_bytes, gemm_workspace_bytes(ph.gemm));   // (any phase may run on the main queue)
+        if (ph.stream == 1) ws_side_bytes = std::max<uint64_t>(ws_side_bytes, gemm_workspace_bytes(ph.gemm));
+      }
     const uint64_t ws_off = arena;
     arena += (ws_bytes + 255) / 256 * 256;
+    const uint64_t ws_side_off = arena;
+    arena += (ws_side_bytes + 255) / 256 * 256;
     rt->scratch_bytes = arena;
     if (arena) {
       hip_check(hipMalloc(&rt->scratch, arena), "hipMalloc(scratch)");
@@ -722,6 +772,14 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
       rt->node_ptr[v] = ctx_ptr;
       for (auto& kv : local_off) rt->node_ptr[v][kv.first] = bases[v] + kv.second;
       rt->gemm_ws[v] = ws_bytes ? bases[v] + ws_off : nullptr;
+    }
+    rt->gemm_ws_side = ws_side_bytes ? bases[0] + ws_side_off : nullptr;
+    for (size_t pi = 0; pi < cr.plan.phases.size(); ++pi) {
+      if (cr.plan.phases[pi].stream != 1) continue;
+      std::pair<hipEvent_t, hipEvent_t> ev{nullptr, nullptr};
+      hip_check(hipEventCreateWithFlags(&ev.first, hipEventDisableTiming), "hipEventCreateWithFlags");
+      rt->side_events[(int)pi] = ev;   // (registered before the second is made, so that a failure releases the first)
+      hip_check(hipEventCreateWithFlags(&rt->side_events[(int)pi].second, hipEventDisableTiming), "hipEventCreateWithFlags");
     }
     for (auto& s : cr.r.statics) rt->statics[s.sym] = 0;
     if (!cr.binary.empty()) hip_check(hipModuleLoadData(&rt->module, cr.binary.data()), "hipModuleLoadData");
@@ -747,7 +805,10 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
         l.grid_y = (unsigned)((blocks + kRow - 1) / kRow);
         l.block = (unsigned)gk.block;
         size_t np = 0, ni = 0;
-        for (auto& p : gk.params) (p.kind != KernelParam::StaticIdx ? np : ni)++;
+        for (auto& p : gk.params) {
+          if (p.kind == KernelParam::StaticIdx) ++ni;
+          else if (p.kind != KernelParam::LogId) ++np;
+        }
         // (sized once: the argument arrays below point into these vectors)
         l.idx_vals.assign(ni, 0);
         for (auto& p : gk.params) if (p.kind == KernelParam::StaticIdx) l.idx_syms.push_back(p.id);
@@ -756,6 +817,7 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
           size_t ip = 0, ii = 0;
           for (auto& p : gk.params) {
             if (p.kind == KernelParam::StaticIdx) { l.args[v].push_back(&l.idx_vals[ii++]); continue; }
+            if (p.kind == KernelParam::LogId) { l.args[v].push_back(&rt->log_id); continue; }
             if (p.kind == KernelParam::NodePtr) l.ptr_vals[v][ip] = rt->node_ptr[v].at(p.id);
             else l.merge_slot = (int)ip;
             l.args[v].push_back(&l.ptr_vals[v][ip++]);
@@ -796,6 +858,13 @@ int ocannl_hip_routine_run_static_scratch(ocannl_hip_routine* rt) {
                       " bytes of the library's static scratch array: use ocannl_hip_routine_run");
     if (!rt->static_ok) throw RuntimeError("run_static_scratch: the device's static scratch array was not set up");
     enqueue(*rt, nullptr, 0, 1);
+  });
+}
+
+int ocannl_hip_routine_log_id(ocannl_hip_routine* rt, int* log_id) {
+  return guarded([&] {
+    if (!rt || !log_id) throw InvalidArgument("log_id: null argument");
+    *log_id = rt->log_id;
   });
 }
 

@@ -519,7 +519,8 @@ def fmt_g16(c: float) -> str:
     return "%.16g" % c
 
 
-def to_ll(r: Routine, with_prec: bool = False) -> str:
+def _ll_printers(with_prec: bool = False):
+    """(scalar printer, statement printer) of the ``.ll`` text form."""
     def ident(n: Node) -> str:
         return n.ident + (f"<{n.prec}>" if with_prec else "")
 
@@ -580,6 +581,18 @@ def to_ll(r: Routine, with_prec: bool = False) -> str:
         if isinstance(c, DeclareLocal):
             return f"declare {local(c.scope)};"
         raise TypeError(c)
+
+    return sc, st
+
+
+def ll_statement(c: "Stmt", with_prec: bool = False) -> str:
+    """One statement in the ``.ll`` text form: what the reference attaches to a ``Set`` as its
+    ``debug`` string (the text that in-routine logging prints after ``# ``)."""
+    return _ll_printers(with_prec)[1](c)
+
+
+def to_ll(r: Routine, with_prec: bool = False) -> str:
+    _, st = _ll_printers(with_prec)
 
     def static(s: StaticSymbol) -> str:
         if s.range is None:
@@ -642,6 +655,9 @@ def _wire_scalar(s: Scalar) -> str:
     raise TypeError(s)
 
 
+_WIRE_DEBUG = [False]   # to_wire(..., debug=True): every Set carries its `.ll` text
+
+
 def _wire_stmt(c: Stmt) -> str:
     if isinstance(c, Comment):
         return f"(comment {_q(c.text)})"
@@ -650,6 +666,8 @@ def _wire_stmt(c: Stmt) -> str:
     if isinstance(c, ZeroOut):
         return f"(zero_out {c.node.id})"
     if isinstance(c, Set):
+        if _WIRE_DEBUG[0]:
+            return f"(set {c.node.id} {_wire_idcs(c.idcs)} {_wire_scalar(c.value)} {_q(ll_statement(c))})"
         return f"(set {c.node.id} {_wire_idcs(c.idcs)} {_wire_scalar(c.value)})"
     if isinstance(c, SetFromVec):
         return (f"(set_vec {c.node.id} {_wire_idcs(c.idcs)} {c.length} {c.op} {c.arg_prec} "
@@ -666,8 +684,9 @@ def _wire_stmts(body: Sequence[Stmt]) -> str:
     return "(" + "\n".join(_wire_stmt(c) for c in body) + ")"
 
 
-def to_wire(r: Routine) -> str:
-    """Serialise a routine.  Grammar (S-expressions; atoms are integers, identifiers,
+def to_wire(r: Routine, debug: bool = False) -> str:
+    """Serialise a routine (``debug``: every ``set`` carries, as a last string, the statement's
+    ``.ll`` text -- the ``debug`` field of ``Low_level.Set`` that in-routine logging prints).  Grammar (S-expressions; atoms are integers, identifiers,
     C99 hex floats, or double-quoted strings)::
 
         (routine NAME
@@ -676,6 +695,11 @@ def to_wire(r: Routine) -> str:
           (nodes (ID IDENT PREC MODE ZERO_INIT READ_ONLY (DIM ...)) ...)
           (body STMT ...))
     """
+    _WIRE_DEBUG[0] = debug
+    try:
+        body_text = _wire_stmts(r.body)[1:-1]
+    finally:
+        _WIRE_DEBUG[0] = False
     statics = " ".join(f"({s.sym} {-1 if s.range is None else s.range})"
                        for s in r.static_indices)
     nodes = "\n".join(
@@ -684,4 +708,4 @@ def to_wire(r: Routine) -> str:
         for n in r.nodes())
     merge = -1 if r.merge_node is None else r.merge_node.id
     return (f"(routine {_q(r.name)}\n(static {statics})\n(merge {merge})\n(nodes\n{nodes})\n"
-            f"(body\n{_wire_stmts(r.body)[1:-1]}))\n")
+            f"(body\n{body_text}))\n")

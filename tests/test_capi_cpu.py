@@ -222,3 +222,37 @@ def test_compile_batch_holds_every_routine():
     assert len(code.kernels(0)) >= 1 and len(code.kernels(1)) >= 1
     assert "second_routine_k0" in code.source()
     assert lib.ocannl_hip_code_routine_name(code._h, 2, buf, 64) == -2
+
+
+def test_debug_log_source_follows_the_reference_line_format():
+    # c_syntax.ml:493-535: `# <statement>` then `lhs[%u]{=old} = new = <expression with {=value} after
+    # every read>`; comments as `COMMENT: text`; cuda_backend.ml:874-893: `<log id>: ` prefix, `$` for \n
+    a = L.Node(1, "a", "single", (4,)); b = L.Node(2, "b", "bfloat16", (4,)); c = L.Node(3, "c", "single", (4,))
+    L.reset_symbols(0)
+    i = L.fresh_symbol()
+    r = L.Routine("logged", [L.Comment("c fwd"), L.For(i, 0, 3, [L.Set(c, (L.It(i),), L.Ternop(
+        "fma", L.Get(a, (L.It(i),)), L.Get(b, (L.It(i),)), L.Const(0.5)))]), L.Comment("end")])
+    code = B.compile(r, "debug_log=1")
+    src = code.source()
+    assert 'printf("%d: COMMENT: c fwd$", log_id);' in src and 'printf("%d: COMMENT: end$", log_id);' in src
+    assert 'printf("%d: # c[i1] := fma(a[i1], b[i1], 0.5);$", log_id);' in src
+    assert ('printf("%d: c[%u]{=%g} = %g = fmaf(a[%u]{=%g}, bfloat16_to_single(b[%u]){=%g}, (float)(0.5))$", log_id, '
+            '(unsigned)(i1), (double)(c[i1]), (double)(new_set_v), (unsigned)(i1), (double)(a[i1]), (unsigned)(i1), '
+            '(double)(bfloat16_to_single(b[i1])));') in src
+    # one thread walks the loop in order; the kernel takes the log id; without the option nothing is printed
+    assert "for (uint32_t i1 = 0; i1 <= 3; ++i1)" in src and "const int log_id" in src
+    assert "printf" not in B.compile(r).source().split("extern \"C\"", 1)[1]
+
+
+def test_weight_gradients_go_to_the_side_queue_and_fused_prologues_show_up():
+    kw = dict(batch=32, seq=256, d_model=512, heads=8, d_ff=1024, layers=2, vocab=512, prec="bfloat16", grad_prec="single")
+    w = W.transformer(**kw)
+    ks = B.compile(w.routine).kernels()
+    side = [k for k in ks if k["queue"] == 1]
+    assert side and all(k["kind"] == "mfma" for k in side)
+    assert all(k["queue"] == 0 for k in B.compile(w.routine, "side_queue=0").kernels())
+    # Q K^T ahead of the soft-max chain runs inside the row-wise kernel (one launch less per block)
+    fused, apart = B.compile(w.routine), B.compile(w.routine, "fused=0")
+    assert "ocn_rowtile_contract<256, 64, 16, unsigned short>" in fused.source().split("extern \"C\"", 1)[1]
+    n = lambda c: sum(k["kind"] == "mfma" for k in c.kernels())
+    assert n(fused) == n(apart) - 2

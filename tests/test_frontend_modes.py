@@ -1,0 +1,80 @@
+"""Which tensors the harness (ocannl_amd/frontend.py) leaves materialised, against the one picture of
+that the reference holds: test/einsum/moons_demo_variant.expected:4-80 lists, for a one-hidden-layer MLP
+training step compiled as one routine (test/einsum/moons_demo_variant.ml:29-48), every tensor node with
+its final memory mode after the reference's optimiser.
+
+The harness inlines a tensor only when ONE statement reads it (once per cell).  The reference goes
+further (arrayjit/lib/low_level.ml:496-552): a read at the position being assigned does not count as a
+visit, so chains of pointwise operations -- and the gradients of pointwise operations -- are inlined
+into every reader and recomputed there.  The harness therefore materialises a SUPERSET of what the
+reference materialises: its routines move more bytes than real OCANNL's would, never fewer.  This test
+pins both halves: the nodes on which the two agree, and the exact list of nodes the harness keeps in
+memory although the reference virtualises them."""
+import numpy as np
+
+from ocannl_amd import llir as L
+from ocannl_amd.frontend import ConstT, Graph, make_routine
+from ocannl_amd.workloads import _SliceT
+
+# moons_demo_variant.expected:15-80 -- node -> mode ("On-dev" = context, "Local" = routine-local, "Virt")
+REFERENCE_MODES = {
+    "w2": "On-dev", "b1": "On-dev", "w1": "On-dev", "w2.grad": "Local", "b1.grad": "Local", "w1.grad": "Local",
+    "w1x": "Virt", "w1x.grad": "Local", "plus": "Virt", "plus.grad": "Virt", "relu": "Local", "relu.grad": "Virt",
+    "mlp": "Virt", "mlp.grad": "Local", "pointmul": "Virt", "pointmul.grad": "Virt", "minus": "Virt", "minus.grad": "Virt",
+    "margin_loss": "Virt", "margin_loss.grad": "Virt", "sum": "Local", "sum.grad": "Virt",
+    "scalar_loss": "On-dev", "scalar_loss.grad": "Virt", "learning_rate": "On-dev",
+    "sgd_delta_w2": "Virt", "sgd_delta_b1": "Virt", "sgd_delta_w1": "Virt",
+}
+# what the harness keeps in memory although the reference inlines it (see the module docstring)
+HARNESS_MATERIALISES_MORE = {"plus", "minus", "plus.grad", "relu.grad", "pointmul.grad", "minus.grad", "margin_loss.grad", "sum.grad",
+                             "scalar_loss.grad", "sgd_delta_w2", "sgd_delta_b1", "sgd_delta_w1"}
+# the one node the harness inlines although the reference keeps it: the batch sum feeds only the division
+HARNESS_MATERIALISES_LESS = {"sum"}
+
+
+def moons_variant():
+    L.reset_symbols(0)
+    g = Graph("single", "single")
+    nb, batch, hidden = 40, 10, 16
+    batch_n = L.StaticSymbol(L.fresh_symbol(), nb)
+    data = g.input("moons_flat", ("n", "b", "i"), (nb, batch, 2))
+    classes = g.input("moons_classes", ("n", "b", "o"), (nb, batch, 1))
+    w2 = g.param("w2", ("o", "h"), (1, hidden)); b1 = g.param("b1", ("h",), (hidden,)); w1 = g.param("w1", ("h", "i"), (hidden, 2))
+    lrate = g.input("learning_rate", ("one",), (1,))
+    xs = _SliceT(data.value, ("b", "i"), (batch, 2), lambda idx: L.Get(data.value, (L.It(batch_n.sym), idx["b"], idx["i"])))
+    ys = _SliceT(classes.value, ("b", "o"), (batch, 1), lambda idx: L.Get(classes.value, (L.It(batch_n.sym), idx["b"], idx["o"])))
+    h = g.unary("relu", g.add(b1, g.einsum(w1, xs, ("b", "h"), ident="w1x"), ("b", "h"), ident="plus"))
+    f = g.einsum(w2, h, ("b", "o"), ident="mlp")
+    margin = g.unary("relu", g.sub(ConstT(1.0), g.mul(ys, f, ("b", "o"), ident="pointmul"), ("b", "o"), ident="minus"), ident="margin_loss")
+    total = g.reduce(margin, ("l",), ident="sum")
+    loss = g.div(total, ConstT(10.0), ("l",), ident="scalar_loss")
+    body = g.grad_update(loss) + g.sgd_update([w2, b1, w1], lrate, momentum=0.0, weight_decay=1e-4)
+    return make_routine(g, "moons_variant", body, [batch_n], inline=True, outputs=[loss.value])
+
+
+def test_harness_memory_modes_against_the_reference_golden():
+    r = moons_variant()
+    mine = {}
+    seen = set()
+    for n in r.nodes():
+        label = n.ident.rsplit("_", 1)[0]
+        label = label[:-5] + ".grad" if label.endswith("_grad") else label
+        mine[label] = {"ctx": "On-dev", "local": "Local", "virtual": "Virt"}[n.mode]
+        seen.add(label)
+    # nodes that no longer appear in the routine at all were inlined away
+    for label in REFERENCE_MODES:
+        mine.setdefault(label, "Virt")
+    assert set(REFERENCE_MODES) <= set(mine), set(REFERENCE_MODES) - set(mine)
+    agree = {k for k in REFERENCE_MODES if (mine[k] == "Virt") == (REFERENCE_MODES[k] == "Virt")}
+    more = {k for k in REFERENCE_MODES if mine[k] != "Virt" and REFERENCE_MODES[k] == "Virt"}
+    less = {k for k in REFERENCE_MODES if mine[k] == "Virt" and REFERENCE_MODES[k] != "Virt"}
+    assert more == HARNESS_MATERIALISES_MORE, (more ^ HARNESS_MATERIALISES_MORE)
+    assert less == HARNESS_MATERIALISES_LESS, (less ^ HARNESS_MATERIALISES_LESS)
+    # parameters, their gradients, the activations that the matrix products re-read, the loss, the rate
+    for k in ("w1", "w2", "b1", "w1.grad", "w2.grad", "b1.grad", "relu", "w1x", "mlp", "w1x.grad", "mlp.grad", "scalar_loss",
+              "learning_rate", "pointmul", "margin_loss"):
+        assert k in agree, k
+    # On-dev exactly where the reference has it
+    for k, v in REFERENCE_MODES.items():
+        if v == "On-dev":
+            assert mine[k] == "On-dev", k

@@ -5,6 +5,7 @@ import pytest
 # brings up the system's: imported here (at collection), not inside the one test that uses it.
 import torch
 
+from ocannl_amd import backend as B
 from ocannl_amd import workloads as W
 from parity import HipRun, OracleRun, rel_err
 
@@ -277,3 +278,24 @@ def test_small_transformer_loss_curve_100_steps():
     assert lo[-1] < lo[0] - 0.2
     assert np.max(np.abs(np.array(lh) - np.array(lo))) <= 1e-3, float(np.max(np.abs(np.array(lh) - np.array(lo))))
     hip.close()
+
+
+@pytest.mark.parametrize("shape", [dict(b=2, h=4, q=64, k=128, d=32), dict(b=3, h=2, q=96, k=256, d=64), dict(b=2, h=2, q=32, k=512, d=16)])
+def test_contraction_as_row_group_prologue_equals_the_separate_launches(shape):
+    # Q K^T ahead of the soft-max chain and dOut V^T ahead of its backward chain run inside the row-wise
+    # kernels (32 rows at a time on the matrix cores, into LDS) instead of as launches of their own that
+    # write the scores to memory; `fused=0` keeps them apart.  Same products, same roundings, same
+    # summation order inside a row: every tensor of the routine has to come out bit for bit the same.
+    w = W.attention(prec="bfloat16", grad_prec="single", **shape)
+    # (by default only a product that is planner scratch is taken in; `fused=2` also takes dOut V^T, whose
+    # result is a context node and is stored by the kernel as well)
+    fused, apart = HipRun(w.routine, w.init, "min_mfma_flops=1;fused=2"), HipRun(w.routine, w.init, "min_mfma_flops=1;fused=0")
+    nf = sum(k["kind"] == "mfma" for k in fused.code.kernels()); na = sum(k["kind"] == "mfma" for k in apart.code.kernels())
+    assert nf == na - 2, (nf, na)   # the two contractions that feed row groups are gone
+    nd = sum(k["kind"] == "mfma" for k in B.compile(w.routine, "min_mfma_flops=1").kernels())
+    assert nd == na - 1, (nd, na)
+    assert "ocn_rowtile_contract<" in fused.code.source().split("extern \"C\"", 1)[1]
+    fused.step(); apart.step()
+    for n in w.routine.param_nodes():
+        assert np.array_equal(fused.get(n), apart.get(n)), n.ident
+    fused.close(); apart.close()
