@@ -120,10 +120,13 @@ int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** code);
    of tiny phases as one single-workgroup kernel), groups=0|1 (independent contractions of identical
    shapes share a launch), chains=0|1 (`c =+ a * b` statements into one result with identical operand
    shapes share a launch), parallel=0|1 (consecutive small phases that do not depend on one another
-   run side by side in one launch), debug_log=0|1 (in-routine logging, see
+   run side by side in one launch), graphs=0|1 (a routine's
+   kernels are captured into a HIP graph per combination of static-index values and replayed as one unit
+   by ocannl_hip_routine_run; off by default), debug_log=0|1 (in-routine logging, see
    ocannl_hip_routine_log_id; the wire form then carries every Set's text), side_queue=0|1 (contractions
    whose results nothing needs for a while -- weight gradients -- run on a second queue of the device, beside
-   the kernels that follow), fused=0|1|2 (a short-K contraction whose only reader is the row-wise
+   the kernels that follow), epilogues=0|1 (`y := x + bias` and `z := relu(y)` right behind the
+   contraction that produces x run in that contraction's epilogue), fused=0|1|2 (a short-K contraction whose only reader is the row-wise
    kernel that follows -- attention scores ahead of the soft-max chain -- runs on the matrix cores as that
    kernel's prologue, into LDS, instead of as a launch of its own; 2: also when its result is a context
    node that has to be stored anyway), min_mfma_flops=<n>, large_models=0|1 (64-bit loop

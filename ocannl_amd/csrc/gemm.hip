@@ -247,9 +247,13 @@ __device__ __forceinline__ bf16x8 tr_fragment(const unsigned short* at_lane, int
 // kOutF32Copy: fp32 result plus its bf16 rounding at the same element offset of a second tensor.
 enum : int { kOutF32 = 0, kOutBf16 = 1, kOutF32Copy = 2 };
 
+// bf16 bits <-> float, as the generated code converts them
+__device__ __forceinline__ float bf2f(unsigned b) { return __uint_as_float(b << 16); }
+
 template <int TN, int OUT, bool ACC, bool CHECK>
 __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, long ld, int lane,
-                                               long rows_left, long cols_left, void* origin2 = nullptr) {
+                                               long rows_left, long cols_left, void* origin2 = nullptr,
+                                               const unsigned short* bias = nullptr, unsigned short* relu_out = nullptr) {
   using T = typename std::conditional<OUT == kOutBf16, unsigned short, float>::type;
   T* const base = static_cast<T*>(origin);
   unsigned short* const base2 = static_cast<unsigned short*>(origin2);
@@ -283,7 +287,12 @@ __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, 
       float v = acc[j][e];
       if (ACC) v += old[ACC ? j : 0][e];
       if (!CHECK || ((long)(r + rb) < rows_left && (long)(j * 32 + col) < cols_left)) {
-        if (OUT == kOutBf16) p[loff] = (unsigned short)f2bf(v);
+        if (OUT == kOutBf16) {
+          unsigned b = f2bf(v);
+          if (!ACC && bias) b = f2bf(bf2f(b) + bf2f(bias[j * 32 + col]));   // (bias: at the tile row's first column)
+          p[loff] = (unsigned short)b;
+          if (!ACC && relu_out) (relu_out + (long)r * ld + j * 32)[loff] = (unsigned short)(((b & 0x8000u) || (b & 0x7FFFu) > 0x7F80u) ? 0u : b);   // fmaxf(0, y): negatives and NaN give +0
+        }
         else p[loff] = v;
         if (OUT == kOutF32Copy) (base2 + (long)r * ld + j * 32)[loff] = (unsigned short)f2bf(v);
       }
@@ -300,7 +309,8 @@ __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, 
 // floats of this wave's own; LDS operations of one wave complete in order, so no barrier is needed.
 template <int TN, int OUT, bool ACC>
 __device__ __forceinline__ void store_tile_row_wide(f32x16 (&acc)[TN], float* stage, void* origin, long ld, int lane,
-                                                    void* origin2 = nullptr) {
+                                                    void* origin2 = nullptr, const unsigned short* bias = nullptr,
+                                                    unsigned short* relu_out = nullptr) {
   constexpr int CW = TN * 32, LS = CW + 4;
   static_assert(TN == 2 || TN == 4, "tile rows of 2 or 4 tiles");
   asm volatile("" : "+a"(acc[0]), "+a"(acc[1]));
@@ -329,7 +339,25 @@ __device__ __forceinline__ void store_tile_row_wide(f32x16 (&acc)[TN], float* st
         v0 += f32x4{__uint_as_float(o.x << 16), __uint_as_float(o.x & 0xFFFF0000u), __uint_as_float(o.y << 16), __uint_as_float(o.y & 0xFFFF0000u)};
         v1 += f32x4{__uint_as_float(o.z << 16), __uint_as_float(o.z & 0xFFFF0000u), __uint_as_float(o.w << 16), __uint_as_float(o.w & 0xFFFF0000u)};
       }
-      *dst = u32x4{pack2(v0.x, v0.y), pack2(v0.z, v0.w), pack2(v1.x, v1.y), pack2(v1.z, v1.w)};
+      u32x4 out = u32x4{pack2(v0.x, v0.y), pack2(v0.z, v0.w), pack2(v1.x, v1.y), pack2(v1.z, v1.w)};
+      if (!ACC && bias) {
+        // x rounded to bf16 (above), then y = bf16(x + bias[n]): eight columns per lane
+        const u32x4 bb = *reinterpret_cast<const u32x4*>(bias + cc);
+        auto add2 = [](unsigned x, unsigned b) { return pack2(__uint_as_float(x << 16) + __uint_as_float(b << 16),
+                                                               __uint_as_float(x & 0xFFFF0000u) + __uint_as_float(b & 0xFFFF0000u)); };
+        out = u32x4{add2(out.x, bb.x), add2(out.y, bb.y), add2(out.z, bb.z), add2(out.w, bb.w)};
+      }
+      *dst = out;
+      if (!ACC && relu_out) {
+        // relu on bf16 bits, as fmaxf(0, y) gives it: negatives (and NaN) become +0
+        auto relu2 = [](unsigned x) {
+          const unsigned lo = x & 0xFFFFu, hi = x >> 16;
+          const unsigned rl = ((lo & 0x8000u) || (lo & 0x7FFFu) > 0x7F80u) ? 0u : lo;
+          const unsigned rh = ((hi & 0x8000u) || (hi & 0x7FFFu) > 0x7F80u) ? 0u : hi;
+          return rl | (rh << 16);
+        };
+        *reinterpret_cast<u32x4*>(relu_out + row_off + goff) = u32x4{relu2(out.x), relu2(out.y), relu2(out.z), relu2(out.w)};
+      }
     } else {
       f32x4* const dst = reinterpret_cast<f32x4*>(static_cast<float*>(origin) + row_off + goff);
       if (ACC) v0 += *dst;
@@ -364,23 +392,30 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, void* c
   // 16-byte stores need rows that start on 16-byte boundaries (and 8-byte ones for the bf16 copy)
   const bool wide = full && ((reinterpret_cast<unsigned long>(origin) | (unsigned long)(ld * (bf ? 2 : 4))) & 15) == 0 &&
                     (!copy || ((reinterpret_cast<unsigned long>(origin2) | (unsigned long)(ld * 2)) & 7) == 0) &&
+                    (!g.relu_out || ((reinterpret_cast<unsigned long>(g.relu_out) + (unsigned long)first * 2) & 15) == 0) &&
+                    (!g.bias || ((reinterpret_cast<unsigned long>(g.bias) + (unsigned long)n * 2) & 15) == 0) &&
                     (unsigned long)ld * 32 < 0x100000000ul;
   // fp32 results already leave as 128-byte row pieces per half-wave and go out directly (measured:
   // staging them gains nothing, the burst of a tile's results is bound by the memory system); bf16
   // results and bf16 copies would leave as 2-byte elements and take the staged form
   const int variant = (copy ? 8 : bf ? 4 : 0) + ((!to_ws && g.accumulate) ? 2 : 0) + ((copy || bf) ? (wide ? 0 : 1) : (full ? 0 : 1));
+  // folded consumers (bf16 results, stored, not accumulated): bias at this block's first column, relu output at its origin
+  const bool epi = bf && !g.accumulate;
+  const unsigned short* const bias = epi && g.bias ? static_cast<const unsigned short*>(g.bias) + n : nullptr;
+  char* const origin3 = epi && g.relu_out ? static_cast<char*>(g.relu_out) + first * 2 : nullptr;
   static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
     constexpr int i = decltype(ic)::value;
     void* o = origin + (long)i * 32 * ld * (bf ? 2 : 4);
     void* o2 = origin2 + (long)i * 32 * ld * 2;
+    void* o3 = origin3 ? origin3 + (long)i * 32 * ld * 2 : nullptr;
     const long rl = rows_left - i * 32;
     switch (variant) {
       case 0: store_tile_row<TN, kOutF32, false, false>(acc[i], o, ld, lane, rl, cols_left); break;
       case 1: store_tile_row<TN, kOutF32, false, true>(acc[i], o, ld, lane, rl, cols_left); break;
       case 2: store_tile_row<TN, kOutF32, true, false>(acc[i], o, ld, lane, rl, cols_left); break;
       case 3: store_tile_row<TN, kOutF32, true, true>(acc[i], o, ld, lane, rl, cols_left); break;
-      case 4: store_tile_row_wide<TN, kOutBf16, false>(acc[i], stage, o, ld, lane); break;
-      case 5: store_tile_row<TN, kOutBf16, false, true>(acc[i], o, ld, lane, rl, cols_left); break;
+      case 4: store_tile_row_wide<TN, kOutBf16, false>(acc[i], stage, o, ld, lane, nullptr, bias, reinterpret_cast<unsigned short*>(o3)); break;
+      case 5: store_tile_row<TN, kOutBf16, false, true>(acc[i], o, ld, lane, rl, cols_left, nullptr, bias, reinterpret_cast<unsigned short*>(o3)); break;
       case 6: store_tile_row_wide<TN, kOutBf16, true>(acc[i], stage, o, ld, lane); break;
       case 7: store_tile_row<TN, kOutBf16, true, true>(acc[i], o, ld, lane, rl, cols_left); break;
       case 8: store_tile_row_wide<TN, kOutF32Copy, false>(acc[i], stage, o, ld, lane, o2); break;
@@ -828,7 +863,7 @@ TileConfig tile_config(const GemmDesc& d) {
     // bf16 sources: towards one workgroup per CU, which then loads two stages ahead (below);
     // otherwise towards two per CU
     const long target = bf16_sources ? 256 : 512;
-    if (t128 < 256) {
+    if (t128 < 256 && d.epi_bias < 0 && d.epi_relu < 0) {   // (folded consumers are applied by the contraction's own epilogue)
       while (s * 2 * t128 <= target && s * 2 <= d.K / 512 && s < 64) s *= 2;
     }
     c.splits = (int)s;

@@ -37,6 +37,11 @@ struct GemmArgs {
   // offsets (C must be fp32).  It feeds later bf16 contractions that read C.
   void* c2;
   void* c2_more[3];
+  // Epilogue fusion (bf16 C, no accumulation, no K split): when `bias` is not null the stored value is
+  // bf16(bf16(acc) + bias[n]) (bias: bf16, indexed by the column); when `relu_out` is not null, relu of
+  // the stored value also goes to that tensor at the same element offsets.
+  const void* bias;
+  void* relu_out;
 };
 
 // Picks the kernel instance for the operand precisions / layouts and launches it on `stream`.

@@ -502,7 +502,7 @@ bool phase_touches(const Phase& ph, int node) {
   if (ph.kind == Phase::Fill) return ph.fill_node == node;
   if (ph.kind == Phase::Contraction) {
     for (auto& m : ph.gemm.group) if (m.a.node == node || m.b.node == node || m.c.node == node || m.c_copy == node) return true;
-    if (ph.gemm.c_copy == node) return true;
+    if (ph.gemm.c_copy == node || ph.gemm.epi_bias == node || ph.gemm.epi_relu == node) return true;
     for (auto& pr : ph.gemm.more) if (pr.first.node == node || pr.second.node == node) return true;
     return ph.gemm.a.node == node || ph.gemm.b.node == node || ph.gemm.c.node == node;
   }
@@ -1200,7 +1200,8 @@ void merge_contractions(Plan& plan, bool chain, int window = 1 << 30) {
       if (!chain && (long)j - (long)i > (long)window) break;
       Phase& q = plan.phases[j];
       const GemmDesc& h = q.gemm;
-      bool candidate = q.kind == Phase::Contraction && h.group.empty() && h.more.empty() && h.M == g.M && h.N == g.N &&
+      bool candidate = q.kind == Phase::Contraction && h.group.empty() && h.more.empty() && h.epi_bias < 0 && h.epi_relu < 0 &&
+                       g.epi_bias < 0 && g.epi_relu < 0 && h.M == g.M && h.N == g.N &&
                        h.K == g.K && h.nbatch == g.nbatch && same_layout(h.a, g.a) && same_layout(h.b, g.b) && same_layout(h.c, g.c);
       for (int b = 0; b < g.nbatch && candidate; ++b) candidate = h.batch_ext[b] == g.batch_ext[b];
       const std::vector<Member> mine = members_of(g);
@@ -1470,7 +1471,7 @@ bool phase_writes(const Phase& ph, int node) {
   if (ph.kind == Phase::Fill) return ph.fill_node == node;
   if (ph.kind == Phase::Contraction) {
     for (auto& m : ph.gemm.group) if (m.c.node == node || m.c_copy == node) return true;
-    return ph.gemm.c.node == node || ph.gemm.c_copy == node;
+    return ph.gemm.c.node == node || ph.gemm.c_copy == node || ph.gemm.epi_relu == node;
   }
   auto writes = [&](const Phase& q) {
     std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
@@ -1845,6 +1846,8 @@ void assign_side_queue(Plan& plan) {
     const GemmDesc& g = ph.gemm;
     s.outs = {g.c.node}; s.ins = {g.a.node, g.b.node};
     if (g.c_copy >= 0) s.outs.push_back(g.c_copy);
+    if (g.epi_relu >= 0) s.outs.push_back(g.epi_relu);
+    if (g.epi_bias >= 0) s.ins.push_back(g.epi_bias);
     for (auto& m : g.group) { s.outs.push_back(m.c.node); if (m.c_copy >= 0) s.outs.push_back(m.c_copy); s.ins.push_back(m.a.node); s.ins.push_back(m.b.node); }
     for (auto& pr : g.more) { s.ins.push_back(pr.first.node); s.ins.push_back(pr.second.node); }
     for (int o : std::vector<int>(s.outs)) { auto m = plan.mirrors.find(o); if (m != plan.mirrors.end()) s.outs.push_back(m->second); }
@@ -1876,6 +1879,75 @@ void assign_side_queue(Plan& plan) {
 
 }  // namespace
 
+// ---- pointwise consumers folded into a contraction's epilogue ----------------------------------------
+// `y[..] := x + bias[n]` (either order) right after the contraction that produces the inlined product
+// x, optionally followed by `z[..] := relu(y[..])`: an mlp layer (lib/nn_blocks.ml:108-135).  The
+// contraction then stores y (and z) itself; x, which was planner scratch, is never written.
+namespace {
+
+void fold_epilogues(Routine& r, Plan& plan) {
+  std::set<int> scratch;
+  for (auto& n : plan.scratch) scratch.insert(n.id);
+  auto identity_set = [&](const Phase& q, int64_t rank) -> const Stmt* {   // Set through plain full-range iterators, no loops left inside a thread
+    if (q.kind != Phase::Generic || !q.members.empty() || !q.seq_syms.empty() || q.coop_lanes != 1) return nullptr;
+    if (q.inner.size() != 1 || q.inner[0]->kind != Stmt::Set) return nullptr;
+    const Stmt& st = *q.inner[0];
+    if ((int64_t)st.idcs.size() != rank || !writes_whole_node(r, q, st.node)) return nullptr;
+    for (auto& ix : st.idcs) if (ix.kind != AxisIndex::Iter) return nullptr;
+    return &st;
+  };
+  for (size_t i = 0; i + 1 < plan.phases.size(); ++i) {
+    Phase& P = plan.phases[i];
+    GemmDesc& g = P.gemm;
+    if (P.kind != Phase::Contraction || !scratch.count(g.c.node) || g.accumulate || g.c_copy >= 0 || !g.group.empty() || !g.more.empty()) continue;
+    const int X = g.c.node;
+    const Node xn = r.node(X);
+    if (xn.prec != Prec::Bfloat16 || g.c.offset != 0 || !g.c.static_terms.empty()) continue;
+    int64_t written = g.M * g.N;
+    for (int b = 0; b < g.nbatch; ++b) written *= g.batch_ext[b];
+    if (written != xn.num_elems() || g.N != xn.dims.back()) continue;
+    const Stmt* ys = identity_set(plan.phases[i + 1], (int64_t)xn.dims.size());
+    if (!ys) continue;
+    const Node& yn = r.node(ys->node);
+    const Scalar& v = *ys->value;
+    if (yn.prec != Prec::Bfloat16 || yn.dims != xn.dims || !(v.kind == Scalar::Bin && v.bin == Binop::Add)) continue;
+    const Scalar* xg = nullptr; const Scalar* bg = nullptr;
+    for (const Scalar* s : {v.a.get(), v.b.get()}) {
+      if (s->kind == Scalar::Get && s->node == X && s->idcs == ys->idcs) xg = s;
+      else if (s->kind == Scalar::Get && s->idcs.size() == 1 && s->idcs[0] == ys->idcs.back()) bg = s;
+    }
+    if (!xg || !bg) continue;
+    const Node& bn = r.node(bg->node);
+    if (bn.prec != Prec::Bfloat16 || bn.dims.size() != 1 || bn.dims[0] != g.N || bn.mode == Mode::Virtual) continue;
+    // an optional relu of y right behind
+    int Z = -1;
+    if (i + 2 < plan.phases.size()) {
+      const Stmt* zs = identity_set(plan.phases[i + 2], (int64_t)xn.dims.size());
+      if (zs && zs->node != ys->node) {
+        const Node& zn = r.node(zs->node);
+        const Scalar& zv = *zs->value;
+        if (zn.prec == Prec::Bfloat16 && zn.dims == xn.dims && zv.kind == Scalar::Un && zv.un == Unop::Relu && zv.a->kind == Scalar::Get &&
+            zv.a->node == ys->node && zv.a->idcs == zs->idcs)
+          Z = zs->node;
+      }
+    }
+    // x must have no other reader
+    bool alone = true;
+    for (size_t q = 0; q < plan.phases.size(); ++q) if (q != i && q != i + 1 && phase_touches(plan.phases[q], X)) alone = false;
+    if (!alone) continue;
+    const double tensor_bytes = (double)xn.size_in_bytes();
+    g.c.node = ys->node;
+    g.epi_bias = bg->node;
+    g.epi_relu = Z;
+    P.bytes += (double)bn.size_in_bytes() + (Z >= 0 ? tensor_bytes : 0.0);
+    P.label += " + bias" + std::string(Z >= 0 ? " + relu" : "");
+    r.nodes.at(X).mode = Mode::Virtual;   // never stored
+    plan.phases.erase(plan.phases.begin() + i + 1, plan.phases.begin() + i + (Z >= 0 ? 3 : 2));
+  }
+}
+
+}  // namespace
+
 Plan make_plan(Routine& r, const PlanOptions& requested) {
   PlanOptions opt = requested;
   if (r.merge_node >= 0) {
@@ -1885,11 +1957,12 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
   }
   if (opt.debug_log) {
     opt.enable_mfma = opt.enable_coop = opt.enable_row_groups = opt.enable_serial_group = opt.enable_parallel_groups = false;
-    opt.enable_bf16_copies = opt.fuse_row_contractions = opt.side_queue = false;
+    opt.enable_bf16_copies = opt.fuse_row_contractions = opt.side_queue = opt.fuse_epilogues = false;
   }
   struct SeqGuard { bool old; SeqGuard(bool v) : old(g_all_sequential) { g_all_sequential = v; } ~SeqGuard() { g_all_sequential = old; } } seq_guard(opt.debug_log);
   Plan plan;
   plan.debug_log = opt.debug_log;
+  plan.use_graphs = opt.use_graphs;
   plan.large_index = opt.large_models;
   for (auto& kv : r.nodes) if (kv.second.num_elems() > (int64_t)0x7FFFFFFF) plan.large_index = true;
   std::string label;
@@ -1986,6 +2059,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     plan.phases.push_back(std::move(ph));
   }
   plan.trailing_comments.swap(pending_comments);
+  if (opt.enable_mfma && opt.fuse_epilogues) fold_epilogues(r, plan);
   if (opt.enable_mfma && opt.merge_chains) merge_contractions(plan, true);
   if (opt.enable_mfma && opt.group_contractions) merge_contractions(plan, false, opt.group_window);
   if (opt.enable_coop && opt.enable_row_groups) group_rows(r, plan);

@@ -49,6 +49,13 @@ struct GemmDesc {
   // >= 0: a bf16 scratch tensor of C's shape that the epilogue fills with the rounded result (C is
   // fp32 and written whole): it feeds later bf16 contractions that read C, in place of a conversion pass
   int c_copy = -1;
+  // Pointwise consumers folded into the epilogue (bf16 results only; never with a K split, a group or a
+  // chain).  The optimiser inlines the product `x = a * b` into `y := x + bias[n]` (either order) and
+  // `z := relu(y)` reads y (lib/nn_blocks.ml:108-135, an mlp layer): the kernel then rounds x as the
+  // inlined scalar would be, adds the bias, rounds again and stores that as C (= y), and stores relu of
+  // it to `epi_relu`.  -1: absent.
+  int epi_bias = -1;     // vector indexed by n, bf16
+  int epi_relu = -1;     // tensor of C's shape and precision that receives relu(C)
   double flops() const {
     double f = 2.0 * (double)M * (double)N * (double)K * (double)(1 + group.size()) * (double)(1 + more.size());
     for (int i = 0; i < nbatch; ++i) f *= (double)batch_ext[i];
@@ -139,8 +146,14 @@ struct PlanOptions {
   // every top-level statement becomes a kernel of ONE thread that walks its loops in order, and none
   // of the fusing rewrites applies.
   bool debug_log = false;
+  // plain runs replay a captured HIP graph of the routine's kernels.  Off by default: measured on
+  // MI355X / ROCm 7.2 it pays only for a routine of about ten tiny kernels (half-moons step as ten
+  // launches: 40 -> 26 us); nine kernels of the char-MLP step went 36 -> 42 us and the 127 kernels of
+  // the transformer step 3.68 -> 3.73 ms.
+  bool use_graphs = false;
   int group_window = 1 << 30;        // contractions share a launch only when at most this many phases apart
   bool side_queue = true;            // contractions off the critical path run on a second queue beside the rest
+  bool fuse_epilogues = true;        // bias / relu consumers of an inlined contraction run in the contraction's epilogue
   bool fuse_row_contractions = true; // a short-K contraction feeding a row group runs as that kernel's prologue ...
   bool fuse_stored_rows = false;     // ... also when its result has to be stored anyway (a context node): measured slower
   bool enable_bf16_copies = true;   // keep bf16 copies of fp32 operands of mixed contractions (written by the producing kernels)
@@ -153,6 +166,7 @@ struct Plan {
   // the node also stores the rounded value to the copy): the copy feeds bf16 contractions
   std::map<int, int> mirrors;
   bool large_index = false;    // generated kernels compute offsets in 64 bits
+  bool use_graphs = false;     // plain runs are replayed from a captured HIP graph
   bool debug_log = false;      // generated kernels print what they compute (and take an `int log_id` argument)
   std::vector<std::string> trailing_comments;   // debug logging: comments after the last phase
 };

@@ -132,7 +132,9 @@ PlanOptions parse_options(const char* options) {
     else if (k == "chains") o.merge_chains = v != "0";
     else if (k == "side_queue") o.side_queue = v != "0";
     else if (k == "debug_log") o.debug_log = v != "0";
+    else if (k == "graphs") o.use_graphs = v != "0";
     else if (k == "group_window") o.group_window = std::stoi(v);
+    else if (k == "epilogues") o.fuse_epilogues = v != "0";
     else if (k == "fused") { o.fuse_row_contractions = v != "0"; o.fuse_stored_rows = v == "2"; }
     else if (k == "parallel") o.enable_parallel_groups = v != "0";
     else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
@@ -157,6 +159,11 @@ struct ocannl_hip_routine {
   void* scratch = nullptr;           // the routine's own arena: local nodes, planner scratch, split-K workspace
   uint64_t scratch_bytes = 0;
   bool counted = false;              // included in the device's live_routines
+  // Replay: the kernel list of a plain run, captured once per combination of static-index values into
+  // a HIP graph (fills recorded as kernels, the side queue as a branch) and launched as one unit from
+  // then on: a routine of many short kernels stops paying a host call and a queue round trip per kernel.
+  std::map<std::vector<int64_t>, hipGraphExec_t> graphs;
+  bool warmed = false;               // one direct run first (it configures kernel attributes)
   int log_id = 0;                    // debug logging: prefix of this run's log lines (cuda_backend.ml:992-993)
   // Everything that names arena memory exists twice: [0] bound to the routine's own arena, [1] bound to
   // the library's static scratch array (valid when static_ok).
@@ -215,6 +222,7 @@ void destroy_routine(ocannl_hip_routine* rt) {
     if (kv.second.second) (void)hipEventDestroy(kv.second.second);
   }
   if (!rt->side_events.empty()) (void)hipStreamSynchronize(rt->dev->side_stream);
+  for (auto& kv : rt->graphs) (void)hipGraphExecDestroy(kv.second);
   for (auto e : rt->profile_events) (void)hipEventDestroy(e);
   if (rt->module) (void)hipModuleUnload(rt->module);
   if (rt->scratch) { (void)hipFree(rt->scratch); rt->dev->scratch_used -= rt->scratch_bytes; }
@@ -224,7 +232,7 @@ void destroy_routine(ocannl_hip_routine* rt) {
 
 // `v` = 0: the routine's own arena; 1: the library's static scratch array, with fills as kernels
 // and no call that allocates (no events: kernel_ms must be null and bracketing is off).
-void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0) {
+void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0, bool capturing = false) {
   ocannl_hip_device& dev = *rt.dev;
   dev.make_current();
   const Routine& r = rt.code->r;
@@ -297,13 +305,13 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0) {
       hip_check(hipEventRecord(rt.profile_events[rt.profile_used], stream), "hipEventRecord");
     }
     if (ph.kind == Phase::Fill) {
-      if (v == 0) {
+      if (v == 0 && !capturing) {
         hip_check(hipMemsetAsync(l.fill_ptr[0], 0, l.fill_bytes, dev.stream), "hipMemsetAsync");
       } else {
         // local nodes sit at 256-byte offsets and are padded to 256 bytes: whole 16-byte stores
         const uint64_t n16 = (l.fill_bytes + 15) / 16;
         hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, dev.stream,
-                           static_cast<uint4*>(l.fill_ptr[1]), n16);
+                           static_cast<uint4*>(l.fill_ptr[v]), n16);
         hip_check(hipGetLastError(), "fill_zero_kernel");
       }
     } else if (ph.kind == Phase::Generic) {
@@ -330,6 +338,8 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0) {
       a.accumulate = g.accumulate ? 1 : 0;
       a.c_is_bf16 = g.c.prec == Prec::Bfloat16;
       a.c2 = g.c_copy >= 0 ? rt.node_ptr[v].at(g.c_copy) : nullptr;
+      a.bias = g.epi_bias >= 0 ? rt.node_ptr[v].at(g.epi_bias) : nullptr;
+      a.relu_out = g.epi_relu >= 0 ? rt.node_ptr[v].at(g.epi_relu) : nullptr;
       a.npairs = 1 + (int)g.more.size();
       for (size_t p = 0; p < g.more.size(); ++p) { a.a_more[p] = base(g.more[p].first); a.b_more[p] = base(g.more[p].second); }
       a.ngroups = 1 + (int)g.group.size();
@@ -842,10 +852,48 @@ int ocannl_hip_routine_set_static(ocannl_hip_routine* rt, int symbol, int64_t va
   });
 }
 
+// A plain run, replayed from a captured graph when it can be: several kernels, no merge buffer (bound
+// at launch), no event bracketing, no device printing, and a graph for this combination of static indices
+// (at most kMaxGraphs of them are kept; beyond that, and on the very first run, the kernels are
+// launched one by one).
+static void run_plain(ocannl_hip_routine& rt) {
+  constexpr size_t kMaxGraphs = 128;
+  const auto& plan = rt.code->plan;
+  bool bracketing = false;
+  for (char m : rt.profile_mask) bracketing = bracketing || m;
+  const bool graphable = plan.use_graphs && rt.launches.size() >= 2 && rt.code->r.merge_node < 0 && !bracketing && !plan.debug_log;
+  if (!graphable || !rt.warmed) { enqueue(rt, nullptr, 0); rt.warmed = true; return; }
+  std::vector<int64_t> key;
+  for (auto& s : rt.code->r.statics) key.push_back(rt.statics[s.sym]);
+  auto it = rt.graphs.find(key);
+  ocannl_hip_device& dev = *rt.dev;
+  if (it == rt.graphs.end()) {
+    if (rt.graphs.size() >= kMaxGraphs) { enqueue(rt, nullptr, 0); return; }
+    dev.make_current();
+    hip_check(hipStreamBeginCapture(dev.stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+    hipGraph_t graph = nullptr;
+    try {
+      enqueue(rt, nullptr, 0, 0, true);
+    } catch (...) {
+      (void)hipStreamEndCapture(dev.stream, &graph);
+      if (graph) (void)hipGraphDestroy(graph);
+      throw;
+    }
+    hip_check(hipStreamEndCapture(dev.stream, &graph), "hipStreamEndCapture");
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    hip_check(e, "hipGraphInstantiate");
+    it = rt.graphs.emplace(key, exec).first;
+  }
+  dev.make_current();
+  hip_check(hipGraphLaunch(it->second, dev.stream), "hipGraphLaunch");
+}
+
 int ocannl_hip_routine_run(ocannl_hip_routine* rt) {
   return guarded([&] {
     if (!rt) throw InvalidArgument("run: null routine");
-    enqueue(*rt, nullptr, 0);
+    run_plain(*rt);
   });
 }
 

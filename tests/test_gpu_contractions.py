@@ -342,3 +342,43 @@ def test_mixed_precision_product_against_the_reference_semantics(copies):
     print(f"fp32 x bf16 product: relative Frobenius error against the serial fp32-operand semantics {err:.2e}")
     assert 1e-4 < err <= 2e-2      # a real deviation (one bf16 rounding of an operand), well inside the bar
     hip.close()
+
+
+@pytest.mark.parametrize("shape", [(256, 384, 128), (136, 72, 200), (1024, 2048, 512)])
+def test_bias_and_relu_consumers_folded_into_the_epilogue(shape):
+    # an mlp layer as the optimiser hands it over: y[b, o] := (the inlined product w x) + bias[o];
+    # z := relu(y).  By default the contraction's epilogue stores y and z itself (`epilogues=0`: the
+    # product goes to scratch and two pointwise statements follow).  Same roundings in the same order:
+    # bit for bit the same y and z, on full tiles (16-byte stores) and ragged ones.
+    from ocannl_amd.frontend import Graph, make_routine
+    from ocannl_amd import backend as B
+    Bn, O, I = shape
+    L.reset_symbols(0)
+    g = Graph("bfloat16", "single")
+    x = g.input("x", ("b", "i"), (Bn, I)); w = g.param("w", ("o", "i"), (O, I)); bias = g.param("bias", ("o",), (O,))
+    y = g.add(g.einsum(w, x, ("b", "o"), ident="wx"), bias, ("b", "o"), ident="y")
+    z = g.unary("relu", y, ident="z")
+    r = make_routine(g, "mlp_layer", g.forward(z), outputs=[y.value, z.value])
+    rng = np.random.default_rng(Bn)
+    init = {x.value.id: W.as_prec(rng.standard_normal((Bn, I)).astype(np.float32), "bfloat16"),
+            w.value.id: W.as_prec((rng.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32), "bfloat16"),
+            bias.value.id: W.as_prec(rng.standard_normal(O).astype(np.float32), "bfloat16")}
+    folded, apart = HipRun(r, init, "min_mfma_flops=1"), HipRun(r, init, "min_mfma_flops=1;epilogues=0;fused=0")
+    kf, ka = folded.code.kernels(), apart.code.kernels()
+    assert [k["kind"] for k in kf] == ["mfma"] and len(ka) > 1, (kf, ka)
+    folded.step(); apart.step()
+    yf, zf = folded.get(y.value), folded.get(z.value)
+    assert np.array_equal(yf, apart.get(y.value)) and np.array_equal(zf, apart.get(z.value))
+    # (with a contracted extent of at most 128 the third form exists too: the product as the prologue of
+    # the row-wise kernel that adds the bias and applies relu)
+    third = HipRun(r, init, "min_mfma_flops=1;epilogues=0")
+    if [k["kind"] for k in third.code.kernels()] == ["generated"]:
+        third.step()
+        assert np.array_equal(yf, third.get(y.value)) and np.array_equal(zf, third.get(z.value))
+    third.close()
+    # and against the mathematics: relu(w x + bias) in float64 from the same bf16 inputs
+    want = W.to_float(init[x.value.id], "bfloat16") @ W.to_float(init[w.value.id], "bfloat16").T + W.to_float(init[bias.value.id], "bfloat16")
+    assert np.max(np.abs(W.to_float(yf, "bfloat16") - want)) <= 2.0 ** -7 * np.max(np.abs(want))
+    assert np.array_equal(W.to_float(zf, "bfloat16"), np.maximum(W.to_float(yf, "bfloat16"), 0.0))
+    assert np.any(W.to_float(zf, "bfloat16") > 0) and np.any(W.to_float(yf, "bfloat16") < 0)
+    folded.close(); apart.close()
