@@ -228,3 +228,73 @@ __device__ __forceinline__ void ocn_rowtile_contract(const unsigned short* __res
     for (int e = 0; e < 16; ++e) ocn_rowtile_put(out + ((e >> 2) * 8 + (e & 3)) * T, acc[e]);
   }
 }
+
+// Row group with a contraction epilogue: the workgroup's 32 finished rows y[32][T] (bf16 bits in LDS,
+// YS elements from row to row) times b[T][N] (bf16 in memory, unit stride along n, b_row elements from
+// t to t + 1) give c[32][N] (c_row elements from row to row; `copy`, when given, receives the same
+// values as bf16 at the same offsets).  Wave w takes the 32-column block w % (N / 32) and part
+// w / (N / 32) of the KP parts of T; with KP > 1 the partial results meet in `ps` (LDS, KP x 32 x N
+// floats) and are added in a fixed order.  Every wave of the workgroup calls it (it holds a barrier).
+OCN_DEV void ocn_rowtile_put4(unsigned short* p, const float* v) {
+  typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+  u32x2 w;
+  w[0] = (unsigned int)single_to_bfloat16(v[0]) | ((unsigned int)single_to_bfloat16(v[1]) << 16);
+  w[1] = (unsigned int)single_to_bfloat16(v[2]) | ((unsigned int)single_to_bfloat16(v[3]) << 16);
+  *reinterpret_cast<u32x2*>(p) = w;
+}
+OCN_DEV void ocn_rowtile_put4(float* p, const float* v) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  f32x4 w;
+  w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
+  *reinterpret_cast<f32x4*>(p) = w;
+}
+
+template <int T, int N, int NW, int KP, int YS, typename CT>
+__device__ __forceinline__ void ocn_rowtile_project(const unsigned short* ys, const unsigned short* __restrict__ b, long long b_row,
+                                                    float* ps, CT* __restrict__ c, long long c_row, unsigned short* __restrict__ copy) {
+  static_assert(T % (16 * KP) == 0 && N % 32 == 0 && (N / 32) * KP <= NW, "row-tile epilogue: shape");
+  constexpr int NB = N / 32, KS = T / 16 / KP;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (wave < NB * KP) {
+    const int nb = wave % NB, kp = wave / NB;
+    ocn_f32x16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+    const unsigned short* yp = ys + (lane & 31) * YS + kp * (KS * 16) + (lane >> 5) * 8;
+    const unsigned short* bp = b + (long long)(kp * (KS * 16) + (lane >> 5) * 8) * b_row + nb * 32 + (lane & 31);
+#pragma unroll 4
+    for (int kk = 0; kk < KS; ++kk) {
+      const ocn_bf16x8 af = __builtin_bit_cast(ocn_bf16x8, *reinterpret_cast<const ocn_u32x4*>(yp + kk * 16));
+      ocn_u32x4 bw;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        bw[j] = (unsigned int)bp[(long long)(kk * 16 + 2 * j) * b_row] | ((unsigned int)bp[(long long)(kk * 16 + 2 * j + 1) * b_row] << 16);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, __builtin_bit_cast(ocn_bf16x8, bw), acc, 0, 0, 0);
+    }
+    const int col = nb * 32 + (lane & 31);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int row = (e >> 2) * 8 + (e & 3) + (lane >> 5) * 4;
+      if (KP > 1) ps[(kp * 32 + row) * N + col] = acc[e];
+      else {
+        ocn_rowtile_put(c + row * c_row + col, acc[e]);
+        if (copy) copy[row * c_row + col] = single_to_bfloat16(acc[e]);
+      }
+    }
+  }
+  if (KP > 1) {
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 32 * N / 4; idx += NW * 64) {
+      const int row = idx / (N / 4), c4 = (idx % (N / 4)) * 4;
+      float v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = ps[row * N + c4 + q];
+#pragma unroll
+      for (int p = 1; p < KP; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] += ps[(p * 32 + row) * N + c4 + q];
+      ocn_rowtile_put4(c + row * c_row + c4, v);
+      if (copy) ocn_rowtile_put4(copy + row * c_row + c4, v);
+    }
+  }
+}

@@ -302,6 +302,7 @@ struct Printer {
   // group is also kept in `cache_name` (an array indexed by the unrolled row iteration `it_` for
   // row-position values, a scalar every lane holds for per-row values) and later reads of it
   // inside the group use that instead of memory.
+  bool row_vec4 = false;                    // see row_loop
   int row_iters = 0;                        // > 0: loops over the row position run `it_` = 0..row_iters-1, unrolled
   std::map<int, std::string> cache_name;    // node -> register expression
   std::set<int> cache_defined;              // nodes whose cache holds the current value
@@ -360,11 +361,20 @@ struct Printer {
     }
   }
 
+  // the row position that unrolled iteration `it_` of a lane stands for
+  std::string row_pos(int lanes) const {
+    if (row_vec4 && row_iters % 4 == 0) return "lane_ * 4u + (it_ & 3u) + (it_ >> 2) * " + std::to_string(lanes * 4) + "u";
+    return "lane_ + it_ * " + std::to_string(lanes);
+  }
   // header of a loop over the row position shared by `lanes` lanes
   std::string row_loop(const std::string& sym, int64_t from, int64_t to, int lanes, const std::string& ind) {
-    if (row_iters > 0 && from == 0)
-      return ind + "_Pragma(\"unroll\") for (uint32_t it_ = 0; it_ < " + std::to_string(row_iters) + "; ++it_) { const " + idx_t + " " +
-             sym + " = lane_ + it_ * " + std::to_string(lanes) + ";";
+    if (row_iters > 0 && from == 0) {
+      const std::string head = ind + "_Pragma(\"unroll\") for (uint32_t it_ = 0; it_ < " + std::to_string(row_iters) + "; ++it_) { const " +
+                               idx_t + " " + sym + " = ";
+      // a lane takes runs of four neighbouring positions, so that the unrolled loads and stores of a
+      // unit-stride tensor combine into 16-byte (fp32) or 8-byte (bf16) accesses
+      return head + row_pos(lanes) + ";";
+    }
     return ind + "for (" + idx_t + " " + sym + " = " + std::to_string(from) + " + lane_; " + sym + " <= " + std::to_string(to) +
            "; " + sym + " += " + std::to_string(lanes) + ") {";
   }
@@ -880,6 +890,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
     if (plan.large_index) pr.idx_t = "uint64_t";
     pr.mirrors = &plan.mirrors;
     pr.debug_log = plan.debug_log;
+    pr.row_vec4 = plan.row_vec4;
     std::vector<std::string> body;
     const std::string ind = "  ";
 
@@ -981,7 +992,38 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           }
           body.push_back(rind + "}");
         }
+        // contraction epilogue: the finished row of y replaces the row of x in LDS, as bf16 (the wave owns
+        // both; a row of y takes at most the bytes of a row of x)
+        const int64_t ys = q.row_len * (int64_t)prec_in_bytes(xn.prec) / 2;   // row stride of y in LDS, in bf16 elements
+        if (q.proj_y >= 0) {
+          auto yc = pr.cache_name.find(q.proj_y);
+          if (yc == pr.cache_name.end() || yc->second.find("[it_]") == std::string::npos) throw InvalidArgument("planner: row-group epilogue over a tensor the group does not keep");
+          const std::string bits = r.node(q.proj_y).prec == Prec::Bfloat16 ? yc->second : "single_to_bfloat16(" + yc->second + ")";
+          body.push_back(rind + "_Pragma(\"unroll\") for (uint32_t it_ = 0; it_ < " + std::to_string(pr.row_iters) + "; ++it_) ((unsigned short*)xs_)[" +
+                         pr.lds_row + " * " + std::to_string(ys) + "u + " + pr.row_pos(QG) + "] = " + bits + ";");
+        }
         body.push_back(pind + "}");
+        if (q.proj_y >= 0) {
+          const int NB = (int)(q.proj_n / 32);
+          const int KP = q.proj_kp;
+          if (KP < 1 || KP * NB > NW || (q.row_len / 16) % KP != 0) throw InvalidArgument("planner: row-group epilogue split the kernel does not take");
+          pr.used_nodes.insert(q.proj_b.node); pr.used_nodes.insert(q.proj_c.node);
+          if (q.proj_c_copy >= 0) pr.used_nodes.insert(q.proj_c_copy);
+          std::string bo = std::to_string(q.proj_b.offset) + "ull", co = std::to_string(q.proj_c.offset) + "ull";
+          for (size_t k = 0; k < n; ++k) {
+            const std::string tk = "(uint64_t)t" + std::to_string(k) + "_" + (k == (size_t)ma ? " * 32ull" : "");
+            if (q.proj_b_stride[k]) bo += " + " + tk + " * " + std::to_string(q.proj_b_stride[k]) + "ull";
+            if (q.proj_c_stride[k]) co += " + " + tk + " * " + std::to_string(q.proj_c_stride[k]) + "ull";
+          }
+          if (KP > 1) body.push_back(pind + "__shared__ __attribute__((aligned(16))) float ps_[" + std::to_string((int64_t)KP * 32 * q.proj_n) + "];");
+          body.push_back(pind + "__syncthreads();");
+          body.push_back(pind + "ocn_rowtile_project<" + std::to_string(q.row_len) + ", " + std::to_string(q.proj_n) + ", " + std::to_string(NW) + ", " +
+                         std::to_string(KP) + ", " + std::to_string(ys) + ">((const unsigned short*)xs_, " +
+                         r.node(q.proj_b.node).ident + " + (" + bo + "), " + std::to_string(q.proj_b_row) + "ll, " +
+                         (KP > 1 ? "ps_" : "(float*)0") + ", " + r.node(q.proj_c.node).ident + " + (" + co + "), " +
+                         std::to_string(q.proj_c_stride[ma]) + "ll, " +
+                         (q.proj_c_copy >= 0 ? r.node(q.proj_c_copy).ident + " + (" + co + ")" : std::string("(unsigned short*)0")) + ");");
+        }
         pr.lds_node = -1;
         pr.row_iters = 0; pr.cache_name.clear(); pr.cache_defined.clear();
         return (uint64_t)(QP * (uint64_t)fused_block);

@@ -508,6 +508,7 @@ bool phase_touches(const Phase& ph, int node) {
   }
   if (!ph.parallel_members.empty()) { for (auto& m : ph.parallel_members) if (phase_touches(m, node)) return true; return false; }
   if (ph.fused_x >= 0 && (ph.fused_x == node || ph.fused_a.node == node || ph.fused_b.node == node)) return true;
+  if (ph.proj_y >= 0 && (ph.proj_b.node == node || ph.proj_c.node == node || ph.proj_c_copy == node)) return true;
   if (!ph.members.empty()) { for (auto& m : ph.members) if (phase_touches(m, node)) return true; return false; }
   if (!ph.serial_members.empty()) { for (auto& m : ph.serial_members) if (phase_touches(m, node)) return true; return false; }
   std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
@@ -1481,6 +1482,7 @@ bool phase_writes(const Phase& ph, int node) {
     return false;
   };
   if (ph.fused_x == node && ph.fused_x_store) return true;
+  if (ph.proj_y >= 0 && (ph.proj_c.node == node || ph.proj_c_copy == node)) return true;
   if (!ph.members.empty()) { for (auto& m : ph.members) if (writes(m)) return true; return false; }
   if (!ph.parallel_members.empty()) { for (auto& m : ph.parallel_members) if (phase_writes(m, node)) return true; return false; }
   if (!ph.serial_members.empty()) { for (auto& m : ph.serial_members) if (phase_writes(m, node)) return true; return false; }
@@ -1826,6 +1828,142 @@ void fuse_row_contractions(Routine& r, Plan& plan, bool also_stored) {
   }
 }
 
+
+// ---- ... and a contraction as the epilogue of the row group that produces its operand -------------------
+// `c[o.., n] (=) sum_t y[o.., t] * b[.., t, n]` right behind a row group with a prologue, y being what one
+// of its members stores per row position (attention weights times V: lib/nn_blocks.ml:233-236): the
+// group's workgroup, which holds 32 finished rows of y, multiplies them with b itself.  Saves a launch
+// and the read of y; y is still stored (it is a context node).
+void fuse_row_projections(Routine& r, Plan& plan) {
+  std::map<int, int> mirror_source;
+  for (auto& kv : plan.mirrors) mirror_source[kv.second] = kv.first;
+  auto source_of = [&](int node) { auto m = mirror_source.find(node); return m == mirror_source.end() ? node : m->second; };
+  for (size_t j = 0; j < plan.phases.size(); ++j) {
+    Phase& G = plan.phases[j];
+    if (G.kind != Phase::Generic || G.members.empty() || G.fused_x < 0 || G.proj_y >= 0) continue;
+    const size_t n_outer = G.row_outer_ext.size();
+    const int ma = G.fused_m_axis;
+    std::string identity;
+    for (size_t k = 0; k < n_outer; ++k) identity += "o" + std::to_string(k) + ",";
+    identity += "r,";
+    // per-position results of the group: node -> index of the last member that stores it
+    std::map<int, size_t> stored_by;
+    for (size_t mi = 0; mi < G.members.size(); ++mi) {
+      const Phase& m = G.members[mi];
+      if (m.inner.size() != 1 || m.inner[0]->kind != Stmt::Set) continue;
+      const Stmt& st = *m.inner[0];
+      if (m.row_role == Phase::RowPointwise && row_signature(m, st.idcs) == identity) stored_by[st.node] = mi;
+      else stored_by.erase(st.node);
+    }
+    for (size_t i = j + 1; i < plan.phases.size() && G.proj_y < 0; ++i) {
+      const Phase& P = plan.phases[i];
+      if (P.kind != Phase::Contraction) continue;
+      const GemmDesc& g = P.gemm;
+      if (g.accumulate || !g.group.empty() || !g.more.empty() || g.epi_bias >= 0 || g.epi_relu >= 0) continue;
+      if (P.inner.size() != 1 || P.inner[0]->kind != Stmt::Set) continue;
+      const Stmt& set = *P.inner[0];
+      const Scalar& v = *set.value;
+      const Scalar *pa = nullptr, *pb = nullptr;
+      if (v.kind == Scalar::Tern && v.tern == Ternop::Fma) { pa = v.a.get(); pb = v.b.get(); }
+      else if (v.kind == Scalar::Bin && v.bin == Binop::Add) {
+        const Scalar* mul = v.b->kind == Scalar::Bin && v.b->bin == Binop::Mul ? v.b.get() : v.a->kind == Scalar::Bin && v.a->bin == Binop::Mul ? v.a.get() : nullptr;
+        if (mul) { pa = mul->a.get(); pb = mul->b.get(); }
+      }
+      if (!pa || !pb || pa->kind != Scalar::Get || pb->kind != Scalar::Get) continue;
+      const Scalar* yget = stored_by.count(pa->node) ? pa : stored_by.count(pb->node) ? pb : nullptr;
+      if (!yget) continue;
+      const Scalar* bget = yget == pa ? pb : pa;
+      const int Y = yget->node;
+      if (stored_by.count(bget->node) || bget->node == G.fused_x) continue;
+      const Node& yn = r.node(Y);
+      if (!(yn.prec == Prec::Bfloat16 || yn.prec == Prec::Single) || yn.dims.size() != n_outer + 1 || yn.dims.back() != G.row_len) continue;
+      // which operand of the planned contraction stands for y (itself, or the bf16 copy its stores keep in step)
+      auto is_y = [&](const GemmOperand& o) { return o.node == Y || source_of(o.node) == Y; };
+      if (is_y(g.a) == is_y(g.b)) continue;
+      const GemmOperand& yop = is_y(g.a) ? g.a : g.b;
+      const GemmOperand& bop = is_y(g.a) ? g.b : g.a;
+      if (yop.prec != Prec::Bfloat16 || bop.prec != Prec::Bfloat16) continue;
+      if (r.node(bop.node).dims != r.node(bget->node).dims) continue;   // (a bf16 copy has its source's layout)
+      if (!(g.c.prec == Prec::Bfloat16 || g.c.prec == Prec::Single)) continue;
+      // y read through plain iterators, one per axis; those loops run over the group's rows
+      std::map<int, std::pair<int64_t, int64_t>> range;   // symbol -> (from, extent)
+      for (size_t q = 0; q < P.par_syms.size(); ++q) range[P.par_syms[q]] = {P.par_from[q], P.par_ext[q]};
+      for (size_t q = 0; q < P.seq_syms.size(); ++q) range[P.seq_syms[q]] = {P.seq_from[q], P.seq_to[q] - P.seq_from[q] + 1};
+      std::vector<int> ysym;
+      bool plain = yget->idcs.size() == yn.dims.size();
+      std::set<int> distinct;
+      for (size_t p = 0; p < yget->idcs.size() && plain; ++p) {
+        const AxisIndex& ix = yget->idcs[p];
+        const int64_t want = p < n_outer ? G.row_outer_ext[p] : G.row_len;
+        if (ix.kind == AxisIndex::Fixed && ix.fixed == 0 && want == 1) { ysym.push_back(-1); continue; }
+        plain = ix.kind == AxisIndex::Iter && !r.is_static(ix.sym) && distinct.insert(ix.sym).second && range.count(ix.sym) &&
+                range[ix.sym].first == 0 && range[ix.sym].second == want && yn.dims[p] == want;
+        ysym.push_back(ix.sym);
+      }
+      if (!plain || ysym.back() < 0) continue;
+      const int tsym = ysym.back();
+      std::vector<int> others;
+      for (auto& kv : range) if (!distinct.count(kv.first) && kv.second.second != 1) others.push_back(kv.first);
+      if (others.size() != 1 || range[others[0]].first != 0) continue;
+      const int nsym = others[0];
+      const int64_t N = range[nsym].second;
+      if (N % 32 != 0 || N > 128) continue;
+      const Strides sb = strides_of(r, bget->node, bget->idcs), sc = strides_of(r, set.node, set.idcs);
+      if (!sb.statics.empty() || !sc.statics.empty()) continue;
+      if (get_stride(sb, nsym) != 1 || get_stride(sc, nsym) != 1 || get_stride(sc, tsym) != 0 || get_stride(sb, tsym) <= 0) continue;
+      Phase F;
+      bool ok = sb.offset % 4 == 0 && sc.offset % 4 == 0 && sb.offset >= 0 && sc.offset >= 0;
+      for (size_t k = 0; k < n_outer; ++k) {
+        const int64_t bk = ysym[k] < 0 ? 0 : get_stride(sb, ysym[k]), ck = ysym[k] < 0 ? 0 : get_stride(sc, ysym[k]);
+        F.proj_b_stride.push_back(bk); F.proj_c_stride.push_back(ck);
+        ok = ok && bk >= 0 && ck >= 0 && ck % 4 == 0 && ((int)k != ma || (bk == 0 && ck > 0));
+      }
+      if (!ok) continue;
+      // c must keep its rows apart: one (outer.., n) cell per (rows, n)
+      {
+        std::vector<std::pair<int64_t, int64_t>> ax{{1, N}};   // (stride, extent)
+        for (size_t k = 0; k < n_outer; ++k) if (G.row_outer_ext[k] > 1) ax.push_back({F.proj_c_stride[k], G.row_outer_ext[k]});
+        std::sort(ax.begin(), ax.end());
+        for (size_t q = 1; q < ax.size(); ++q) ok = ok && ax[q].first >= ax[q - 1].first * ax[q - 1].second;
+      }
+      if (!ok) continue;
+      // the contraction moves up to the group: nothing in between may write b or touch c
+      bool free_to_move = true;
+      for (size_t q = j + 1; q < i && free_to_move; ++q) {
+        const Phase& mid = plan.phases[q];
+        free_to_move = !phase_writes(mid, bop.node) && !phase_writes(mid, source_of(bop.node)) && !phase_touches(mid, g.c.node) &&
+                       (g.c_copy < 0 || !phase_touches(mid, g.c_copy));
+        auto cm = plan.mirrors.find(g.c.node);
+        if (cm != plan.mirrors.end()) free_to_move = free_to_move && !phase_touches(mid, cm->second);
+      }
+      if (!free_to_move || plan.mirrors.count(g.c.node)) continue;
+      // ... and the group itself must not touch c or write b
+      if (phase_touches(G, g.c.node) || phase_writes(G, bop.node) || phase_writes(G, source_of(bop.node))) continue;
+      // the sum over t is split over the waves that the static LDS budget lets hold a partial result;
+      // with fewer than four waves at work the separate launch is faster (measured: 1024-long rows,
+      // whose bf16 tile fills the 64 KiB: 2.78 against 2.69 ms for the attention step)
+      const int NW = G.row_len <= 512 ? 16 : 8, NB = (int)(N / 32);
+      int KP = 1;
+      while (KP * 2 * NB <= NW && KP < 4 && (G.row_len / 16) % (KP * 2) == 0 &&
+             32 * G.row_len * (int64_t)prec_in_bytes(r.node(G.fused_x).prec) + (int64_t)(KP * 2) * 32 * N * 4 <= 60 * 1024) KP *= 2;
+      if (KP * NB < 4) continue;
+      G.proj_kp = KP;
+      G.proj_y = Y;
+      G.proj_b = bop; G.proj_b.offset = sb.offset;
+      G.proj_c = g.c; G.proj_c.offset = sc.offset;
+      G.proj_b_stride = F.proj_b_stride; G.proj_c_stride = F.proj_c_stride;
+      G.proj_b_row = get_stride(sb, tsym);
+      G.proj_n = N;
+      G.proj_c_copy = g.c_copy;
+      G.flops += P.flops;
+      G.bytes += P.bytes - (double)yn.num_elems() * 2.0;   // y is not read back
+      G.label += " -> " + P.label;
+      plan.phases.erase(plan.phases.begin() + i);
+      break;
+    }
+  }
+}
+
 }  // namespace
 
 // ---- contractions off the critical path ---------------------------------------------------------------
@@ -1962,6 +2100,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
   struct SeqGuard { bool old; SeqGuard(bool v) : old(g_all_sequential) { g_all_sequential = v; } ~SeqGuard() { g_all_sequential = old; } } seq_guard(opt.debug_log);
   Plan plan;
   plan.debug_log = opt.debug_log;
+  plan.row_vec4 = opt.row_vec4;
   plan.use_graphs = opt.use_graphs;
   plan.large_index = opt.large_models;
   for (auto& kv : r.nodes) if (kv.second.num_elems() > (int64_t)0x7FFFFFFF) plan.large_index = true;
@@ -2064,6 +2203,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
   if (opt.enable_mfma && opt.group_contractions) merge_contractions(plan, false, opt.group_window);
   if (opt.enable_coop && opt.enable_row_groups) group_rows(r, plan);
   if (opt.enable_mfma && opt.enable_coop && opt.enable_row_groups && opt.fuse_row_contractions) fuse_row_contractions(r, plan, opt.fuse_stored_rows);
+  if (opt.enable_mfma && opt.enable_coop && opt.enable_row_groups && opt.fuse_row_contractions && opt.fuse_row_projections) fuse_row_projections(r, plan);
   if (opt.enable_serial_group) serialise_tiny(r, plan);
   if (opt.enable_coop && opt.enable_parallel_groups) group_independent(r, plan);
   if (opt.enable_mfma && opt.side_queue && r.merge_node < 0) assign_side_queue(plan);

@@ -115,6 +115,18 @@ struct Phase {
   int64_t fused_b_row = 0;                            // stride of B along the row position
   int64_t fused_k = 0;                                // contracted extent (unit stride in both operands)
   int fused_m_axis = -1;
+  // ... and a contraction epilogue (proj_y >= 0; only with a prologue, whose 32-row workgroups it shares):
+  // `c[o.., n] = sum_t y[o.., t] * b[.., t, n]`, where y is what a member of the group stores per row
+  // position -- attention weights times V, the gradient of the scores times K -- is taken out of the
+  // plan as well: the rows of y stay in LDS as bf16 and the workgroup multiplies its 32 x T tile with
+  // b on the matrix cores.  b and c are unit-stride along n.
+  int proj_y = -1;
+  GemmOperand proj_b, proj_c;                           // node, precision, constant offset
+  std::vector<int64_t> proj_b_stride, proj_c_stride;    // element stride per outer axis of the group
+  int64_t proj_b_row = 0;                               // stride of b along t
+  int64_t proj_n = 0;
+  int proj_kp = 1;                                      // parts of T that separate waves sum up (partial results meet in LDS)
+  int proj_c_copy = -1;                                 // bf16 copy of an fp32 c, stored alongside
   // Fill
   int fill_node = -1;
   // Contraction
@@ -146,6 +158,10 @@ struct PlanOptions {
   // every top-level statement becomes a kernel of ONE thread that walks its loops in order, and none
   // of the fusing rewrites applies.
   bool debug_log = false;
+  // row groups: a lane takes runs of four neighbouring row positions, for 16-byte accesses.  Off:
+  // measured on the transformer step the wide accesses were 5-8% slower than one position per lane
+  // per unrolled iteration (these kernels are bound by the memory system, not by instruction count).
+  bool row_vec4 = false;
   // plain runs replay a captured HIP graph of the routine's kernels.  Off by default: measured on
   // MI355X / ROCm 7.2 it pays only for a routine of about ten tiny kernels (half-moons step as ten
   // launches: 40 -> 26 us); nine kernels of the char-MLP step went 36 -> 42 us and the 127 kernels of
@@ -155,6 +171,7 @@ struct PlanOptions {
   bool side_queue = true;            // contractions off the critical path run on a second queue beside the rest
   bool fuse_epilogues = true;        // bias / relu consumers of an inlined contraction run in the contraction's epilogue
   bool fuse_row_contractions = true; // a short-K contraction feeding a row group runs as that kernel's prologue ...
+  bool fuse_row_projections = true;   // contraction epilogue of a row group with a prologue (see Phase::proj_y)
   bool fuse_stored_rows = false;     // ... also when its result has to be stored anyway (a context node): measured slower
   bool enable_bf16_copies = true;   // keep bf16 copies of fp32 operands of mixed contractions (written by the producing kernels)
 };
@@ -167,6 +184,7 @@ struct Plan {
   std::map<int, int> mirrors;
   bool large_index = false;    // generated kernels compute offsets in 64 bits
   bool use_graphs = false;     // plain runs are replayed from a captured HIP graph
+  bool row_vec4 = false;       // row groups: a lane takes runs of four neighbouring row positions (16-byte accesses)
   bool debug_log = false;      // generated kernels print what they compute (and take an `int log_id` argument)
   std::vector<std::string> trailing_comments;   // debug logging: comments after the last phase
 };
