@@ -491,6 +491,35 @@ struct Printer {
 
   struct Def { int scope; std::vector<std::string> lines; };
 
+  // An operand of a C conditional (`where`, `relu_gate`) that reads memory is loaded ahead of the
+  // statement: written inside `c ? x[i] : 0` the load would wait for the condition -- two dependent
+  // trips to memory per element (the relu backward pass of the transformer step ran at 3.2 TB/s).
+  // Only reads through loop iterators and fixed positions are moved: those are in range whatever the
+  // condition says.  Same value either way.
+  static bool safe_reads(const Scalar& s, bool* any) {
+    switch (s.kind) {
+      case Scalar::Get:
+        for (auto& ix : s.idcs) if (ix.kind != AxisIndex::Iter && ix.kind != AxisIndex::Fixed) return false;
+        *any = true;
+        return true;
+      case Scalar::Const: case Scalar::Bits: case Scalar::GetLocal: case Scalar::Index: return true;
+      case Scalar::Un: return s.un != Unop::Uniform1 && safe_reads(*s.a, any);
+      case Scalar::Bin: return safe_reads(*s.a, any) && safe_reads(*s.b, any);
+      case Scalar::Tern: return safe_reads(*s.a, any) && safe_reads(*s.b, any) && safe_reads(*s.c, any);
+      default: return false;
+    }
+  }
+  int hoisted = 1;
+  std::string eager(Prec prec, const Scalar& s, const std::string& expr, const std::string& ind, std::vector<Def>& defs) {
+    bool any = false;
+    if (debug_log || !safe_reads(s, &any) || !any) return expr;
+    const std::string t = "w" + std::to_string(fresh++) + "_";
+    Def d; d.scope = -(++hoisted);   // (definitions of one scope id are printed once: give each load its own)
+    d.lines.push_back(ind + "const " + c_typ(prec) + " " + t + " = " + expr + ";");
+    defs.push_back(std::move(d));
+    return t;
+  }
+
   std::string scalar(Prec prec, const Scalar& s, const std::string& ind, std::vector<Def>& defs) {
     switch (s.kind) {
       case Scalar::LocalScope: {
@@ -555,6 +584,7 @@ struct Printer {
         std::string a = scalar(s.tern == Ternop::Where ? s.arg_prec : prec, *s.a, ind, defs);
         std::string b = scalar(prec, *s.b, ind, defs);
         std::string c = scalar(prec, *s.c, ind, defs);
+        if (s.tern == Ternop::Where) { b = eager(prec, *s.b, b, ind, defs); c = eager(prec, *s.c, c, ind, defs); }
         return emit_ternop(prec, s.tern, a, b, c);
       }
       case Scalar::Bin: {
@@ -562,6 +592,7 @@ struct Printer {
         if (s.bin == Binop::Arg2) return scalar(prec, *s.b, ind, defs);
         std::string a = scalar(prec, *s.a, ind, defs);
         std::string b = scalar(prec, *s.b, ind, defs);
+        if (s.bin == Binop::ReluGate) b = eager(prec, *s.b, b, ind, defs);
         return emit_binop(prec, s.bin, a, b);
       }
       case Scalar::Un: {
@@ -962,7 +993,11 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
             pr.cache_name[st.node] = base;
           }
         }
-        body.push_back(pind + "for (uint32_t rl_ = 0; rl_ < " + std::to_string(RPW) + "u; ++rl_) {");
+        // the rows of a wave are independent: unrolled (while what they keep in registers stays small), the
+        // loads, shuffles and stores of one row fill the waits of the other
+        const int row_unroll = RPW * pr.row_iters <= 16 ? RPW : pr.row_iters <= 8 ? 2 : 1;
+        body.push_back(pind + (row_unroll > 1 ? "_Pragma(\"unroll " + std::to_string(row_unroll) + "\") " : "") +
+                       "for (uint32_t rl_ = 0; rl_ < " + std::to_string(RPW) + "u; ++rl_) {");
         const std::string rind = pind + "  ";
         for (size_t k = 0; k < n; ++k)
           body.push_back(rind + "const " + pr.idx_t + " row" + std::to_string(k) + "_ = t" + std::to_string(k) + "_" +
