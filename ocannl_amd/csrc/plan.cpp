@@ -1927,11 +1927,12 @@ void fuse_row_projections(Routine& r, Plan& plan) {
         for (size_t q = 1; q < ax.size(); ++q) ok = ok && ax[q].first >= ax[q - 1].first * ax[q - 1].second;
       }
       if (!ok) continue;
-      // the contraction moves up to the group: nothing in between may write b or touch c
+      // the contraction moves up to the group: nothing in between may write y or b, or touch c
       bool free_to_move = true;
       for (size_t q = j + 1; q < i && free_to_move; ++q) {
         const Phase& mid = plan.phases[q];
-        free_to_move = !phase_writes(mid, bop.node) && !phase_writes(mid, source_of(bop.node)) && !phase_touches(mid, g.c.node) &&
+        free_to_move = !phase_writes(mid, Y) && !phase_writes(mid, yop.node) &&
+                       !phase_writes(mid, bop.node) && !phase_writes(mid, source_of(bop.node)) && !phase_touches(mid, g.c.node) &&
                        (g.c_copy < 0 || !phase_touches(mid, g.c_copy));
         auto cm = plan.mirrors.find(g.c.node);
         if (cm != plan.mirrors.end()) free_to_move = free_to_move && !phase_touches(mid, cm->second);

@@ -259,3 +259,23 @@ def test_weight_gradients_go_to_the_side_queue_and_fused_prologues_show_up():
     # ... and attention weights times V runs in there as well
     assert "ocn_rowtile_project<256, 64, 16, 4, 256>" in fused.source().split("extern \"C\"", 1)[1]
     assert n(fused) == n(apart) - 4
+
+
+def test_memory_operands_of_conditionals_are_loaded_ahead_of_the_statement():
+    # `g[i] = relu_gate(a[i], b[i])` and `w[i] = where(a[i], b[i], c[i])`: written as C conditionals the
+    # loads of b and c would wait for the condition (two dependent trips to memory); reads through plain
+    # loop iterators are in range whatever the condition says and are issued first.  A read through an
+    # affine index (a convolution window that the condition may be guarding) stays where it is.
+    L.reset_symbols(0)
+    n = 4096
+    a, b, c = (L.Node(k + 1, s, "single", (n,)) for k, s in enumerate("abc"))
+    g, w, v = L.Node(4, "g", "single", (n,)), L.Node(5, "w", "single", (n,)), L.Node(6, "v", "single", (n // 2,))
+    i, j, k = L.fresh_symbol(), L.fresh_symbol(), L.fresh_symbol()
+    body = [L.For(i, 0, n - 1, [L.Set(g, (L.It(i),), L.Binop("relu_gate", L.Get(a, (L.It(i),)), L.Get(b, (L.It(i),))))]),
+            L.For(j, 0, n - 1, [L.Set(w, (L.It(j),), L.Ternop("where", L.Get(a, (L.It(j),)), L.Get(b, (L.It(j),)), L.Get(c, (L.It(j),))))]),
+            L.For(k, 0, n // 2 - 1, [L.Set(v, (L.It(k),), L.Binop("relu_gate", L.Get(a, (L.It(k),)),
+                                                                   L.Get(b, (L.Affine([(2, k)], 1),))))])]
+    src = B.compile(L.Routine("conditionals", body), "parallel=0;rows=0").source().split("extern \"C\"", 1)[1]
+    assert re.search(r"const float (w\d+_) = b\[i\d+\];\s*g\[i\d+\] = \(a\[i\d+\] > 0\.0 \? \1 : 0\.0\);", src), src
+    assert len(re.findall(r"const float w\d+_ = [bc]\[", src)) == 3, src
+    assert re.search(r"v\[[^\]]*\] = \(a\[[^\]]*\] > 0\.0 \? b\[[^\]]*\] : 0\.0\);", src), src
