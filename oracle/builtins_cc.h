@@ -9,10 +9,14 @@
  *   threefry4x32 light (2)    builtins.c:156-196,284-329  pinned: test/operations/
  *                                                    test_threefry4x32.ml:37-46 and
  *                                                    threefry4x32_demo.ml:31-73
- *   threefry4x32 crypto (20)  builtins.c:199-281     PARITY UNPINNED: the reference holds no
- *                                                    vector for it and it is not Random123's
- *                                                    Threefry-4x32 (it uses the 2x32 rotation
- *                                                    set); shares the round with the light one
+ *   threefry4x32 crypto (20)  builtins.c:199-281     pinned: the reference's own C text of
+ *                                                    builtins.c (math.h include down to the
+ *                                                    OCaml wrappers) compiled unchanged into
+ *                                                    oracle/_ref/builtins_ref.so and compared
+ *                                                    bit for bit on 20 000 random key/counter
+ *                                                    pairs, as are the light variant, the
+ *                                                    uniform converters and the conversions
+ *                                                    (tests/test_oracle_builtins.py)
  *   uint4x32 -> uniform       builtins.c:345-528     pinned: same KATs + closed forms
  *   X -> uint4x32             builtins.c:531-606     pinned: same KATs (counter spreading)
  *   bf16 / fp8(E5M2)          builtins.c:611-743     pinned: arrayjit/test/
