@@ -163,7 +163,7 @@ def measure(workload: str, steps: int, warmup: int, options=None, kernel_table: 
         dom_name = kernels[longest_gen[1]]["name"]
         bound = "hbm"
     if kernel_table:
-        for k, ms in sorted(zip(kernels, per), key=lambda x: -x[1])[:60]:
+        for k, ms in sorted(zip(kernels, per), key=lambda x: -x[1]):
             print(f"{ms*1e3:9.1f} us  {k['kind']:9s} {k['name'][:70]:70s} flops={k['flops']:.3g} bytes={k['bytes']:.3g} "
                   f"mnk={k['m']}x{k['n']}x{k['k']}x{k['batch']} coop={k['coop_lanes']}", file=sys.stderr)
 

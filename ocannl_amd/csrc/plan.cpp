@@ -1884,7 +1884,7 @@ void fuse_row_projections(Routine& r, Plan& plan) {
       const GemmOperand& bop = is_y(g.a) ? g.b : g.a;
       if (yop.prec != Prec::Bfloat16 || bop.prec != Prec::Bfloat16) continue;
       if (r.node(bop.node).dims != r.node(bget->node).dims) continue;   // (a bf16 copy has its source's layout)
-      if (!(g.c.prec == Prec::Bfloat16 || g.c.prec == Prec::Single)) continue;
+      if (g.c.prec != Prec::Bfloat16 || g.c_copy >= 0) continue;   // (what the attention blocks produce; fp32 results and copies stay launches)
       // y read through plain iterators, one per axis; those loops run over the group's rows
       std::map<int, std::pair<int64_t, int64_t>> range;   // symbol -> (from, extent)
       for (size_t q = 0; q < P.par_syms.size(); ++q) range[P.par_syms[q]] = {P.par_from[q], P.par_ext[q]};

@@ -303,7 +303,7 @@ def test_contraction_as_row_group_prologue_equals_the_separate_launches(shape):
 
 
 @pytest.mark.parametrize("shape", [dict(b=2, h=4, q=64, k=128, d=32), dict(b=3, h=2, q=96, k=256, d=64), dict(b=2, h=2, q=32, k=512, d=64),
-                                   dict(b=2, h=2, q=64, k=256, d=128)])
+                                   dict(b=2, h=2, q=64, k=256, d=128), dict(b=2, h=2, q=64, k=512, d=128)])
 def test_contraction_as_row_group_epilogue_against_the_separate_launch(shape):
     # attention weights times V (lib/nn_blocks.ml:233-236) runs inside the kernel that produced the
     # weights: the workgroup keeps its 32 finished rows in LDS and multiplies them with V on the matrix
