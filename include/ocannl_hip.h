@@ -129,7 +129,11 @@ int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** code);
    contraction that produces x run in that contraction's epilogue), fused=0|1|2 (a short-K contraction whose only reader is the row-wise
    kernel that follows -- attention scores ahead of the soft-max chain -- runs on the matrix cores as that
    kernel's prologue, into LDS, instead of as a launch of its own; 2: also when its result is a context
-   node that has to be stored anyway), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
+   node that has to be stored anyway), proj=0|1 (a contraction over the row position whose operand such a
+   kernel produces -- attention weights times V -- runs as that kernel's epilogue on the 32 rows the
+   workgroup holds in LDS), row_waves=4|8|16 (waves per workgroup of those kernels), row_vec=0|1 (a lane
+   takes runs of four neighbouring row positions; off), group_window=<n> (how many phases apart
+   contractions may be and still share a launch), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
    indices and offsets in generated kernels, the `large_models` setting of c_syntax.ml:111-112; a
    routine with a node of more than 2^31 - 1 elements gets them without asking). */
 int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, ocannl_hip_code** code);

@@ -947,7 +947,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
         for (size_t k = 0; k < n; ++k) QP *= (uint64_t)(k == (size_t)ma ? q.row_outer_ext[k] / 32 : q.row_outer_ext[k]);
         // 16 waves of two rows each for short rows; long rows keep more of what they produce in
         // registers and take 8 waves of four rows
-        const int NW = q.row_len <= 512 ? 16 : 8, RPW = 32 / NW;
+        const int NW = q.fused_waves, RPW = 32 / NW;
         fused_block = NW * 64;
         body.pop_back(); body.pop_back();   // (lane_ / pt_ as laid out for lane groups: redone per workgroup)
         body.push_back(pind + "const uint32_t lane_ = threadIdx.x & 63u, wave_ = threadIdx.x >> 6;");

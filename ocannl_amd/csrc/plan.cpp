@@ -1712,7 +1712,7 @@ void lift_routine_locals(Routine& r, Plan& plan) {
 // is planner scratch, and its read in either case.
 namespace {
 
-void fuse_row_contractions(Routine& r, Plan& plan, bool also_stored) {
+void fuse_row_contractions(Routine& r, Plan& plan, bool also_stored, int waves) {
   std::map<int, int> mirror_source;
   for (auto& kv : plan.mirrors) mirror_source[kv.second] = kv.first;
   for (size_t j = 0; j < plan.phases.size(); ++j) {
@@ -1816,6 +1816,7 @@ void fuse_row_contractions(Routine& r, Plan& plan, bool also_stored) {
       G.fused_a = F.fused_a; G.fused_b = F.fused_b;
       G.fused_a_stride = F.fused_a_stride; G.fused_b_stride = F.fused_b_stride;
       G.fused_b_row = F.fused_b_row; G.fused_k = F.fused_k; G.fused_m_axis = m_axis;
+      G.fused_waves = waves == 4 || waves == 8 || waves == 16 ? waves : G.row_len <= 512 ? 16 : 8;
       G.flops = P.flops;
       const double x_bytes = (double)xn.size_in_bytes();
       G.bytes += P.bytes - 2.0 * x_bytes + (G.fused_x_store ? x_bytes : 0.0);   // x is neither written (unless stored) nor read
@@ -1943,7 +1944,7 @@ void fuse_row_projections(Routine& r, Plan& plan) {
       // the sum over t is split over the waves that the static LDS budget lets hold a partial result;
       // with fewer than four waves at work the separate launch is faster (measured: 1024-long rows,
       // whose bf16 tile fills the 64 KiB: 2.78 against 2.69 ms for the attention step)
-      const int NW = G.row_len <= 512 ? 16 : 8, NB = (int)(N / 32);
+      const int NW = G.fused_waves, NB = (int)(N / 32);
       int KP = 1;
       while (KP * 2 * NB <= NW && KP < 4 && (G.row_len / 16) % (KP * 2) == 0 &&
              32 * G.row_len * (int64_t)prec_in_bytes(r.node(G.fused_x).prec) + (int64_t)(KP * 2) * 32 * N * 4 <= 60 * 1024) KP *= 2;
@@ -2203,7 +2204,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
   if (opt.enable_mfma && opt.merge_chains) merge_contractions(plan, true);
   if (opt.enable_mfma && opt.group_contractions) merge_contractions(plan, false, opt.group_window);
   if (opt.enable_coop && opt.enable_row_groups) group_rows(r, plan);
-  if (opt.enable_mfma && opt.enable_coop && opt.enable_row_groups && opt.fuse_row_contractions) fuse_row_contractions(r, plan, opt.fuse_stored_rows);
+  if (opt.enable_mfma && opt.enable_coop && opt.enable_row_groups && opt.fuse_row_contractions) fuse_row_contractions(r, plan, opt.fuse_stored_rows, opt.row_tile_waves);
   if (opt.enable_mfma && opt.enable_coop && opt.enable_row_groups && opt.fuse_row_contractions && opt.fuse_row_projections) fuse_row_projections(r, plan);
   if (opt.enable_serial_group) serialise_tiny(r, plan);
   if (opt.enable_coop && opt.enable_parallel_groups) group_independent(r, plan);

@@ -115,6 +115,7 @@ struct Phase {
   int64_t fused_b_row = 0;                            // stride of B along the row position
   int64_t fused_k = 0;                                // contracted extent (unit stride in both operands)
   int fused_m_axis = -1;
+  int fused_waves = 16;                               // waves per workgroup (each takes 32 / fused_waves of the rows)
   // ... and a contraction epilogue (proj_y >= 0; only with a prologue, whose 32-row workgroups it shares):
   // `c[o.., n] = sum_t y[o.., t] * b[.., t, n]`, where y is what a member of the group stores per row
   // position -- attention weights times V, the gradient of the scores times K -- is taken out of the
@@ -171,6 +172,7 @@ struct PlanOptions {
   bool side_queue = true;            // contractions off the critical path run on a second queue beside the rest
   bool fuse_epilogues = true;        // bias / relu consumers of an inlined contraction run in the contraction's epilogue
   bool fuse_row_contractions = true; // a short-K contraction feeding a row group runs as that kernel's prologue ...
+  int row_tile_waves = 0;            // waves per workgroup of those kernels (4, 8 or 16); 0: 16 for rows of at most 512, else 8
   bool fuse_row_projections = true;   // contraction epilogue of a row group with a prologue (see Phase::proj_y)
   bool fuse_stored_rows = false;     // ... also when its result has to be stored anyway (a context node): measured slower
   bool enable_bf16_copies = true;   // keep bf16 copies of fp32 operands of mixed contractions (written by the producing kernels)
