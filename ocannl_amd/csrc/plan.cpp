@@ -1976,20 +1976,35 @@ void fuse_row_projections(Routine& r, Plan& plan) {
 // or rewrites one of its operands waits for it.  Same kernels, same operands, same bits.
 namespace {
 
-void assign_side_queue(Plan& plan) {
+void assign_side_queue(Plan& plan, bool also_generated) {
   std::map<int, int> mirror_source;
   for (auto& kv : plan.mirrors) mirror_source[kv.second] = kv.first;
   auto source_of = [&](int node) { auto m = mirror_source.find(node); return m == mirror_source.end() ? node : m->second; };
-  struct Sets { std::vector<int> outs, ins; };
+  struct Sets { std::vector<int> outs, ins; bool ok = true; };
+  // what a generated phase reads and writes (false: something in it is not tracked per tensor)
+  std::function<bool(const Phase&, Sets&)> generic_sets = [&](const Phase& ph, Sets& s) -> bool {
+    if (!ph.serial_members.empty() || ph.fused_x >= 0 || ph.proj_y >= 0) return false;
+    if (!ph.parallel_members.empty()) { for (auto& m : ph.parallel_members) if (!generic_sets(m, s)) return false; return true; }
+    if (!ph.members.empty()) { for (auto& m : ph.members) if (!generic_sets(m, s)) return false; return true; }
+    std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
+    block_accesses(ph.inner, acc, w, f, d);
+    if (w || f) return false;
+    for (auto& a : acc) (a.write ? s.outs : s.ins).push_back(a.node);
+    return true;
+  };
   auto sets_of = [&](const Phase& ph) {
     Sets s;
-    const GemmDesc& g = ph.gemm;
-    s.outs = {g.c.node}; s.ins = {g.a.node, g.b.node};
-    if (g.c_copy >= 0) s.outs.push_back(g.c_copy);
-    if (g.epi_relu >= 0) s.outs.push_back(g.epi_relu);
-    if (g.epi_bias >= 0) s.ins.push_back(g.epi_bias);
-    for (auto& m : g.group) { s.outs.push_back(m.c.node); if (m.c_copy >= 0) s.outs.push_back(m.c_copy); s.ins.push_back(m.a.node); s.ins.push_back(m.b.node); }
-    for (auto& pr : g.more) { s.ins.push_back(pr.first.node); s.ins.push_back(pr.second.node); }
+    if (ph.kind == Phase::Generic) {
+      s.ok = generic_sets(ph, s);
+    } else {
+      const GemmDesc& g = ph.gemm;
+      s.outs = {g.c.node}; s.ins = {g.a.node, g.b.node};
+      if (g.c_copy >= 0) s.outs.push_back(g.c_copy);
+      if (g.epi_relu >= 0) s.outs.push_back(g.epi_relu);
+      if (g.epi_bias >= 0) s.ins.push_back(g.epi_bias);
+      for (auto& m : g.group) { s.outs.push_back(m.c.node); if (m.c_copy >= 0) s.outs.push_back(m.c_copy); s.ins.push_back(m.a.node); s.ins.push_back(m.b.node); }
+      for (auto& pr : g.more) { s.ins.push_back(pr.first.node); s.ins.push_back(pr.second.node); }
+    }
     for (int o : std::vector<int>(s.outs)) { auto m = plan.mirrors.find(o); if (m != plan.mirrors.end()) s.outs.push_back(m->second); }
     return s;
   };
@@ -1998,14 +2013,20 @@ void assign_side_queue(Plan& plan) {
     for (int i : s.ins) if (phase_writes(later, i) || phase_writes(later, source_of(i))) return true;
     return false;
   };
-  constexpr size_t kMinSlack = 4;   // phases that must lie between the contraction and its first dependant
+  constexpr size_t kMinSlack = 4;   // phases that must lie between the phase and its first dependant
   for (size_t p = 0; p < plan.phases.size(); ++p) {
     Phase& ph = plan.phases[p];
-    if (ph.kind != Phase::Contraction || ph.flops < 4e9) continue;
+    // a contraction of some size, or a generated kernel that moves a few MB (the partial sums of bias and
+    // gain gradients: column sums over all rows, wanted by the optimiser only)
+    const bool contraction = ph.kind == Phase::Contraction && ph.flops >= 4e9;
+    const bool generated = also_generated && ph.kind == Phase::Generic && ph.bytes >= (double)(4 << 20);
+    if (!contraction && !generated) continue;
     const Sets s = sets_of(ph);
+    if (!s.ok) continue;
     size_t q = p + 1;
     while (q < plan.phases.size() && !conflicts(s, plan.phases[q])) ++q;
-    if (q - p > kMinSlack) ph.stream = 1;
+    if (q - p > kMinSlack && q < plan.phases.size()) ph.stream = 1;
+    else if (q - p > kMinSlack && contraction) ph.stream = 1;
   }
   // every phase of the main queue waits for the side-queue phases before it that it conflicts with
   // (side-queue phases among themselves run in order)
@@ -2208,7 +2229,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
   if (opt.enable_mfma && opt.enable_coop && opt.enable_row_groups && opt.fuse_row_contractions && opt.fuse_row_projections) fuse_row_projections(r, plan);
   if (opt.enable_serial_group) serialise_tiny(r, plan);
   if (opt.enable_coop && opt.enable_parallel_groups) group_independent(r, plan);
-  if (opt.enable_mfma && opt.side_queue && r.merge_node < 0) assign_side_queue(plan);
+  if (opt.enable_mfma && opt.side_queue && r.merge_node < 0) assign_side_queue(plan, opt.side_queue_generated);
   return plan;
 }
 

@@ -170,6 +170,7 @@ struct PlanOptions {
   bool use_graphs = false;
   int group_window = 1 << 30;        // contractions share a launch only when at most this many phases apart
   bool side_queue = true;            // contractions off the critical path run on a second queue beside the rest
+  bool side_queue_generated = false;  // ... and generated kernels of a few MB that nothing waits for (side_queue=2): measured, no gain
   bool fuse_epilogues = true;        // bias / relu consumers of an inlined contraction run in the contraction's epilogue
   bool fuse_row_contractions = true; // a short-K contraction feeding a row group runs as that kernel's prologue ...
   int row_tile_waves = 0;            // waves per workgroup of those kernels (4, 8 or 16); 0: 16 for rows of at most 512, else 8

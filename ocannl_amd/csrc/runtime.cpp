@@ -130,7 +130,7 @@ PlanOptions parse_options(const char* options) {
     else if (k == "large_models") o.large_models = v != "0";
     else if (k == "groups") o.group_contractions = v != "0";
     else if (k == "chains") o.merge_chains = v != "0";
-    else if (k == "side_queue") o.side_queue = v != "0";
+    else if (k == "side_queue") { o.side_queue = v != "0"; o.side_queue_generated = v == "2"; }
     else if (k == "debug_log") o.debug_log = v != "0";
     else if (k == "row_vec") o.row_vec4 = v != "0";
     else if (k == "graphs") o.use_graphs = v != "0";
@@ -320,7 +320,7 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0, bool 
     } else if (ph.kind == Phase::Generic) {
       for (size_t i = 0; i < l.idx_syms.size(); ++i) l.idx_vals[i] = (uint64_t)rt.statics[l.idx_syms[i]];
       if (l.merge_slot >= 0) l.ptr_vals[v][l.merge_slot] = merge_base;
-      hip_check(hipModuleLaunchKernel(l.fn, l.grid, l.grid_y, 1, l.block, 1, 1, 0, dev.stream, l.args[v].data(), nullptr),
+      hip_check(hipModuleLaunchKernel(l.fn, l.grid, l.grid_y, 1, l.block, 1, 1, 0, stream, l.args[v].data(), nullptr),
                 "hipModuleLaunchKernel");
     } else {
       const GemmDesc& g = ph.gemm;
@@ -353,15 +353,15 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0, bool 
       // a bracketed contraction is timed without its split-K reduction (a kernel of its own)
       hip_check(launch_gemm(g, a, on_side ? rt.gemm_ws_side : rt.gemm_ws[v], stream, bracket ? rt.profile_events[rt.profile_used + 1] : nullptr),
                 "launch_gemm");
-      if (on_side) {
-        hip_check(hipEventRecord(rt.side_events.at((int)li).second, dev.side_stream), "hipEventRecord");
-        last_side = (int)li;
-      }
+    }
+    if (on_side) {
+      hip_check(hipEventRecord(rt.side_events.at((int)li).second, dev.side_stream), "hipEventRecord");
+      last_side = (int)li;
     }
     if (timed) hip_check(hipEventRecord(rt.timing_events[li + 1], dev.stream), "hipEventRecord");
     if (bracket) {
       if (ph.kind != Phase::Contraction)
-        hip_check(hipEventRecord(rt.profile_events[rt.profile_used + 1], dev.stream), "hipEventRecord");
+        hip_check(hipEventRecord(rt.profile_events[rt.profile_used + 1], stream), "hipEventRecord");
       rt.profile_used += 2;
     }
   }
