@@ -328,3 +328,27 @@ def test_contraction_as_row_group_epilogue_against_the_separate_launch(shape):
     fused.step()
     assert np.array_equal(first, fused.get(w.nodes["out"]))
     fused.close(); apart.close()
+
+
+def test_two_queues_leave_what_one_queue_leaves():
+    # contractions (and, with side_queue=2, generated kernels) that nothing waits for run on the device's
+    # second queue, ordered against the main one by events: same kernels, same operands, so every tensor
+    # has to come out bit for bit as with everything in order on one queue, step after step
+    kw = dict(batch=32, seq=256, d_model=512, heads=8, d_ff=1024, layers=2, vocab=512, prec="bfloat16", grad_prec="single", lr=0.05)
+    w = W.transformer(**kw)
+    runs = {o: HipRun(w.routine, w.init, o) for o in ("side_queue=0", "side_queue=1", "side_queue=2")}
+    assert not any(k["queue"] for k in runs["side_queue=0"].code.kernels())
+    side1 = [k for k in runs["side_queue=1"].code.kernels() if k["queue"] == 1]
+    side2 = [k for k in runs["side_queue=2"].code.kernels() if k["queue"] == 1]
+    assert side1 and all(k["kind"] == "mfma" for k in side1)
+    assert len(side2) > len(side1) and any(k["kind"] == "generated" for k in side2)
+    names = ("loss", "w_q_l0", "w_o_l1", "w_ffn1_l0", "w_ffn2_l1", "w_out", "w_embed", "b_ffn1_l1", "gamma_ln1_l0", "beta_ln2_l1")
+    for step in range(4):
+        for h in runs.values():
+            h.step()
+        for name in names:
+            base = runs["side_queue=0"].get(w.nodes[name])
+            for o in ("side_queue=1", "side_queue=2"):
+                assert np.array_equal(runs[o].get(w.nodes[name]), base), (step, name, o)
+    for h in runs.values():
+        h.close()
