@@ -262,8 +262,9 @@ __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, 
   // Pin the tiles to accumulation registers up to this point: without it the register allocator
   // may move all accumulators of the block into ordinary registers right after the main loop and
   // spill most of them.
-  static_assert(TN == 2 || TN == 4, "tile rows of 2 or 4 tiles");
-  asm volatile("" : "+a"(acc[0]), "+a"(acc[1]));
+  static_assert(TN == 1 || TN == 2 || TN == 4, "tile rows of 1, 2 or 4 tiles");
+  if constexpr (TN == 1) asm volatile("" : "+a"(acc[0]));
+  else asm volatile("" : "+a"(acc[0]), "+a"(acc[1]));
   if constexpr (TN == 4) asm volatile("" : "+a"(acc[2]), "+a"(acc[3]));
   float old[ACC ? TN : 1][16];
   if (ACC) {
@@ -312,8 +313,9 @@ __device__ __forceinline__ void store_tile_row_wide(f32x16 (&acc)[TN], float* st
                                                     void* origin2 = nullptr, const unsigned short* bias = nullptr,
                                                     unsigned short* relu_out = nullptr) {
   constexpr int CW = TN * 32, LS = CW + 4;
-  static_assert(TN == 2 || TN == 4, "tile rows of 2 or 4 tiles");
-  asm volatile("" : "+a"(acc[0]), "+a"(acc[1]));
+  static_assert(TN == 1 || TN == 2 || TN == 4, "tile rows of 1, 2 or 4 tiles");
+  if constexpr (TN == 1) asm volatile("" : "+a"(acc[0]));
+  else asm volatile("" : "+a"(acc[0]), "+a"(acc[1]));
   if constexpr (TN == 4) asm volatile("" : "+a"(acc[2]), "+a"(acc[3]));
   float* const wr = stage + ((lane >> 5) * 4) * LS + (lane & 31);
   static_for<TN>([&](auto jc) OCN_LAMBDA_INLINE {
@@ -848,7 +850,7 @@ long batch_count(const GemmDesc& d) {
 // runs 128x128 tiles, two workgroups per CU, and when those are fewer than 256 K is split
 // towards ~512 workgroups (~256 for bf16 sources), never below 8 K stages per split.  Splits are summed in index order by
 // splitk_reduce_kernel (deterministic).
-struct TileConfig { bool big; int splits; int prefetch; };
+struct TileConfig { bool big; int splits; int prefetch; bool narrow = false; };
 
 TileConfig tile_config(const GemmDesc& d) {
   const long nb = batch_count(d);
@@ -872,8 +874,13 @@ TileConfig tile_config(const GemmDesc& d) {
   // each runs at least 8 K stages (measured: 8192x512x2048 bf16 595 -> 738 TFLOP/s)
   c.prefetch = (!c.big && bf16_sources && t128 * c.splits <= 256 && d.K / c.splits >= 512) ? 2 : 1;
   if (!d.more.empty()) c.prefetch = 2;   // the only variant built for chains
+  // results of at most 64 columns (the attention products against V, K, Q: N = head size) take a
+  // 128 x 64 tile: with 128 columns half of every tile would be masked and the launch would run the
+  // checked loop for ragged tiles
+  c.narrow = !c.big && bf16_sources && d.more.empty() && d.N <= 64 && d.N > 16;
   return c;
 }
+bool narrow_tile(const GemmDesc& d) { return tile_config(d).narrow; }
 
 bool big_tile(const GemmDesc& d) { return tile_config(d).big; }
 int split_count(const GemmDesc& d) { return tile_config(d).splits; }
@@ -932,12 +939,12 @@ const char* gemm_kernel_name(const GemmDesc& d) {
   // the instantiation as a profiler prints it (without namespaces)
   static thread_local char buf[128];
   const bool af = d.a.prec == Prec::Single, bf = d.b.prec == Prec::Single;
-  const int tile = big_tile(d) ? 256 : 128;
+  const int tile = big_tile(d) ? 256 : 128, tile_n = narrow_tile(d) ? 64 : tile;
   const char* tf[2] = {"false", "true"};
   if (af && bf)
     snprintf(buf, sizeof buf, "gemm_f32_kernel<%d, %d, %s, %s>", tile, tile, tf[a_kcontig(d)], tf[b_kcontig(d)]);
   else
-    snprintf(buf, sizeof buf, "gemm_bf16_kernel<%d, %d, %s, %s, %s, %s, %d, %s>", tile, tile, af ? "float" : "unsigned short",
+    snprintf(buf, sizeof buf, "gemm_bf16_kernel<%d, %d, %s, %s, %s, %s, %d, %s>", tile, tile_n, af ? "float" : "unsigned short",
              bf ? "float" : "unsigned short", tf[a_kcontig(d)], tf[b_kcontig(d)], prefetch_depth(d), tf[!d.more.empty()]);
   return buf;
 }
@@ -956,8 +963,8 @@ hipError_t launch_gemm(const GemmDesc& d, const GemmArgs& a_in, void* workspace,
   {
     // XCD partition: every A panel is read by each of the xcd_n rectangle columns, every B panel
     // by each of the xcd_m rows
-    const long tile = big ? 256 : 128;
-    const long tiles_m = (d.M + tile - 1) / tile, tiles_n = (d.N + tile - 1) / tile;
+    const long tile = big ? 256 : 128, tile_n = narrow_tile(d) ? 64 : tile;
+    const long tiles_m = (d.M + tile - 1) / tile, tiles_n = (d.N + tile_n - 1) / tile_n;
     const double a_bytes = (double)d.M * prec_in_bytes(d.a.prec), b_bytes = (double)d.N * prec_in_bytes(d.b.prec);
     // a grouped launch of 2 or 4 unbatched members without a K split: each member on 4 or 2 XCDs of
     // its own, so that its panels are fetched into that many L2 caches instead of all eight
@@ -983,6 +990,9 @@ hipError_t launch_gemm(const GemmDesc& d, const GemmArgs& a_in, void* workspace,
   if (!af && !bf) {
     if (a.npairs > 1) return launch_bf16_layout<128, 128, unsigned short, unsigned short, 2, true>(akc, bkc, a, s, ev);
     if (big) return launch_bf16_layout<256, 256, unsigned short, unsigned short>(akc, bkc, a, s, ev);
+    if (narrow_tile(d))
+      return prefetch_depth(d) == 2 ? launch_bf16_layout<128, 64, unsigned short, unsigned short, 2>(akc, bkc, a, s, ev)
+                                    : launch_bf16_layout<128, 64, unsigned short, unsigned short>(akc, bkc, a, s, ev);
     return prefetch_depth(d) == 2 ? launch_bf16_layout<128, 128, unsigned short, unsigned short, 2>(akc, bkc, a, s, ev)
                                   : launch_bf16_layout<128, 128, unsigned short, unsigned short>(akc, bkc, a, s, ev);
   }
