@@ -169,7 +169,10 @@ struct PlanOptions {
   // the transformer step 3.68 -> 3.73 ms.
   bool use_graphs = false;
   int group_window = 1 << 30;        // contractions share a launch only when at most this many phases apart
-  bool side_queue = true;            // contractions off the critical path run on a second queue beside the rest
+  // contractions off the critical path run on a second queue beside the rest (side_queue=1).  Off:
+  // measured on the transformer step it gains 0.9 % (3.528 -> 3.495 ms), less than the step varies from
+  // box to box, and every per-kernel duration (profilers, event brackets) becomes a time on a shared chip
+  bool side_queue = false;
   bool side_queue_generated = false;  // ... and generated kernels of a few MB that nothing waits for (side_queue=2): measured, no gain
   bool fuse_epilogues = true;        // bias / relu consumers of an inlined contraction run in the contraction's epilogue
   bool fuse_row_contractions = true; // a short-K contraction feeding a row group runs as that kernel's prologue ...

@@ -41,9 +41,9 @@ def test_char_mlp_adam_steps_replayed():
 def test_transformer_steps_with_fills_side_queue_and_split_k_replayed():
     kw = dict(batch=8, seq=128, d_model=256, heads=4, d_ff=512, layers=2, vocab=512, prec="bfloat16", grad_prec="single", lr=0.05)
     w = W.transformer(**kw)
-    ks = B.compile(w.routine).kernels()
+    ks = B.compile(w.routine, "side_queue=1").kernels()
     assert any(k["kind"] == "mfma" for k in ks)
-    _same_after_every_step(w, 5, lambda s: None, ("loss", "w_q_l0", "w_ffn2_l1", "w_out", "b_ffn1_l0", "beta_ln2_l1"))
+    _same_after_every_step(w, 5, lambda s: None, ("loss", "w_q_l0", "w_ffn2_l1", "w_out", "b_ffn1_l0", "beta_ln2_l1"), "side_queue=1")
 
 
 def test_attention_replayed_and_bad_static_index_still_refused():
