@@ -125,7 +125,7 @@ int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** code);
    by ocannl_hip_routine_run; off by default), debug_log=0|1 (in-routine logging, see
    ocannl_hip_routine_log_id; the wire form then carries every Set's text), side_queue=0|1|2 (contractions
    whose results nothing needs for a while -- weight gradients -- run on a second queue of the device, beside
-   the kernels that follow; 2: generated kernels of a few MB as well), epilogues=0|1 (`y := x + bias` and `z := relu(y)` right behind the
+   the kernels that follow; 2: generated kernels of a few MB as well; off by default), epilogues=0|1 (`y := x + bias` and `z := relu(y)` right behind the
    contraction that produces x run in that contraction's epilogue), fused=0|1|2 (a short-K contraction whose only reader is the row-wise
    kernel that follows -- attention scores ahead of the soft-max chain -- runs on the matrix cores as that
    kernel's prologue, into LDS, instead of as a launch of its own; 2: also when its result is a context
