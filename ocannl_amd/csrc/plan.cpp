@@ -1081,7 +1081,12 @@ void group_rows(const Routine& r, Plan& plan) {
     // such a group was measured slower than its members as separate, overlapping launches)
     if (shape.len < 0 && shape.outer.empty() && run.size() >= 2) shape.len = 1;   // scalars only
     const int64_t points = rows * std::max<int64_t>(shape.len, 1);
-    if (run.size() >= 2 && shape.len >= 1 && ((shape.len >= 16 && points >= (1 << 16)) || (launch_bound && points < 8192))) {
+    // ... or be a chain of tiny phases over the same few points (the steps between the loss and the
+    // gradient of the logits: 8192 points, 6 us of launch latency each, four launches less in the
+    // transformer step)
+    bool tiny_chain = run.size() >= 2 && points <= 16384;
+    for (auto& m : run) tiny_chain = tiny_chain && m.bytes <= (double)(1 << 20);
+    if (run.size() >= 2 && shape.len >= 1 && ((shape.len >= 16 && points >= (1 << 16)) || (launch_bound && points < 8192) || tiny_chain)) {
       Phase g;
       g.kind = Phase::Generic;
       g.label = run.front().label + " .. " + run.back().label;
