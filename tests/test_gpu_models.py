@@ -73,6 +73,23 @@ def test_attention_fwd_bwd(prec, tol, opts):
     hip.close()
 
 
+@pytest.mark.parametrize("shape", [dict(b=2, h=4, q=64, k=128, d=32), dict(b=3, h=2, q=96, k=256, d=64)])
+def test_attention_with_matrix_core_prologue_and_epilogue_against_the_checker(shape):
+    # rows of 128 / 256 scores: Q K^T runs as the prologue and the product with V as the epilogue of the
+    # soft-max kernel (one kernel for the whole forward pass); judged like every bf16 routine against
+    # the checker in single precision on the same, exactly widened inputs
+    w = W.attention(prec="bfloat16", grad_prec="single", **shape)
+    wr = W.attention(prec="single", grad_prec="single", **shape)
+    hip, ora = HipRun(w.routine, w.init, "min_mfma_flops=1"), OracleRun(wr.routine, _widened_init(w, wr))
+    src = hip.code.source().split("extern \"C\"", 1)[1]
+    assert "ocn_rowtile_contract<" in src and "ocn_rowtile_project<" in src
+    hip.step(); ora.step()
+    for name, p in (("out", "bfloat16"), ("attn", "bfloat16"), ("dq", "single"), ("dk", "single"), ("dv", "single")):
+        got = W.to_float(hip.get(w.nodes[name]), p)
+        assert _err(got, ora.get(wr.nodes[name]), "bfloat16") <= 2e-2, name
+    hip.close()
+
+
 @pytest.mark.parametrize("prec,tol,steps", [("single", 1e-4, 5), ("bfloat16", 2e-2, 3)])
 def test_transformer_step(prec, tol, steps):
     kw = dict(batch=2, seq=16, d_model=32, heads=2, d_ff=64, layers=2, vocab=64, grad_prec="single", lr=0.05)
