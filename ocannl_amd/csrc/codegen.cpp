@@ -174,6 +174,10 @@ bool via_float(Prec p, std::string* to_f, std::string* from_f) {
 
 std::string emit_ternop(Prec prec, Ternop op, const std::string& a, const std::string& b, const std::string& c) {
   std::string tf, ff;
+  // bf16 `where`: the result is one of two bf16 values, and rounding a widened bf16 value gives it back
+  // (its low 16 bits are zero: the rounding increment cannot carry), so the choice is made on the bits
+  // (the condition is widened as the reference writes it, cc_backend.ml:169-186)
+  if (op == Ternop::Where && prec == Prec::Bfloat16) return "((bfloat16_to_single(" + a + ")) != 0.0 ? (" + b + ") : (" + c + "))";
   if (via_float(prec, &tf, &ff)) {
     Syn4 s = ternop_syntax(Prec::Single, op);
     return ff + s.p + tf + a + ")" + s.i1 + " " + tf + b + ")" + s.i2 + " " + tf + c + ")" + s.s + ")";
