@@ -18,7 +18,9 @@ inlined.  This module restates just enough of it:
   docs/migration_guide.md:639-652;
 * inlining of nodes that are computed once and read once per cell (the effect of
   ``virtualize_max_visits = 1``, arrayjit/lib/low_level.ml:535-571,1165-1316), producing the
-  ``Local_scope`` reductions seen in test/einsum/inline_permuted_view-c_fwd.ll.expected;
+  ``Local_scope`` reductions seen in test/einsum/inline_permuted_view-c_fwd.ll.expected; an opt-in
+  mode (``inline="visits"``) also treats reads at the position being assigned as free, as the
+  reference's visit count does (low_level.ml:496-552);
 * memory modes: parameters, inputs and outputs in context; other nodes ``local`` when at most
   ``stack_threshold_in_bytes`` = 16384 bytes, else in context (arrayjit/lib/tnode.ml:152-171).
 
@@ -90,6 +92,7 @@ class Graph:
         g = self.node(ident + "_grad", dims, self.grad_prec)
         v._is_param = True
         g._is_grad = True
+        g._is_param_grad = True
         return T(v, tuple(axes), g, label=ident)
 
     def input(self, ident: str, axes: Sequence[str], dims: Sequence[int], prec: Optional[str] = None) -> T:
@@ -526,9 +529,16 @@ def _perfect_nest(stmt: L.Stmt):
     return loops, [cur]
 
 
-def inline_single_use(g: Graph, body: List[L.Stmt], keep: Sequence[L.Node] = ()) -> List[L.Stmt]:
+def inline_single_use(g: Graph, body: List[L.Stmt], keep: Sequence[L.Node] = (), visits: bool = False) -> List[L.Stmt]:
     """Inline every local/intermediate node that is defined by one statement group and read
-    exactly once, by a statement whose loops all index that read (one visit per cell)."""
+    exactly once, by a statement whose loops all index that read (one visit per cell).
+
+    ``visits=True`` follows the reference's visit count more closely (arrayjit/lib/low_level.ml:496-552
+    with ``virtualize_max_visits`` = 1): a read at the very position being assigned is not a visit, so a
+    tensor computed once per cell by a pointwise statement is inlined into ANY number of such readers
+    (and recomputed there), plus at most one reader that visits every cell once; and a gradient that is
+    zeroed and then accumulated into by a single pointwise statement counts as computed once (the
+    gradients of parameters stay in memory: the optimiser's routine reads them)."""
     keep_ids = {n.id for n in keep} | set(g.forced_ctx)
     body = list(body)
     changed = True
@@ -545,13 +555,16 @@ def inline_single_use(g: Graph, body: List[L.Stmt], keep: Sequence[L.Node] = ())
                         writes.setdefault(w.id, []).append(i)
         for nid, idxs in writes.items():
             node = _node_at(body, idxs[0], nid)
-            if node is None or nid in keep_ids or getattr(node, "_is_param", False) or getattr(node, "_is_grad", False):
+            if node is None or nid in keep_ids or getattr(node, "_is_param", False):
+                continue
+            if getattr(node, "_is_grad", False) and (not visits or getattr(node, "_is_param_grad", False)):
                 continue
             idxs = sorted(set(idxs))
             # definition group: [Set nest] or [ZeroOut/neutral-fill, accumulate nest], contiguous
+            # (visits: the zero fill may stand anywhere ahead, as zero_grads puts it)
             if len(idxs) == 1:
                 def_i, fill_i = idxs[0], None
-            elif len(idxs) == 2 and idxs[1] == idxs[0] + 1:
+            elif len(idxs) == 2 and (idxs[1] == idxs[0] + 1 or (visits and isinstance(body[idxs[0]], L.ZeroOut))):
                 fill_i, def_i = idxs
             else:
                 continue
@@ -563,9 +576,10 @@ def inline_single_use(g: Graph, body: List[L.Stmt], keep: Sequence[L.Node] = ())
                 continue
             if fill_i is not None and not _is_neutral_fill(body[fill_i], node):
                 continue
-            if _count_gets(body[def_i + 1:], node) != 1:
+            uses = [i for i in range(def_i + 1, len(body)) if _count_gets([body[i]], node)]
+            if not uses or (not visits and _count_gets(body[def_i + 1:], node) != 1):
                 continue
-            use_i = next(i for i in range(def_i + 1, len(body)) if _count_gets([body[i]], node) == 1)
+            use_i = uses[-1]
             if not _inputs_unchanged(body, def_i, use_i, dset):
                 continue
             # the definition's lhs axes must be distinct plain iterators (or Fixed 0)
@@ -581,16 +595,38 @@ def inline_single_use(g: Graph, body: List[L.Stmt], keep: Sequence[L.Node] = ())
             red = [(s, f, t) for (s, f, t) in loops if s not in par]
             if not ok or (fill_i is None and red):
                 continue
-            new_use = _inline_into(g, body[use_i], node, dset, par, red, fill_i is not None)
-            if new_use is None:
+            if len(uses) == 1 and _count_gets([body[use_i]], node) == 1:
+                new_uses = {use_i: _inline_into(g, body[use_i], node, dset, par, red, fill_i is not None)}
+            else:
+                # several reads: only a pointwise definition, every read but one at the position being assigned
+                if red:
+                    continue
+                # (the one reader that visits every cell once is given up when the definition itself holds an
+                # inlined reduction: nested into a second reduction it would be recomputed per addend)
+                budget = {"visits": 0 if _has_local_scope(dset.value) else 1}
+                new_uses = {u: _inline_into(g, body[u], node, dset, par, red, fill_i is not None, budget) for u in uses}
+            if any(v is None for v in new_uses.values()):
                 continue
-            body[use_i] = new_use
+            for u, v in new_uses.items():
+                body[u] = v
             for i in sorted([x for x in (def_i, fill_i) if x is not None], reverse=True):
                 del body[i]
             node.mode = "virtual"
             changed = True
             break
     return body
+
+
+def _has_local_scope(s: L.Scalar) -> bool:
+    if isinstance(s, L.LocalScope):
+        return True
+    if isinstance(s, L.Unop):
+        return _has_local_scope(s.arg)
+    if isinstance(s, L.Binop):
+        return _has_local_scope(s.a) or _has_local_scope(s.b)
+    if isinstance(s, L.Ternop):
+        return _has_local_scope(s.a) or _has_local_scope(s.b) or _has_local_scope(s.c)
+    return False
 
 
 def _written_nodes(stmts) -> List[L.Node]:
@@ -657,8 +693,11 @@ def _inputs_unchanged(body, def_i, use_i, dset) -> bool:
     return True
 
 
-def _inline_into(g: Graph, use_stmt, node, dset, par, red, is_reduction):
-    """Rewrite the single ``Get node`` inside ``use_stmt``; None if the read is not one-visit."""
+def _inline_into(g: Graph, use_stmt, node, dset, par, red, is_reduction, budget=None):
+    """Rewrite the single ``Get node`` inside ``use_stmt``; None if the read is not one-visit.
+    With ``budget`` (a dict holding the visits still allowed, shared over all statements that read the
+    node): rewrite every read; a read at the position the statement assigns is free, any other has to
+    be one-visit and takes one from the budget."""
     found = {"n": 0}
 
     def enclosing_ok(get: L.Get, loop_syms: List[int]) -> bool:
@@ -689,18 +728,32 @@ def _inline_into(g: Graph, use_stmt, node, dset, par, red, is_reduction):
             neutral = float("-inf") if dset.value.op == "max" else float("inf")
         return L.LocalScope(sc, [L.SetLocal(sc, L.Const(neutral))] + inner)
 
-    def sc_rw(s, loop_syms):
+    def wrap(get: L.Get, lhs):
+        v = build(get)
+        # a value of another precision than the statement it lands in is still rounded to its own first
+        if budget is not None and lhs is not None and lhs.node.prec != node.prec and not isinstance(v, L.LocalScope):
+            sc = g.scope(node)
+            return L.LocalScope(sc, [L.SetLocal(sc, v)])
+        return v
+
+    def sc_rw(s, loop_syms, lhs=None):
         if isinstance(s, L.Get) and s.node is node:
-            if not enclosing_ok(s, loop_syms):
-                raise _NoInline()
+            positional = budget is not None and lhs is not None and tuple(s.idcs) == tuple(lhs.idcs)
+            if not positional:
+                if not enclosing_ok(s, loop_syms):
+                    raise _NoInline()
+                if budget is not None:
+                    if budget["visits"] <= 0:
+                        raise _NoInline()
+                    budget["visits"] -= 1
             found["n"] += 1
-            return build(s)
+            return wrap(s, lhs)
         if isinstance(s, L.Unop):
-            return L.Unop(s.op, sc_rw(s.arg, loop_syms), s.arg_prec)
+            return L.Unop(s.op, sc_rw(s.arg, loop_syms, lhs), s.arg_prec)
         if isinstance(s, L.Binop):
-            return L.Binop(s.op, sc_rw(s.a, loop_syms), sc_rw(s.b, loop_syms))
+            return L.Binop(s.op, sc_rw(s.a, loop_syms, lhs), sc_rw(s.b, loop_syms, lhs))
         if isinstance(s, L.Ternop):
-            return L.Ternop(s.op, sc_rw(s.a, loop_syms), sc_rw(s.b, loop_syms), sc_rw(s.c, loop_syms), s.a_prec)
+            return L.Ternop(s.op, sc_rw(s.a, loop_syms, lhs), sc_rw(s.b, loop_syms, lhs), sc_rw(s.c, loop_syms, lhs), s.a_prec)
         if isinstance(s, L.LocalScope):
             if _count_gets(s.body, node):
                 raise _NoInline()
@@ -711,15 +764,19 @@ def _inline_into(g: Graph, use_stmt, node, dset, par, red, is_reduction):
         if isinstance(c, L.For):
             return L.For(c.sym, c.from_, c.to, [st_rw(x, loop_syms + [c.sym]) for x in c.body])
         if isinstance(c, L.Set):
-            return L.Set(c.node, c.idcs, sc_rw(c.value, loop_syms))
+            return L.Set(c.node, c.idcs, sc_rw(c.value, loop_syms, c))
         if isinstance(c, L.SetLocal):
             return L.SetLocal(c.scope, sc_rw(c.value, loop_syms))
+        if isinstance(c, L.SetFromVec) and _count_gets([c], node):
+            raise _NoInline()
         return c
 
     try:
         new = st_rw(use_stmt, [])
     except _NoInline:
         return None
+    if budget is not None:
+        return new if found["n"] >= 1 else None
     return new if found["n"] == 1 else None
 
 
@@ -734,7 +791,7 @@ def make_routine(g: Graph, name: str, body: List[L.Stmt], statics: Sequence[L.St
     for n in outputs:
         n.mode = "ctx"
     if inline:
-        body = inline_single_use(g, body, keep=outputs)
+        body = inline_single_use(g, body, keep=outputs, visits=inline == "visits")
     return L.Routine(name, body, list(statics))
 
 

@@ -369,3 +369,17 @@ def test_two_queues_leave_what_one_queue_leaves():
                 assert np.array_equal(runs[o].get(w.nodes[name]), base), (step, name, o)
     for h in runs.values():
         h.close()
+
+
+def test_routine_inlined_by_the_visit_rule_against_the_checker():
+    # the harness's opt-in inlining mode (reads at the assigned position are free: more tensors inlined,
+    # deeper expressions, inlined gradients) produces another routine for the same step; device and
+    # checker have to agree on it as on the default one
+    kw = dict(batch=2, seq=16, d_model=32, heads=2, d_ff=64, layers=2, vocab=64, prec="single", grad_prec="single", lr=0.05)
+    w = W.transformer(inline="visits", **kw)
+    hip, ora = HipRun(w.routine, w.init, "min_mfma_flops=100000"), OracleRun(w.routine, w.init)
+    for _ in range(3):
+        hip.step(); ora.step()
+    for name in ("loss", "w_q_l0", "w_o_l1", "w_ffn1_l0", "w_ffn2_l1", "w_out", "w_embed", "pos_encoding", "gamma_ln1_l0", "beta_ln2_l1", "b_ffn1_l0"):
+        assert rel_err(hip.get(w.nodes[name]), ora.get(w.nodes[name]), "single") <= 1e-4, name
+    hip.close()
