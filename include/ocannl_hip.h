@@ -67,7 +67,8 @@ typedef struct {
                               one result as a longer k                                                 */
   char name[96];
   int32_t queue;           /* 0 = the device's main queue; 1 = its side queue: a contraction off the critical
-                              path that runs beside the kernels that follow it (compile option side_queue=0|1) */
+                              path that runs beside the kernels that follow it (compile option side_queue=1|2;
+                              without it every kernel reports 0) */
   int32_t reserved;
 } ocannl_hip_kernel_info;
 
