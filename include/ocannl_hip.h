@@ -83,6 +83,11 @@ int ocannl_hip_get_name(ocannl_hip_device* dev, char* buf, size_t cap);  /* Devi
 int ocannl_hip_static_properties(char* buf, size_t cap);   /* static_properties sexp, :231; cuda_backend.ml:1092-1112 */
 int ocannl_hip_get_used_memory(ocannl_hip_device* dev, uint64_t* bytes); /* get_used_memory, :239 */
 int ocannl_hip_get_debug_info(ocannl_hip_device* dev, char* buf, size_t cap); /* get_debug_info, :244 */
+/* get_global_debug_info (backend_intf.ml:242; the CUDA backend's reports its live streams,
+   cuda_backend.ml:1088-1090): a sexp of process-wide counters -- live devices (one stream each), events,
+   compiled codes, linked routines, routines compiled, hiprtc modules built, routines rebuilt without
+   16-byte accesses for a context at element-aligned offsets, runs enqueued, pools and their bytes. */
+int ocannl_hip_get_global_debug_info(char* buf, size_t cap);
 int ocannl_hip_await(ocannl_hip_device* dev);                            /* await, :247          */
 int ocannl_hip_is_idle(ocannl_hip_device* dev, int* idle);               /* is_idle, :254        */
 
@@ -147,12 +152,21 @@ int ocannl_hip_code_routine_name(ocannl_hip_code* code, int index, char* buf, si
 int ocannl_hip_code_kparams(ocannl_hip_code* code, int index, ocannl_hip_kparam* params, int cap, int* count);
 /* Generated HIP source (the `.hip` dump under output_debug_files_in_build_directory). */
 int ocannl_hip_code_source(ocannl_hip_code* code, char* buf, size_t cap, size_t* needed);
+/* The gfx950 code object hiprtc built for routine `index` (its generated kernels; empty for a routine
+   made of matrix-core launches and fills only): the `.ptx` dump of cuda_backend.ml:193-202 under
+   output_debug_files_in_build_directory.  An ELF file: `llvm-objdump -d` prints its ISA.  Pass
+   buf = NULL to query the size. */
+int ocannl_hip_code_object(ocannl_hip_code* code, int index, char* buf, size_t cap, size_t* needed);
 int ocannl_hip_code_num_kernels(ocannl_hip_code* code, int index, int* n);
 int ocannl_hip_code_kernel_info(ocannl_hip_code* code, int index, int kernel, ocannl_hip_kernel_info* info);
 
 /* Lowered_backend.link (backend_impl.ml:355; cuda_backend.ml:983-1066): loads the module on `dev`,
    resolves every Kparam_ptr through `locs` (the resulting context's ctx_buffers), allocates the
-   routine-private scratch for `Local` nodes.  Missing nodes raise E_USER (cc_backend.ml:411-415). */
+   routine-private scratch for `Local` nodes.  Missing nodes raise E_USER (cc_backend.ml:411-415).
+   Offsets need only be aligned to the node's element size, as Backends.plan_pool_segments packs them
+   (arrayjit/lib/backends.ml:22-51): when an operand of a matrix-core kernel sits at an offset that is
+   not 16-byte aligned, the routine is linked in a second form, built on first need, in which
+   generated kernels do that work element by element (slower; same results within tolerance). */
 int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, const ocannl_hip_node_loc* locs,
                     int n_locs, ocannl_hip_routine** routine);
 void ocannl_hip_routine_free(ocannl_hip_routine* routine);

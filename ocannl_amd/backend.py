@@ -68,12 +68,12 @@ class KernelInfo(ctypes.Structure):
 EXPORTS = (
     "ocannl_hip_last_error", "ocannl_hip_init", "ocannl_hip_num_devices", "ocannl_hip_get_device",
     "ocannl_hip_get_name", "ocannl_hip_static_properties", "ocannl_hip_get_used_memory",
-    "ocannl_hip_get_debug_info", "ocannl_hip_await", "ocannl_hip_is_idle", "ocannl_hip_all_work",
+    "ocannl_hip_get_debug_info", "ocannl_hip_get_global_debug_info", "ocannl_hip_await", "ocannl_hip_is_idle", "ocannl_hip_all_work",
     "ocannl_hip_sync", "ocannl_hip_is_done", "ocannl_hip_will_wait_for", "ocannl_hip_event_free",
     "ocannl_hip_alloc_pool", "ocannl_hip_free_pool", "ocannl_hip_memset_zero", "ocannl_hip_from_host",
     "ocannl_hip_to_host", "ocannl_hip_device_to_device", "ocannl_hip_compile",
     "ocannl_hip_compile_opts", "ocannl_hip_code_free", "ocannl_hip_code_num_routines",
-    "ocannl_hip_code_routine_name", "ocannl_hip_code_kparams", "ocannl_hip_code_source",
+    "ocannl_hip_code_routine_name", "ocannl_hip_code_kparams", "ocannl_hip_code_source", "ocannl_hip_code_object",
     "ocannl_hip_code_num_kernels", "ocannl_hip_code_kernel_info", "ocannl_hip_link",
     "ocannl_hip_routine_free", "ocannl_hip_routine_set_static", "ocannl_hip_routine_run",
     "ocannl_hip_routine_run_static_scratch", "ocannl_hip_routine_log_id", "ocannl_hip_routine_run_timed",
@@ -103,6 +103,7 @@ def load_library() -> ctypes.CDLL:
         "ocannl_hip_static_properties": (i32, [ctypes.c_char_p, sz]),
         "ocannl_hip_get_used_memory": (i32, [vp, P(u64)]),
         "ocannl_hip_get_debug_info": (i32, [vp, ctypes.c_char_p, sz]),
+        "ocannl_hip_get_global_debug_info": (i32, [ctypes.c_char_p, sz]),
         "ocannl_hip_await": (i32, [vp]),
         "ocannl_hip_is_idle": (i32, [vp, P(i32)]),
         "ocannl_hip_all_work": (i32, [vp, P(vp)]),
@@ -123,6 +124,7 @@ def load_library() -> ctypes.CDLL:
         "ocannl_hip_code_routine_name": (i32, [vp, i32, ctypes.c_char_p, sz]),
         "ocannl_hip_code_kparams": (i32, [vp, i32, P(_Kparam), i32, P(i32)]),
         "ocannl_hip_code_source": (i32, [vp, ctypes.c_char_p, sz, P(sz)]),
+        "ocannl_hip_code_object": (i32, [vp, i32, ctypes.c_char_p, sz, P(sz)]),
         "ocannl_hip_code_num_kernels": (i32, [vp, i32, P(i32)]),
         "ocannl_hip_code_kernel_info": (i32, [vp, i32, i32, P(KernelInfo)]),
         "ocannl_hip_link": (i32, [vp, vp, i32, P(_NodeLoc), i32, P(vp)]),
@@ -213,6 +215,13 @@ def get_debug_info(dev: Device) -> str:
     return buf.value.decode()
 
 
+def get_global_debug_info() -> str:
+    """``get_global_debug_info`` (backend_intf.ml:242; cuda_backend.ml:1088-1090): process-wide counters."""
+    buf = ctypes.create_string_buffer(4096)
+    _check(load_library().ocannl_hip_get_global_debug_info(buf, 4096))
+    return buf.value.decode()
+
+
 def await_(dev: Device) -> None:
     _check(load_library().ocannl_hip_await(dev._h))
 
@@ -296,6 +305,15 @@ class Code:
         _check(load_library().ocannl_hip_code_source(self._h, buf, need.value, None))
         return buf.value.decode()
 
+    def code_object(self, index: int = 0) -> bytes:
+        """The gfx950 code object of the routine's generated kernels (the ``.ptx`` dump of
+        cuda_backend.ml:193-202 under ``output_debug_files_in_build_directory``)."""
+        need = ctypes.c_size_t()
+        _check(load_library().ocannl_hip_code_object(self._h, index, None, 0, ctypes.byref(need)))
+        buf = ctypes.create_string_buffer(max(need.value, 1))
+        _check(load_library().ocannl_hip_code_object(self._h, index, buf, need.value, None))
+        return buf.raw[:need.value]
+
     def kernels(self, index: int = 0) -> List[dict]:
         n = ctypes.c_int()
         _check(load_library().ocannl_hip_code_num_kernels(self._h, index, ctypes.byref(n)))
@@ -323,7 +341,9 @@ def compile(routine: L.Routine, options: Optional[str] = None) -> Code:  # noqa:
 def compile_batch(routines: Sequence[L.Routine], options: Optional[str] = None) -> Code:
     """``Lowered_backend.compile_batch`` (backend_impl.ml:349-353)."""
     # with debug_log=1 every Set carries its text, as Low_level.Set's `debug` field does
-    debug = options is not None and "debug_log=1" in options.replace(" ", "")
+    # (the option is read as the library reads it: any value but "0" switches logging on)
+    debug = any(kv.split("=", 1)[0].strip() == "debug_log" and kv.split("=", 1)[1].strip() != "0"
+                for kv in (options or "").split(";") if "=" in kv)
     text = "".join(L.to_wire(r, debug=debug) for r in routines).encode()
     h = ctypes.c_void_p()
     lib = load_library()

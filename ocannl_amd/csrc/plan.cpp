@@ -1811,6 +1811,11 @@ void fuse_row_contractions(Routine& r, Plan& plan, bool also_stored, int waves) 
                        !phase_writes(mid, source_of(g.a.node)) && !phase_writes(mid, source_of(g.b.node));
       }
       if (!free_to_move) continue;
+      // ... nor may the group itself: a member's stores in one workgroup would race with another
+      // workgroup's prologue loads, which a kernel boundary used to order
+      if (phase_writes(G, g.a.node) || phase_writes(G, g.b.node) || phase_writes(G, source_of(g.a.node)) ||
+          phase_writes(G, source_of(g.b.node)))
+        continue;
       bool later_reader = false;
       for (size_t q = j + 1; q < plan.phases.size(); ++q) later_reader = later_reader || phase_touches(plan.phases[q], X);
       // When the rows have to be stored anyway the separate launches were measured faster (the

@@ -2,6 +2,7 @@
 // and launching.  Mirrors the responsibilities of the reference CUDA backend
 // (arrayjit/lib/cuda_backend.ml) without sharing its structure: one HIP stream per device, slabs
 // from hipMalloc, kernels from hiprtc modules plus the precompiled MFMA kernels of this library.
+#include <atomic>
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
@@ -38,10 +39,19 @@ void hip_check(hipError_t e, const char* what) {
 constexpr uint64_t kStaticScratchBytes = OCANNL_HIP_STATIC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
-// Zero fill as a kernel (16-byte stores), for the path that callers may record into a HIP graph.
-__global__ void __launch_bounds__(256) fill_zero_kernel(uint4* p, uint64_t n16) {
+// Zero fill as a kernel, for the path that callers may record into a HIP graph.  Exactly `bytes`
+// bytes from `p` are cleared, wherever they start: a context node is packed at an offset aligned to
+// its element size only and is followed by its neighbour in the pool, so the unaligned head and tail
+// go out as single bytes and only the 16-byte aligned body as 16-byte stores.
+__global__ void __launch_bounds__(256) fill_zero_kernel(unsigned char* p, uint64_t bytes) {
+  const uint64_t addr = reinterpret_cast<uint64_t>(p);
+  uint64_t head = (16 - (addr & 15)) & 15;
+  if (head > bytes) head = bytes;
+  const uint64_t n16 = (bytes - head) / 16, tail = bytes - head - n16 * 16;
   const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n16) p[i] = uint4{0, 0, 0, 0};
+  if (i < n16) reinterpret_cast<uint4*>(p + head)[i] = uint4{0, 0, 0, 0};
+  if (i < head) p[i] = 0;
+  if (i < tail) p[head + n16 * 16 + i] = 0;
 }
 
 }  // namespace
@@ -80,10 +90,23 @@ struct CompiledRoutine {
   Plan plan;
   GeneratedModule mod;
   std::vector<char> binary;   // gfx950 code object of the generated kernels (empty if none)
+  // What it was compiled from, for the second form below: the serialised batch, this routine's
+  // position in it, and the options as the caller gave them.
+  std::shared_ptr<const std::string> wire;
+  int wire_index = 0;
+  PlanOptions requested;
+  // The same routine planned without any kernel that reads or writes 16 bytes at a time relative to a
+  // node's base (matrix-core contractions, row-tile prologues and epilogues): built by the first link
+  // that finds one of those operands at a pool offset that is not 16-byte aligned.  The shared layer
+  // packs nodes at offsets aligned to the element size only (arrayjit/lib/backends.ml:22-51) and the
+  // reference's backends link whatever it hands them (cuda_backend.ml:983-1051).
+  mutable std::shared_ptr<CompiledRoutine> unaligned;
 };
 
 std::mutex g_mu;
 bool g_inited = false;
+// process-wide counters behind ocannl_hip_get_global_debug_info
+std::atomic<int64_t> g_live_codes{0}, g_compiled_routines{0}, g_hiprtc_modules{0}, g_unaligned_forms{0}, g_routine_runs{0};
 std::vector<std::unique_ptr<ocannl_hip_device>> g_devices;
 
 std::vector<char> hiprtc_compile(const std::string& src, const std::string& name) {
@@ -109,6 +132,7 @@ std::vector<char> hiprtc_compile(const std::string& src, const std::string& name
   std::vector<char> bin(n);
   hiprtcGetCode(prog, bin.data());
   hiprtcDestroyProgram(&prog);
+  ++g_hiprtc_modules;
   return bin;
 }
 
@@ -144,6 +168,55 @@ PlanOptions parse_options(const char* options) {
     else throw InvalidArgument("compile options: unknown key '" + k + "'");
   }
   return o;
+}
+
+// Plan, generate and compile cr.r (which the planner rewrites in place).
+void build_routine(CompiledRoutine& cr, const PlanOptions& opt) {
+  ++g_compiled_routines;
+  cr.plan = make_plan(cr.r, opt);
+  cr.mod = generate_module(cr.r, cr.plan);
+  if (!cr.mod.kernels.empty()) cr.binary = hiprtc_compile(cr.mod.source, cr.r.name);
+}
+
+// Nodes whose base address the plan's kernels access 16 bytes at a time.
+std::vector<int> wide_access_nodes(const Plan& plan) {
+  std::vector<int> ids;
+  auto add = [&](int node) { if (node >= 0) ids.push_back(node); };
+  for (auto& ph : plan.phases) {
+    if (ph.kind == Phase::Contraction) {
+      const GemmDesc& g = ph.gemm;
+      add(g.a.node); add(g.b.node); add(g.c.node); add(g.c_copy); add(g.epi_bias); add(g.epi_relu);
+      for (auto& m : g.group) { add(m.a.node); add(m.b.node); add(m.c.node); add(m.c_copy); }
+      for (auto& pr : g.more) { add(pr.first.node); add(pr.second.node); }
+    } else if (ph.kind == Phase::Generic) {
+      if (ph.fused_x >= 0) { add(ph.fused_a.node); add(ph.fused_b.node); if (ph.fused_x_store) add(ph.fused_x); }
+      if (ph.proj_y >= 0) { add(ph.proj_b.node); add(ph.proj_c.node); add(ph.proj_c_copy); }
+    }
+  }
+  return ids;
+}
+
+// The form of `cr` that makes no 16-byte access (built once, kept with the code).
+const CompiledRoutine& unaligned_form(const CompiledRoutine& cr) {
+  static std::mutex mu;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!cr.unaligned) {
+    auto alt = std::make_shared<CompiledRoutine>();
+    std::vector<Routine> rs = parse_routines(cr.wire->data(), cr.wire->size());
+    alt->r = std::move(rs.at(cr.wire_index));
+    alt->wire = cr.wire;
+    alt->wire_index = cr.wire_index;
+    alt->requested = cr.requested;
+    PlanOptions opt = cr.requested;
+    opt.enable_mfma = false;
+    opt.fuse_row_contractions = opt.fuse_row_projections = opt.fuse_stored_rows = opt.fuse_epilogues = false;
+    opt.row_vec4 = false;
+    build_routine(*alt, opt);
+    ++g_unaligned_forms;
+    if (!wide_access_nodes(alt->plan).empty()) throw InvalidArgument("link: the plan without 16-byte accesses still has some");
+    cr.unaligned = std::move(alt);
+  }
+  return *cr.unaligned;
 }
 
 }  // namespace
@@ -311,10 +384,9 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0, bool 
       if (v == 0 && !capturing) {
         hip_check(hipMemsetAsync(l.fill_ptr[0], 0, l.fill_bytes, dev.stream), "hipMemsetAsync");
       } else {
-        // local nodes sit at 256-byte offsets and are padded to 256 bytes: whole 16-byte stores
-        const uint64_t n16 = (l.fill_bytes + 15) / 16;
+        const uint64_t n16 = l.fill_bytes / 16 + 1;   // one thread per 16-byte store; the first block's 256 threads also cover the <= 15 head and tail bytes
         hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, dev.stream,
-                           static_cast<uint4*>(l.fill_ptr[v]), n16);
+                           static_cast<unsigned char*>(l.fill_ptr[v]), l.fill_bytes);
         hip_check(hipGetLastError(), "fill_zero_kernel");
       }
     } else if (ph.kind == Phase::Generic) {
@@ -465,6 +537,26 @@ int ocannl_hip_get_debug_info(ocannl_hip_device* dev, char* buf, size_t cap) {
     std::ostringstream s;
     s << "((pools " << dev->pools.size() << ") (pool_bytes " << dev->used << ") (scratch_bytes " << dev->scratch_used
       << ") (live_events " << dev->live_events << ") (live_routines " << dev->live_routines << "))";
+    copy_out(s.str(), buf, cap);
+  });
+}
+
+int ocannl_hip_get_global_debug_info(char* buf, size_t cap) {
+  return guarded([&] {
+    std::lock_guard<std::mutex> lock(g_mu);
+    int64_t devices = 0, pools = 0, pool_bytes = 0, scratch_bytes = 0, events = 0, routines = 0;
+    for (auto& d : g_devices) {
+      if (!d) continue;
+      ++devices;
+      pools += (int64_t)d->pools.size(); pool_bytes += (int64_t)d->used; scratch_bytes += (int64_t)d->scratch_used;
+      events += d->live_events; routines += d->live_routines;
+    }
+    std::ostringstream s;
+    s << "(hip_global_debug (live_devices " << devices << ") (live_streams " << devices << ") (live_events " << events
+      << ") (live_codes " << g_live_codes.load() << ") (live_routines " << routines << ") (compiled_routines "
+      << g_compiled_routines.load() << ") (hiprtc_modules " << g_hiprtc_modules.load() << ") (unaligned_forms "
+      << g_unaligned_forms.load() << ") (routine_runs " << g_routine_runs.load() << ") (pools " << pools << ") (pool_bytes "
+      << pool_bytes << ") (scratch_bytes " << scratch_bytes << "))";
     copy_out(s.str(), buf, cap);
   });
 }
@@ -623,16 +715,19 @@ int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, o
     if (!llir || !out) throw InvalidArgument("compile: null argument");
     PlanOptions opt = parse_options(options);
     auto code = std::make_unique<ocannl_hip_code>();
+    auto wire = std::make_shared<const std::string>(llir, len);
     std::vector<Routine> rs = parse_routines(llir, len);
     for (auto& r : rs) {
       CompiledRoutine cr;
       cr.r = std::move(r);
-      cr.plan = make_plan(cr.r, opt);
-      cr.mod = generate_module(cr.r, cr.plan);
-      if (!cr.mod.kernels.empty()) cr.binary = hiprtc_compile(cr.mod.source, cr.r.name);
+      cr.wire = wire;
+      cr.wire_index = (int)code->routines->size();
+      cr.requested = opt;
+      build_routine(cr, opt);
       code->routines->push_back(std::move(cr));
     }
     *out = code.release();
+    ++g_live_codes;
   });
 }
 
@@ -640,7 +735,10 @@ int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** out) {
   return ocannl_hip_compile_opts(llir, len, nullptr, out);
 }
 
-void ocannl_hip_code_free(ocannl_hip_code* code) { delete code; }
+void ocannl_hip_code_free(ocannl_hip_code* code) {
+  if (code) --g_live_codes;
+  delete code;
+}
 
 static const CompiledRoutine& routine_at(ocannl_hip_code* code, int index) {
   if (!code) throw InvalidArgument("null code");
@@ -684,6 +782,17 @@ int ocannl_hip_code_source(ocannl_hip_code* code, char* buf, size_t cap, size_t*
   });
 }
 
+int ocannl_hip_code_object(ocannl_hip_code* code, int index, char* buf, size_t cap, size_t* needed) {
+  return guarded([&] {
+    const CompiledRoutine& cr = routine_at(code, index);
+    if (needed) *needed = cr.binary.size();
+    if (buf) {
+      if (cap < cr.binary.size()) throw InvalidArgument("code_object: buffer too small");
+      std::memcpy(buf, cr.binary.data(), cr.binary.size());
+    }
+  });
+}
+
 int ocannl_hip_code_num_kernels(ocannl_hip_code* code, int index, int* n) {
   return guarded([&] { if (!n) throw InvalidArgument("null argument"); *n = (int)routine_at(code, index).plan.phases.size(); });
 }
@@ -719,9 +828,26 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
                     ocannl_hip_routine** out) {
   return guarded([&] {
     if (!dev || !out) throw InvalidArgument("link: null argument");
-    const CompiledRoutine& cr = routine_at(code, index);
+    const CompiledRoutine& requested = routine_at(code, index);
     if (n_locs > 0 && !locs) throw InvalidArgument("link: null locs");
     dev->make_current();
+    // The matrix-core kernels and the row-tile prologues / epilogues read and write 16-byte chunks
+    // relative to a node's base (local nodes sit at 256-byte offsets).  A context node that one of
+    // them touches at a pool offset that is not 16-byte aligned selects the routine's other form,
+    // in which generated kernels do that work element by element.
+    bool misaligned = false;
+    {
+      std::map<int, const ocannl_hip_node_loc*> where;
+      for (int i = 0; i < n_locs; ++i) where[locs[i].node_id] = &locs[i];
+      for (int id : wide_access_nodes(requested.plan)) {
+        auto it = where.find(id);
+        if (it == where.end() || requested.r.node(id).mode != Mode::Ctx) continue;
+        auto pool = dev->pools.find(it->second->pool_id);
+        const uintptr_t base = pool == dev->pools.end() ? 0 : reinterpret_cast<uintptr_t>(pool->second.first);
+        if ((base + it->second->offset) % 16 != 0) misaligned = true;
+      }
+    }
+    const CompiledRoutine& cr = misaligned ? unaligned_form(requested) : requested;
     // anything that fails below releases what the routine holds so far
     std::unique_ptr<ocannl_hip_routine, void (*)(ocannl_hip_routine*)> rt(new ocannl_hip_routine, destroy_routine);
     rt->dev = dev;
@@ -738,19 +864,6 @@ int ocannl_hip_link(ocannl_hip_device* dev, ocannl_hip_code* code, int index, co
       if (it == by_id.end())
         throw UserError("hip backend link: node " + n.ident + " (id " + std::to_string(n.id) + ") missing from context");
       ctx_ptr[n.id] = dev->resolve(it->second->pool_id, it->second->offset, (uint64_t)n.size_in_bytes(), "link");
-    }
-    // the MFMA kernels read 16-byte chunks relative to the node base (local nodes sit at 256-byte offsets)
-    for (auto& ph : cr.plan.phases) {
-      if (ph.kind != Phase::Contraction) continue;
-      std::vector<const GemmOperand*> ops{&ph.gemm.a, &ph.gemm.b, &ph.gemm.c};
-      for (auto& m : ph.gemm.group) { ops.push_back(&m.a); ops.push_back(&m.b); ops.push_back(&m.c); }
-      for (auto& pr : ph.gemm.more) { ops.push_back(&pr.first); ops.push_back(&pr.second); }
-      for (const GemmOperand* op : ops) {
-        auto it = ctx_ptr.find(op->node);
-        if (it != ctx_ptr.end() && reinterpret_cast<uintptr_t>(it->second) % 16 != 0)
-          throw UserError("hip backend link: node " + cr.r.node(op->node).ident +
-                          " feeds a matrix-core contraction and must sit at a 16-byte aligned pool offset");
-      }
     }
     // local nodes (and planner scratch): one private arena, 256-byte aligned sub-buffers
     uint64_t arena = 0;
@@ -896,6 +1009,7 @@ static void run_plain(ocannl_hip_routine& rt) {
 int ocannl_hip_routine_run(ocannl_hip_routine* rt) {
   return guarded([&] {
     if (!rt) throw InvalidArgument("run: null routine");
+    ++g_routine_runs;
     run_plain(*rt);
   });
 }

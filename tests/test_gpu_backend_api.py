@@ -96,27 +96,81 @@ def test_link_reports_missing_node(dev):
     B.free_pool(dev, pool_id=904)
 
 
-def test_link_rejects_misaligned_contraction_operand(dev):
-    # the matrix-core kernels read 16-byte chunks: an operand packed at a 4-byte aligned offset
-    # (what element-size alignment alone would allow) is a user error, reported at link time
+def test_contraction_operands_at_element_aligned_offsets_against_the_checker(dev):
+    # The shared layer packs nodes at offsets aligned to the element size only
+    # (arrayjit/lib/backends.ml:22-51) and the reference's backends link whatever it hands them
+    # (cuda_backend.ml:983-1051).  The matrix-core kernels read 16-byte chunks, so a context whose
+    # operands sit at 4-byte aligned offsets is linked in the routine's other form (generated
+    # kernels): same results, no error.
     from ocannl_amd import workloads as W
+    from parity import OracleRun, rel_err
     w = W.dense_contraction(b=256, i=128, o=128, prec="single", out_prec="single")
     code = B.compile(w.routine)
     assert any(k["kind"] == "mfma" for k in code.kernels())
     nodes = w.routine.param_nodes()
-    total, locs = 0, {}
-    for n in nodes:
-        locs[n.id] = (905, total)
-        total += (n.size_in_bytes + 255) // 256 * 256
-    B.alloc_pool(dev, pool_id=905, size_in_bytes=total + 256, alignment=256)
-    rt = B.link(dev, code, locs)          # aligned: fine
+    ora = OracleRun(w.routine, w.init)
+    ora.step()
+    for shift in (0, 4):
+        total, locs = shift, {}
+        for n in nodes:                      # tightly packed: every node right behind the previous one
+            locs[n.id] = (905, total)
+            total += n.size_in_bytes
+        B.alloc_pool(dev, pool_id=905, size_in_bytes=total, alignment=256)
+        B.memset_zero(dev, pool_id=905, offset=0, size_in_bytes=total)
+        for n in nodes:
+            if n.id in w.init:
+                B.from_host(dev, pool_id=905, offset=locs[n.id][1], src=np.ascontiguousarray(w.init[n.id]))
+        rt = B.link(dev, code, locs)
+        rt.run()
+        B.await_(dev)
+        for out in w.outputs:
+            got = np.zeros(out.dims, np.float32)
+            B.to_host(dev, pool_id=905, offset=locs[out.id][1], dst=got)
+            B.await_(dev)
+            assert rel_err(got, ora.get(out).reshape(out.dims), "single") <= 1e-4, (shift, out.ident)
+        del rt
+        B.free_pool(dev, pool_id=905)
+
+
+@pytest.mark.parametrize("how", ["graphs", "static_scratch"])
+def test_zero_fill_as_a_kernel_stays_inside_its_node(dev, how):
+    # A Zero_out of a context node whose size is not a multiple of 16 bytes, in a tightly packed pool
+    # (node offsets aligned to the element size, as arrayjit/lib/backends.ml:22-51 packs them): the
+    # fill kernel that replaces hipMemsetAsync under graph capture and in the entry point that may not
+    # allocate must leave the neighbouring node alone.
+    L.reset_symbols(0)
+    g = L.Node(1, "g", "single", (10,)); x = L.Node(2, "x", "single", (10,)); keep = L.Node(3, "keep", "single", (6,))
+    one = L.Node(4, "one", "single", (1,))
+    i = L.fresh_symbol()
+    # (the fill of g survives planning: the statement after it does not touch g everywhere; `one` makes
+    # a second launch so that the routine is worth a graph)
+    r = L.Routine("fills", [L.ZeroOut(g), L.ZeroOut(one),
+                            L.For(i, 0, 4, [L.Set(g, (L.It(i),), L.Binop("add", L.Get(g, (L.It(i),)), L.Get(x, (L.It(i),))))]),
+                            L.Set(one, (L.Fixed(0),), L.Binop("add", L.Get(one, (L.Fixed(0),)), L.Const(1.0)))])
+    code = B.compile(r, "serial=0;parallel=0;graphs=1" if how == "graphs" else "serial=0;parallel=0")
+    assert any(k["kind"] == "fill" for k in code.kernels()), code.kernels()
+    # pool: 4 bytes of lead-in, g (40 bytes) at offset 4, keep right behind it, then one and x
+    locs = {1: (906, 4), 3: (906, 44), 4: (906, 68), 2: (906, 72)}
+    B.alloc_pool(dev, pool_id=906, size_in_bytes=112, alignment=4)
+    sentinel = np.full(28, 7.0, np.float32)
+    B.from_host(dev, pool_id=906, offset=0, src=sentinel)
+    B.from_host(dev, pool_id=906, offset=72, src=np.arange(10, dtype=np.float32))
+    rt = B.link(dev, code, locs)
+    for _ in range(3):                       # (the first run is direct, later ones replay the graph)
+        if how == "graphs":
+            rt.run()
+        else:
+            rt.run_static_scratch()
+        B.await_(dev)
+    got = np.zeros(28, np.float32)
+    B.to_host(dev, pool_id=906, offset=0, dst=got)
+    B.await_(dev)
+    assert got[0] == 7.0                                         # lead-in
+    assert got[1:11].tolist() == [0, 1, 2, 3, 4, 0, 0, 0, 0, 0]  # g
+    assert got[11:17].tolist() == [7.0] * 6                      # keep
+    assert got[17] == 1.0                                        # one
     del rt
-    bad = dict(locs)
-    first = nodes[0].id
-    bad[first] = (905, locs[first][1] + 4)
-    with pytest.raises(B.User_error, match="16-byte"):
-        B.link(dev, code, bad)
-    B.free_pool(dev, pool_id=905)
+    B.free_pool(dev, pool_id=906)
 
 
 def test_compile_batch_links_and_runs_each_routine(dev):
