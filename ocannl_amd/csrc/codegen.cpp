@@ -689,6 +689,7 @@ struct Printer {
         const std::string s = sym_ident(c.sym);
         out.push_back(ind + "for (" + idx_t + " " + s + " = " + std::to_string(c.from) + "; " + s + " <= " +
                       std::to_string(c.to) + "; ++" + s + ") {");
+        if (debug_log) out.push_back(ind + "  " + log_call("index " + s + " = %d", {"(int)(" + s + ")"}));   // c_syntax.ml:458-465
         block(c.body, ind + "  ", out);
         out.push_back(ind + "}");
         break;
@@ -699,6 +700,18 @@ struct Printer {
         used_nodes.insert(c.node);
         const std::string v = "z" + std::to_string(fresh++);
         Pair cv = convert_precision(Prec::Double, n.prec);
+        if (debug_log && loggable(n.prec)) {
+          // every element logs `# <ident> := 0` and its value line (c_syntax.ml:476-479; the loops over
+          // the axes print as one loop over the flat offset, index lines left out)
+          const std::string zero = cv.first + "0" + cv.second, lhs = n.ident + "[" + v + "]";
+          out.push_back(ind + "for (" + idx_t + " " + v + " = 0; " + v + " < " + std::to_string(n.num_elems()) + "; ++" + v + ") {");
+          out.push_back(ind + "  " + log_call("# " + lit(n.ident + " := 0"), {}));
+          out.push_back(ind + "  " + log_call(lit(n.ident) + "[%u]{=%g} = %g = " + lit(zero),
+                                              {"(unsigned)(" + v + ")", as_double(n.prec, lhs), as_double(n.prec, zero)}));
+          out.push_back(ind + "  " + lhs + " = " + zero + ";");
+          out.push_back(ind + "}");
+          break;
+        }
         out.push_back(ind + "for (" + idx_t + " " + v + " = 0; " + v + " < " + std::to_string(n.num_elems()) + "; ++" + v +
                       ") " + n.ident + "[" + v + "] = " + cv.first + "0" + cv.second + ";");
         break;
@@ -743,6 +756,21 @@ struct Printer {
           } else off = offset_str(c.idcs, n.dims) + " + " + std::to_string(i);
           lines.push_back(n.ident + "[" + off + "] = " +
                           (c.length == 1 ? std::string("vec_result") : "vec_result.v[" + std::to_string(i) + "]") + ";");
+        }
+        if (debug_log && loggable(n.prec) && c.length > 1) {
+          // `# text`, then per element `ident[offset]{=old} = vec_result.v[i] = new` (c_syntax.ml:590-640),
+          // ahead of the stores
+          std::vector<std::string> logs;
+          if (!c.text.empty()) logs.push_back(log_call("# " + lit(c.text), {}));
+          for (int i = 0; i < c.length; ++i) {
+            const std::string& store = lines[1 + i];
+            const std::string lhs = store.substr(0, store.find(" = "));
+            const std::string off = lhs.substr(lhs.find('[') + 1, lhs.size() - lhs.find('[') - 2);
+            const std::string lane = "vec_result.v[" + std::to_string(i) + "]";
+            logs.push_back(log_call(lit(n.ident) + "[%u]{=%g} = " + lit(lane) + " = %g",
+                                    {"(unsigned)(" + off + ")", as_double(n.prec, lhs), as_double(n.prec, lane)}));
+          }
+          lines.insert(lines.begin() + 1, logs.begin(), logs.end());
         }
         // always a block here: several statements of one kernel may declare vec_result
         out.push_back(ind + "{");
@@ -1244,5 +1272,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
   mod.source = src.str();
   return mod;
 }
+
+const char* c_typ_name(Prec p) { return p == Prec::Half ? "HALF_T" : c_typ(p); }
 
 }  // namespace ocannl

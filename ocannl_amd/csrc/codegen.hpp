@@ -37,4 +37,8 @@ const char* builtins_hip_source();
 
 GeneratedModule generate_module(const Routine& r, const Plan& plan);
 
+// C type of a precision as the reference's printer declares it (Ops.c_typ_of_prec, ops.ml:324-337),
+// with the host's spelling of the half type: what the parameter lines of a routine's log show.
+const char* c_typ_name(Prec p);
+
 }  // namespace ocannl

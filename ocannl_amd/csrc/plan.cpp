@@ -2140,6 +2140,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
   std::string label;
   int next_sym = 0;
   Bf16Copies copies;
+  std::set<int> debug_zeroed;      // nodes whose first Zero_out has been seen (logging only)
   lift_routine_locals(r, plan);
   std::vector<std::string> pending_comments;
   Block top = r.body;
@@ -2149,6 +2150,40 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     Phase ph;
     ph.label = label;
     ph.stmt = sp;
+    if (sp->kind == Stmt::ZeroOut && opt.debug_log) {
+      // With logging a Zero_out is the loop nest of `tn[..] := 0` statements that the reference prints,
+      // each logging its element under the text `<ident> := 0` (c_syntax.ml:468-479) -- except the
+      // first function-scope Zero_out of a local node that its declaration already zeroes
+      // (c_syntax.ml:424-432), which prints nothing.
+      const Node& n = r.node(sp->node);
+      if (n.mode == Mode::Virtual) continue;
+      const bool first = debug_zeroed.insert(sp->node).second;
+      if (first && n.zero_initialized_by_code && n.mode == Mode::Local) {
+        // (the node still needs its zeros: a fill without log lines)
+        ph.kind = Phase::Fill;
+        ph.fill_node = sp->node;
+        ph.bytes = (double)n.size_in_bytes();
+        plan.phases.push_back(std::move(ph));
+        continue;
+      }
+      auto set = std::make_shared<Stmt>();
+      set->kind = Stmt::Set; set->node = sp->node; set->text = n.ident + " := 0";
+      auto zero = std::make_shared<Scalar>();
+      zero->kind = Scalar::Const; zero->cst = 0.0;
+      set->value = zero;
+      StmtP nest = set;
+      std::vector<int> syms;
+      for (size_t ax = 0; ax < n.dims.size(); ++ax) syms.push_back(fresh_symbol(r, &next_sym));
+      for (size_t ax = 0; ax < n.dims.size(); ++ax) { AxisIndex a; a.kind = AxisIndex::Iter; a.sym = syms[ax]; set->idcs.push_back(a); }
+      for (size_t ax = n.dims.size(); ax-- > 0;) {
+        auto loop = std::make_shared<Stmt>();
+        loop->kind = Stmt::For; loop->sym = syms[ax]; loop->from = 0; loop->to = n.dims[ax] - 1;
+        loop->body.push_back(nest);
+        nest = loop;
+      }
+      sp = nest;
+      ph.stmt = sp;
+    }
     if (sp->kind == Stmt::ZeroOut) {
       const Node& n = r.node(sp->node);
       if (n.mode == Mode::Virtual) continue;

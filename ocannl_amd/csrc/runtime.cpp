@@ -339,6 +339,29 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0, bool 
   if (rt.code->plan.debug_log) {
     static int g_run_id = 0;   // get_global_run_id
     rt.log_id = ++g_run_id;
+    // "Debug initial parameter state" (c_syntax.ml:1112-1150): one line per kernel parameter of the
+    // routine -- the reference's single kernel prints them itself; here the routine is many kernels, so
+    // the host prints them, under the run's log id and ahead of what the kernels print.  Parameters are
+    // sorted by their declaration, as c_syntax.ml:1080-1084 sorts them.
+    std::vector<std::pair<std::string, std::string>> lines;   // (declaration, rest of the line)
+    char buf[64];
+    if (r.merge_node >= 0) {
+      const Node& n = r.node(r.merge_node);
+      snprintf(buf, sizeof buf, "%p", merge_base);
+      lines.emplace_back(std::string("const ") + c_typ_name(n.prec) + " *merge_buffer", " &[" + std::to_string(n.num_elems()) + "] = " + buf);
+    }
+    for (auto& st : r.statics)
+      lines.emplace_back(std::string(rt.code->plan.large_index ? "const uint64_t " : "const uint32_t ") + sym_ident(st.sym),
+                         " = " + std::to_string(rt.statics.at(st.sym)));
+    for (int id : r.node_order) {
+      const Node& n = r.node(id);
+      if (n.mode != Mode::Ctx) continue;
+      snprintf(buf, sizeof buf, "%p", rt.node_ptr[v].at(id));
+      lines.emplace_back(std::string(c_typ_name(n.prec)) + " *" + n.ident, " &[" + std::to_string(n.num_elems()) + "] = " + buf);
+    }
+    std::sort(lines.begin(), lines.end());
+    for (auto& l : lines) printf("%d: %s%s$", rt.log_id, l.first.c_str(), l.second.c_str());
+    fflush(stdout);
   }
   const bool timed = kernel_ms != nullptr;
   if (timed) {

@@ -21,8 +21,12 @@ Pinned by: token-for-token equality with the reference-held generated C
 test_where_precision.c.expected, arrayjit/test/test_zero_out_codegen.expected,
 arrayjit/test/test_local_scope_init.expected) in tests/test_oracle_emit.py.
 
-Layout differs from the reference's PPrint output only in white space (line breaking);
-debug-log emission (``debug_log_from_routines``) is not restated.
+Layout differs from the reference's PPrint output only in white space (line breaking).
+
+Debug-log emission (``debug_log_from_routines``, c_syntax.ml:441-704 log branches, ``debug_float``
+c_syntax.ml:857-1018, the parameter header c_syntax.ml:1112-1150, ``Pure_C_config.pp_log_statement``
+c_syntax.ml:299-321) is restated too (``emit_proc(..., debug_log=True)``): pinned by token equality
+with test/operations/test_log_stmt_format.c.expected (tests/test_oracle_emit.py).
 """
 from __future__ import annotations
 
@@ -358,9 +362,88 @@ def reads_scope_before_set(target: L.Scope, body: Sequence[L.Stmt]) -> bool:
 
 
 class _Emitter:
-    def __init__(self, routine: L.Routine):
+    def __init__(self, routine: L.Routine, debug_log: bool = False, full_printf: bool = True):
         self.r = routine
         self.zero_out_seen = set()
+        # debug_log_from_routines (utils.ml:591): every statement logs what it computes.
+        # full_printf: `%g` values; otherwise (the `prefer_backend_uniformity` setting,
+        # cc_backend.ml:164-165) `%de-3` of the value times 1000 (c_syntax.ml:117-123).
+        self.debug_log = debug_log
+        self.float_log_style = "%g" if full_printf else "%de-3"
+        self.full_printf = full_printf
+
+    # -- logging (Pure_C_config, c_syntax.ml:117-123,293-321)
+    def styled_log_arg(self, doc: str) -> str:
+        return doc if self.full_printf else f"(int)({doc} * 1000.0)"
+
+    def log_statement(self, base_message: str, args: Sequence[str]) -> str:
+        lit = base_message.replace("\n", "\\n")
+        tail = "".join(", " + a for a in args)
+        return f'if (log_file_name && log_file) fprintf(log_file, "{lit}"{tail});'
+
+    def debug_float(self, prec: str, s: L.Scalar, guard: str = None):
+        """c_syntax.ml:857-1018: the expression as the log shows it, with `{=value}` after every read,
+        and the printf arguments behind it: ("acc", offset expression) | ("val", C expression)."""
+        st = self.float_log_style
+
+        def guarded(access: str) -> str:
+            return access if guard is None else f"({guard} ? {access} : 0)"
+
+        if isinstance(s, L.LocalScope):
+            return self.debug_float(prec, L.GetLocal(s.scope), guard)
+        if isinstance(s, L.GetLocal):
+            p, q = convert_precision(s.scope.node.prec, prec)
+            v = f"{p}{self.scope_name(s.scope)}{q}"
+            return v + "{=" + st + "}", [("val", v)]
+        if isinstance(s, L.GetMerge):
+            p, q = convert_precision(s.node.prec, prec)
+            off = array_offset(s.idcs, s.node.dims)
+            return f"{p}merge_buffer[%u]{q}" + "{=" + st + "}", [("acc", off), ("val", guarded(f"{p}merge_buffer[{off}]{q}"))]
+        if isinstance(s, L.Get):
+            p, q = convert_precision(s.node.prec, prec)
+            off = array_offset(s.idcs, s.node.dims)
+            return f"{p}{s.node.ident}[%u]{q}" + "{=" + st + "}", [("acc", off), ("val", guarded(f"{p}{s.node.ident}[{off}]{q}"))]
+        if isinstance(s, L.GetDynamic):
+            p, q = convert_precision(s.dyn_prec, prec)
+            _, idx_e = self.scalar(s.dyn_prec, s.dyn_value, "")
+            return f"{s.node.ident}@dyn_idx" + "{=" + st + "}", [("val", f"{p}{idx_e}{q}")]
+        if isinstance(s, L.Const):
+            p, q = convert_precision("double", prec)
+            return f"{p}{const_str(s.value)}{q}", []
+        if isinstance(s, L.ConstBits):
+            p, q = convert_precision("int64", prec)
+            return f"{p}{int(s.value)}LL{q}", []
+        if isinstance(s, L.EmbedIndex):
+            ix = L.axis_index_str(s.idx)
+            return (ix if ix else "0"), []
+        if isinstance(s, L.Binop) and s.op == "arg1":
+            return self.debug_float(prec, s.a, guard)
+        if isinstance(s, L.Binop) and s.op == "arg2":
+            return self.debug_float(prec, s.b, guard)
+        if isinstance(s, L.Ternop):
+            if s.op == "where":
+                _, cond_c = self.scalar(s.a_prec, s.a, "")
+                compose = lambda c: c if guard is None else f"({guard} && {c})"   # noqa: E731
+                d1, a1 = self.debug_float(s.a_prec, s.a, guard)
+                d2, a2 = self.debug_float(prec, s.b, compose(cond_c))
+                d3, a3 = self.debug_float(prec, s.c, compose(f"(!({cond_c}))"))
+            else:
+                d1, a1 = self.debug_float(prec, s.a, guard)
+                d2, a2 = self.debug_float(prec, s.b, guard)
+                d3, a3 = self.debug_float(prec, s.c, guard)
+            return cc_ternop(prec, s.op, d1, d2, d3), a1 + a2 + a3
+        if isinstance(s, L.Binop):
+            d1, a1 = self.debug_float(prec, s.a, guard)
+            d2, a2 = self.debug_float(prec, s.b, guard)
+            return cc_binop(prec, s.op, d1, d2), a1 + a2
+        if isinstance(s, L.Unop):
+            arg_prec = s.arg_prec if s.op == "uint4x32_to_prec_uniform1" else prec
+            d, a = self.debug_float(arg_prec, s.arg, guard)
+            return cc_unop(prec, s.op, d), a
+        raise TypeError(s)
+
+    def _log_args(self, args) -> List[str]:
+        return [a if kind == "acc" else self.styled_log_arg(a) for kind, a in args]
 
     # -- c_syntax.ml:424-432
     def zero_out_loop_redundant(self, n: L.Node) -> bool:
@@ -373,30 +456,54 @@ class _Emitter:
         p, s = convert_precision("int32", prec)
         return f" = {p}0{s}"
 
-    def stmts(self, body: Sequence[L.Stmt], ind: str, in_loop: bool) -> List[str]:
+    def stmts(self, body: Sequence[L.Stmt], ind: str, in_loop: bool, log_set_locals: bool = True) -> List[str]:
         out: List[str] = []
         for c in body:
-            out.extend(self.stmt(c, ind, in_loop))
+            out.extend(self.stmt(c, ind, in_loop, log_set_locals))
         return out
 
-    def stmt(self, c: L.Stmt, ind: str, in_loop: bool) -> List[str]:
+    def stmt(self, c: L.Stmt, ind: str, in_loop: bool, log_set_locals: bool = True) -> List[str]:
         if isinstance(c, L.Comment):
+            if self.debug_log:
+                return [ind + self.log_statement("COMMENT: " + c.text + "\n", [])]
             return [f"{ind}/* {c.text} */"]
         if isinstance(c, L.For):
             s = L.sym_ident(c.sym)
             head = f"{ind}for ({C_TYP[index_prec()]} {s} = {c.from_}; {s} <= {c.to}; ++{s}) {{"
-            return [head] + self.stmts(c.body, ind + "  ", True) + [ind + "}"]
+            body = self.stmts(c.body, ind + "  ", True, log_set_locals)
+            if self.debug_log:
+                body = [ind + "  " + self.log_statement(f"index {s} = %d\n", [s])] + body
+            return [head] + body + [ind + "}"]
         if isinstance(c, L.ZeroOut):
             first = c.node.id not in self.zero_out_seen
             self.zero_out_seen.add(c.node.id)
             if first and not in_loop and self.zero_out_loop_redundant(c.node):
                 return []
             node = c.node
-            loops = L.loop_over_dims(node.dims, lambda idcs: [L.Set(node, idcs, L.Const(0.0))])
-            return self.stmts(loops, ind, in_loop)
+
+            def zero(idcs):
+                st = L.Set(node, idcs, L.Const(0.0))
+                st.debug = node.ident + " := 0"          # c_syntax.ml:479
+                return [st]
+            loops = L.loop_over_dims(node.dims, zero)
+            return self.stmts(loops, ind, in_loop, log_set_locals)
         if isinstance(c, L.Set):
             defs, val = self.scalar(c.node.prec, c.value, ind + "  ")
-            asg = f"{c.node.ident}[{array_offset(c.idcs, c.node.dims)}] = {val};"
+            off = array_offset(c.idcs, c.node.dims)
+            if self.debug_log:                           # c_syntax.ml:493-535
+                st = self.float_log_style
+                dbg, args = self.debug_float(c.node.prec, c.value)
+                text = getattr(c, "debug", None) or L.ll_statement(c)
+                lhs = f"{c.node.ident}[{off}]"
+                lines = [f"{C_TYP[c.node.prec]} new_set_v = {val};",
+                         self.log_statement("# " + text + "\n", []),
+                         self.log_statement(f"{c.node.ident}[%u]{{={st}}} = {st} = {dbg}\n",
+                                            [off, self.styled_log_arg(lhs), self.styled_log_arg("new_set_v")]
+                                            + self._log_args(args)),
+                         "fflush(log_file);",
+                         f"{lhs} = new_set_v;"]
+                return self._with_defs(defs, lines, ind, always_block=True)
+            asg = f"{c.node.ident}[{off}] = {val};"
             return self._with_defs(defs, [asg], ind)
         if isinstance(c, L.SetFromVec):
             prec = c.node.prec
@@ -412,12 +519,39 @@ class _Emitter:
                     off = array_offset(c.idcs, c.node.dims) + f" + {i}"
                 v = "vec_result" if c.length == 1 else f"vec_result.v[{i}]"
                 lines.append(f"{c.node.ident}[{off}] = {v};")
+            if self.debug_log:                           # c_syntax.ml:590-640
+                st = self.float_log_style
+                text = getattr(c, "debug", None) or L.ll_statement(c)
+                logs = [self.log_statement("# " + text + "\n", [])]
+                for i in range(c.length):
+                    last = c.idcs[-1]
+                    if isinstance(last, L.Fixed):
+                        off = array_offset(tuple(c.idcs[:-1]) + (L.Fixed(last.i + i),), c.node.dims)
+                    else:
+                        off = array_offset(c.idcs, c.node.dims) + f" + {i}"
+                    logs.append(self.log_statement(
+                        f"{c.node.ident}[%u]{{={st}}} = vec_result.v[{i}] = {st}\n",
+                        [off, self.styled_log_arg(f"{c.node.ident}[{off}]"), self.styled_log_arg(f"vec_result.v[{i}]")]))
+                logs.append("fflush(log_file);")
+                return self._with_defs(defs, lines[:1] + logs + lines[1:], ind, always_block=True)
             if not defs:
                 # c_syntax.ml:640: no enclosing block in this case
                 return [ind + ln for ln in lines]
             return self._with_defs(defs, lines, ind)
         if isinstance(c, L.SetLocal):
             defs, val = self.scalar(c.scope.node.prec, c.value, ind + "  ")
+            if self.debug_log and log_set_locals:        # c_syntax.ml:649-684
+                st = self.float_log_style
+                name = self.scope_name(c.scope)
+                dbg, args = self.debug_float(c.scope.node.prec, c.value)
+                lines = [f"{C_TYP[c.scope.node.prec]} new_set_local_v = {val};",
+                         self.log_statement(f"# local {name} := {val}\n", []),
+                         self.log_statement(f"{name}{{={st}}} = {st} = {dbg}\n",
+                                            [self.styled_log_arg(name), self.styled_log_arg("new_set_local_v")]
+                                            + self._log_args(args)),
+                         "fflush(log_file);",
+                         f"{name} = new_set_local_v;"]
+                return self._with_defs(defs, lines, ind, always_block=True)
             return self._with_defs(defs, [f"{self.scope_name(c.scope)} = {val};"], ind)
         if isinstance(c, L.DeclareLocal):
             prec = c.scope.node.prec
@@ -425,7 +559,9 @@ class _Emitter:
             return [f"{ind}{C_TYP[prec]} {self.scope_name(c.scope)}{init};"]
         raise TypeError(c)
 
-    def _with_defs(self, defs, lines: List[str], ind: str) -> List[str]:
+    def _with_defs(self, defs, lines: List[str], ind: str, always_block: bool = False) -> List[str]:
+        if not defs and always_block:
+            return [ind + "{"] + [ind + "  " + ln for ln in lines] + [ind + "}"]
         if not defs:
             return [ind + ln for ln in lines]
         # c_syntax.ml:406-409: dedup by scope id, sorted by scope id
@@ -445,7 +581,7 @@ class _Emitter:
             sp = s.scope.node.prec
             init = self.init_zero(sp) if reads_scope_before_set(s.scope, s.body) else ""
             lines = [f"{ind}{C_TYP[sp]} {self.scope_name(s.scope)}{init};"]
-            lines += self.stmts(s.body, ind, True)
+            lines += self.stmts(s.body, ind, True, log_set_locals=False)   # c_syntax.ml:725
             p, q = convert_precision(sp, prec)
             return [(s.scope.scope_id, lines)], f"{p}{self.scope_name(s.scope)}{q}"
         if isinstance(s, L.GetLocal):
@@ -503,12 +639,14 @@ class _Emitter:
         raise TypeError(s)
 
 
-def kernel_params(r: L.Routine) -> List[Tuple[str, object]]:
+def kernel_params(r: L.Routine, debug_log: bool = False) -> List[Tuple[str, object]]:
     """Parameter declarations sorted by declaration string (c_syntax.ml:1080-1084).
 
-    Returns [(decl, source)] with source a Node (pointer), a StaticSymbol (int) or the
-    string "merge"."""
+    Returns [(decl, source)] with source a Node (pointer), a StaticSymbol (int), the
+    string "merge" or, with logging, "log" (the log file's name, c_syntax.ml:1067-1073)."""
     params: List[Tuple[str, object]] = []
+    if debug_log:
+        params.append(("const char* log_file_name", "log"))
     if r.merge_node is not None:
         params.append((f"const {C_TYP[r.merge_node.prec]} *merge_buffer", "merge"))
     for s in r.static_indices:
@@ -520,13 +658,28 @@ def kernel_params(r: L.Routine) -> List[Tuple[str, object]]:
     return params
 
 
-def emit_proc(r: L.Routine) -> str:
-    """The routine's C function (without builtins), c_syntax.ml:1021-1210."""
-    em = _Emitter(r)
-    params = kernel_params(r)
+def emit_proc(r: L.Routine, debug_log: bool = False, full_printf: bool = True) -> str:
+    """The routine's C function (without builtins), c_syntax.ml:1021-1210.  ``debug_log``: with the
+    statements that log every computed value to the file named by the extra first parameter."""
+    em = _Emitter(r, debug_log, full_printf)
+    params = kernel_params(r, debug_log)
     out = [f" void {r.name}("]
     out.append(",\n".join("    " + d for d, _ in params) + ") {")
-    out.append("")
+    if debug_log:
+        # c_syntax.ml:1098-1150: open the file, then the initial state of every parameter
+        out += ["  FILE* log_file = NULL;", "  if (log_file_name) {", '    log_file = fopen(log_file_name, "w");', "  }",
+                "  /* Debug initial parameter state. */"]
+        for decl, src in params:
+            if src == "log":
+                continue
+            if src == "merge":
+                out.append("  " + em.log_statement(f"{decl} &[{r.merge_node.num_elems}] = %p\n", ["(void*)merge_buffer"]))
+            elif isinstance(src, L.Node):
+                out.append("  " + em.log_statement(f"{decl} &[{src.num_elems}] = %p\n", [f"(void*){src.ident}"]))
+            else:
+                out.append("  " + em.log_statement(f"{decl} = %d\n", [L.sym_ident(src.sym)]))
+    else:
+        out.append("")
     out.append("  /* Local declarations and initialization. */")
     for n in r.nodes():
         if n.mode == "local":
@@ -535,6 +688,8 @@ def emit_proc(r: L.Routine) -> str:
     out.append("")
     out.append("  /* Main logic. */")
     out.extend(em.stmts(r.body, "  ", False))
+    if debug_log:
+        out.append("  if (log_file) { fclose(log_file); log_file = NULL; }")   # c_syntax.ml:1200-1206
     out.append("}")
     return "\n".join(out)
 
@@ -542,10 +697,10 @@ def emit_proc(r: L.Routine) -> str:
 _BUILTINS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "builtins_cc.h")
 
 
-def emit_translation_unit(routines: Sequence[L.Routine]) -> str:
+def emit_translation_unit(routines: Sequence[L.Routine], debug_log: bool = False, full_printf: bool = True) -> str:
     """Builtins + all procedures, as ``Cc_backend.compile_batch`` lays them out
     (cc_backend.ml:345-376); the whole builtins header is prepended instead of the
     reference's per-key filtering (c_syntax.ml:330-362), which only removes dead code."""
     with open(_BUILTINS) as f:
         text = f.read()
-    return text + "\n" + "\n".join(emit_proc(r) for r in routines) + "\n"
+    return text + "\n" + "\n".join(emit_proc(r, debug_log, full_printf) for r in routines) + "\n"

@@ -50,9 +50,13 @@ def host_array(node: L.Node, fill=None) -> np.ndarray:
 class CompiledOracle:
     """A loaded translation unit holding one or more routines."""
 
-    def __init__(self, routines: Sequence[L.Routine], keep_dir: str | None = None):
+    def __init__(self, routines: Sequence[L.Routine], keep_dir: str | None = None, debug_log: bool = False,
+                 full_printf: bool = True):
+        """``debug_log``: the routines log every computed value (``debug_log_from_routines``); ``run``
+        then takes the name of the file to write (cc_backend.ml: the log file per run)."""
         self.routines = {r.name: r for r in routines}
-        self.source = cc_emit.emit_translation_unit(routines)
+        self.debug_log = debug_log
+        self.source = cc_emit.emit_translation_unit(routines, debug_log, full_printf)
         tag = hashlib.sha1(self.source.encode()).hexdigest()[:16]
         d = keep_dir or os.path.join(tempfile.gettempdir(), "ocannl_oracle_cc")
         os.makedirs(d, exist_ok=True)
@@ -73,14 +77,18 @@ class CompiledOracle:
         self.lib = ctypes.CDLL(self.so_path)
 
     def run(self, name: str, buffers: Mapping[int, np.ndarray],
-            static: Mapping[int, int] | None = None, merge: np.ndarray | None = None) -> None:
+            static: Mapping[int, int] | None = None, merge: np.ndarray | None = None,
+            log_file: str | None = None) -> None:
         """Call routine ``name``; ``buffers`` maps node id -> C-contiguous array (mutated in
-        place); ``static`` maps static symbol -> value."""
+        place); ``static`` maps static symbol -> value; ``log_file``: where a routine built with
+        ``debug_log`` writes its log (None: it logs nothing)."""
         r = self.routines[name]
         static = static or {}
         args = []
-        for _decl, src in cc_emit.kernel_params(r):
-            if isinstance(src, L.Node):
+        for _decl, src in cc_emit.kernel_params(r, self.debug_log):
+            if src == "log":
+                args.append(ctypes.c_char_p(log_file.encode() if log_file else None))
+            elif isinstance(src, L.Node):
                 a = buffers[src.id]
                 assert a.flags["C_CONTIGUOUS"] and a.nbytes == src.size_in_bytes, (src, a.shape)
                 args.append(ctypes.c_void_p(a.ctypes.data))

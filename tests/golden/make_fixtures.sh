@@ -2,7 +2,7 @@
 # Regenerates the trimmed expected-output fixtures from a reference checkout.
 REF=${1:-/root/reference}
 cd "$(dirname "$0")"
-for f in top_down_prec zero_out_local_decl test_where_precision; do
+for f in top_down_prec zero_out_local_decl test_where_precision test_log_stmt_format; do
   sed -n '/^ void /,$p' "$REF/test/operations/$f.c.expected" > "$f.proc.c.expected"
 done
 sed -n '3,$p' "$REF/arrayjit/test/test_zero_out_codegen.expected" > test_zero_out_codegen.proc.c.expected

@@ -41,8 +41,27 @@ class OracleRun:
 from ocannl_amd.backend import HipRun  # noqa: E402,F401  (the GPU side lives in the package)
 
 
+def _rows(a: np.ndarray) -> np.ndarray:
+    a = np.asarray(a, np.float64)
+    return a.reshape(-1, a.shape[-1]) if a.ndim >= 2 else a.reshape(1, -1)
+
+
 def rel_err(got: np.ndarray, want: np.ndarray, prec: str) -> float:
-    """max |got - want| / max(|want|_inf, tiny): relative to the tensor's scale."""
+    """Largest |got - want| relative to the scale of the ROW the element sits in (the tensor's last
+    axis; a vector or scalar is one row): max over rows of max|diff| / max|want| of that row.  So an
+    element is judged against max(|want|, its row's scale): a row of small gradients is not excused by
+    large values elsewhere in the tensor.  A row whose expected values are all (nearly) zero is judged
+    at a thousandth of the tensor's scale -- below that a deviation is the noise of sums that cancel,
+    whatever computes them."""
+    g, w = _rows(W.to_float(got, prec)), _rows(W.to_float(want, prec))
+    assert g.shape == w.shape, (g.shape, w.shape)
+    tensor = max(float(np.max(np.abs(w))), 1e-30)
+    scale = np.maximum(np.max(np.abs(w), axis=1), 1e-3 * tensor)
+    return float(np.max(np.max(np.abs(g - w), axis=1) / scale))
+
+
+def tensor_err(got: np.ndarray, want: np.ndarray, prec: str) -> float:
+    """max |got - want| / max |want| over the whole tensor (looser than rel_err: kept for reporting)."""
     g, w = W.to_float(got, prec), W.to_float(want, prec)
     scale = max(float(np.max(np.abs(w))), 1e-30)
     return float(np.max(np.abs(g - w))) / scale

@@ -279,3 +279,42 @@ def test_memory_operands_of_conditionals_are_loaded_ahead_of_the_statement():
     assert re.search(r"const float (w\d+_) = b\[i\d+\];\s*g\[i\d+\] = \(a\[i\d+\] > 0\.0 \? \1 : 0\.0\);", src), src
     assert len(re.findall(r"const float w\d+_ = [bc]\[", src)) == 3, src
     assert re.search(r"v\[[^\]]*\] = \(a\[[^\]]*\] > 0\.0 \? b\[[^\]]*\] : 0\.0\);", src), src
+
+
+def _scores_then_row_chain(rewrite_operand: bool):
+    # x[s, t] = sum_d a[s, d] * b[t, d] feeding a row-wise chain over the rows s (max, exp of the shifted
+    # value); optionally the chain also stores into the operand a itself
+    S, T, D = 512, 128, 128
+    L.reset_symbols(0)
+    a = L.Node(1, "a", "bfloat16", (S, D)); b = L.Node(2, "b", "bfloat16", (T, D))
+    x = L.Node(3, "x", "bfloat16", (S, T), mode="local"); m = L.Node(4, "m", "bfloat16", (S,), mode="local")
+    y = L.Node(5, "y", "bfloat16", (S, T))
+    s, t, d = L.fresh_symbol(), L.fresh_symbol(), L.fresh_symbol()
+    body = [L.ZeroOut(x), L.For(s, 0, S - 1, [L.For(t, 0, T - 1, [L.For(d, 0, D - 1, [L.Set(x, (L.It(s), L.It(t)), L.Ternop(
+        "fma", L.Get(a, (L.It(s), L.It(d))), L.Get(b, (L.It(t), L.It(d))), L.Get(x, (L.It(s), L.It(t)))))])])])]
+    s2, t2 = L.fresh_symbol(), L.fresh_symbol()
+    body.append(L.For(s2, 0, S - 1, [L.Set(m, (L.It(s2),), L.Const(float("-inf")))]))
+    s3 = L.fresh_symbol()
+    body.append(L.For(s3, 0, S - 1, [L.For(t2, 0, T - 1, [L.Set(m, (L.It(s3),), L.Binop(
+        "max", L.Get(m, (L.It(s3),)), L.Get(x, (L.It(s3), L.It(t2)))))])]))
+    s4, t4 = L.fresh_symbol(), L.fresh_symbol()
+    body.append(L.For(s4, 0, S - 1, [L.For(t4, 0, T - 1, [L.Set(y, (L.It(s4), L.It(t4)), L.Unop(
+        "exp", L.Binop("sub", L.Get(x, (L.It(s4), L.It(t4))), L.Get(m, (L.It(s4),)))))])]))
+    if rewrite_operand:
+        s5, t5 = L.fresh_symbol(), L.fresh_symbol()
+        body.append(L.For(s5, 0, S - 1, [L.For(t5, 0, T - 1, [L.Set(a, (L.It(s5), L.It(t5)), L.Get(y, (L.It(s5), L.It(t5))))])]))
+    return L.Routine("scores_chain", body)
+
+
+def test_a_row_group_that_rewrites_an_operand_keeps_the_contraction_apart():
+    # The contraction ahead of a row-wise chain becomes that kernel's prologue (each workgroup computes
+    # its own 32 rows of x) -- unless the chain itself stores into an operand of the contraction: one
+    # workgroup's stores would then race with another workgroup's prologue loads, which a kernel
+    # boundary used to order.
+    fused = B.compile(_scores_then_row_chain(False))
+    body = fused.source().split('extern "C"', 1)[1]
+    assert "ocn_rowtile_contract<" in body and not any(k["kind"] == "mfma" for k in fused.kernels())
+    apart = B.compile(_scores_then_row_chain(True))
+    body = apart.source().split('extern "C"', 1)[1]
+    assert "ocn_rowtile_contract<" not in body
+    assert sum(k["kind"] == "mfma" for k in apart.kernels()) == 1

@@ -12,14 +12,26 @@ from parity import HipRun, OracleRun, rel_err
 pytestmark = pytest.mark.gpu
 
 
-def _err(got, want, prec):
-    """fp32: max |diff| / max |want| (bar 1e-4).  bf16: every stored intermediate carries a 2^-9
-    rounding, so single elements of a chain of ops can be off by more than the bar while the
-    tensor as a whole is not; the bar 2e-2 is applied to the Frobenius-norm relative error."""
+def _err(got, want, prec, elementwise=False):
+    """fp32: the row-scale error of parity.rel_err (bar 1e-4): every element against max(|want|, the
+    scale of its row).  bf16: every stored intermediate carries a 2^-9 rounding, so the bar 2e-2 is
+    applied to the Frobenius-norm relative error of the tensor.  `elementwise` adds a bound on every
+    single element -- within 2^-5 of its row's largest magnitude (eight bf16 steps there; the reference
+    is the checker in single precision, so a chain of bf16-rounded scores, exponentials and weights
+    legitimately leaves elements two to four steps off: 2^-6 measured on the attention output) -- so
+    that a tensor cannot pass on its norm with a few grossly wrong entries.  It is asked for where the
+    chain of bf16 operations is short (the attention routines).  It is not asked of parameters after a
+    training step of the transformer: the layer norm as the reference writes it subtracts the SUM
+    over the axis (lib/nn_blocks.ml:251-258), which puts the signal into small differences of large
+    bf16 values, and gradients that pass through it differ between ANY two evaluation orders by far
+    more than that (0.31 of the row scale between this path and the single-precision checker on the
+    embedding matrix after one step, while both stay within the norm bar)."""
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     if prec == "bfloat16":
+        elem = rel_err(got, want, "double")
+        assert not elementwise or elem <= 2.0 ** -5, f"bf16 element off by {elem:.3g} of its row's scale"
         return float(np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30))
-    return float(np.max(np.abs(got - want)) / max(np.max(np.abs(want)), 1e-30))
+    return rel_err(got, want, "double")
 
 
 def _widened_init(w_low, w_ref):
@@ -64,7 +76,7 @@ def test_attention_fwd_bwd(prec, tol, opts):
     hip.step(); ora.step()
     for name, p in (("out", prec), ("dq", "single"), ("dk", "single"), ("dv", "single")):
         got = W.to_float(hip.get(w.nodes[name]), p)
-        assert _err(got, ora.get(wr.nodes[name]), prec) <= tol, name
+        assert _err(got, ora.get(wr.nodes[name]), prec, elementwise=True) <= tol, name
     if prec == "bfloat16":   # the reference semantics themselves stay within a looser bound
         low = OracleRun(w.routine, w.init)
         low.step()
@@ -86,7 +98,7 @@ def test_attention_with_matrix_core_prologue_and_epilogue_against_the_checker(sh
     hip.step(); ora.step()
     for name, p in (("out", "bfloat16"), ("attn", "bfloat16"), ("dq", "single"), ("dk", "single"), ("dv", "single")):
         got = W.to_float(hip.get(w.nodes[name]), p)
-        assert _err(got, ora.get(wr.nodes[name]), "bfloat16") <= 2e-2, name
+        assert _err(got, ora.get(wr.nodes[name]), "bfloat16", elementwise=True) <= 2e-2, name
     hip.close()
 
 
@@ -136,6 +148,34 @@ def test_full_size_transformer_step_properties():
         assert _err(W.to_float(a, n.prec), W.to_float(p, n.prec).astype(np.float64), n.prec) <= 2e-2, name
     for h in runs + [plain]:
         h.close()
+
+
+def test_full_size_transformer_learns_a_token_mapping():
+    # benchmark configuration 4 at its real size and precision (bf16 values, fp32 gradients) on targets
+    # that can be learnt: the token to predict is a fixed function of the input token, (7 t + 3) mod
+    # vocabulary.  The benchmark's own targets are random (its loss stays at ln 4096), and at its
+    # learning rate three steps move a bf16 weight by less than its last bit; here the learning rate is
+    # 10 -- the loss is a mean over 8192 tokens, so a gradient entry is of the order of 1e-4 -- at which
+    # the bf16 weights do move.  The loss has to fall, step after step, by 0.25 within 60 steps.
+    batch, seq, vocab = 32, 256, 4096
+    w = W.transformer(lr=10.0)
+    by = {n.ident.rsplit("_", 1)[0]: n for n in w.routine.param_nodes()}
+    toks = np.random.default_rng(1).integers(0, vocab, size=(batch, seq))
+    oh_in = np.zeros((batch, seq, vocab), np.float32); oh_tg = np.zeros((batch, seq, vocab), np.float32)
+    np.put_along_axis(oh_in, toks[:, :, None], 1.0, axis=-1)
+    np.put_along_axis(oh_tg, ((toks * 7 + 3) % vocab)[:, :, None], 1.0, axis=-1)
+    init = dict(w.init)
+    init[by["input_batch"].id] = W.as_prec(oh_in, "bfloat16")
+    init[by["target_batch"].id] = W.as_prec(oh_tg, "bfloat16")
+    hip = HipRun(w.routine, init)
+    losses = []
+    for _ in range(60):
+        hip.step()
+        losses.append(float(W.to_float(hip.get(w.nodes["loss"]), w.nodes["loss"].prec)[0]))
+    hip.close()
+    assert abs(losses[0] - np.log(4096.0)) < 0.05, losses[0]
+    assert losses[-1] <= losses[0] - 0.25, losses
+    assert all(b <= a + 2e-2 for a, b in zip(losses, losses[1:])), losses      # no step climbs back
 
 
 def test_full_size_attention_against_torch_autograd():

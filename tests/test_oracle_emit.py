@@ -108,6 +108,43 @@ def test_text_zero_out_codegen():
     assert _norm(cc_emit.emit_proc(r)) == _norm(_golden("test_zero_out_codegen.proc.c.expected"))
 
 
+def _log_stmt_format():
+    # test/operations/test_log_stmt_format.ml: c = a + b on one-element tensors, compiled with
+    # debug_log_from_routines (and `%de-3` values: the prefer_backend_uniformity log style)
+    a = L.Node(1, "a", "single", (1,)); b = L.Node(2, "b", "single", (1,)); c = L.Node(3, "c", "single", (1,))
+    z = (L.Fixed(0),)
+    body = [L.Comment("c fwd"), L.Set(c, z, L.Binop("add", L.Get(a, z), L.Get(b, z))), L.Comment("end")]
+    return L.Routine("c_fwd", body), (a, b, c)
+
+
+def test_text_log_stmt_format():
+    # the log statements of c_syntax.ml:493-535 (Set), :539-546 (comments), :1112-1150 (parameter
+    # header), :1200-1206 (closing the file), as the reference's own golden holds them
+    r, _ = _log_stmt_format()
+    assert _norm(cc_emit.emit_proc(r, debug_log=True, full_printf=False)) == _norm(_golden("test_log_stmt_format.proc.c.expected"))
+    # without the option nothing of it is emitted
+    assert "fprintf" not in cc_emit.emit_proc(r)
+
+
+def test_logging_checker_writes_the_lines_the_format_promises(tmp_path):
+    # the compiled checker, run with a log file: header lines, comments, `# statement`, value line
+    r, (a, b, c) = _log_stmt_format()
+    lib = cc_oracle.CompiledOracle([r], debug_log=True, full_printf=False)
+    bufs = {a.id: np.array([1.0], np.float32), b.id: np.array([1.0], np.float32), c.id: np.zeros(1, np.float32)}
+    log = tmp_path / "c_fwd.log"
+    lib.run("c_fwd", bufs, log_file=str(log))
+    assert bufs[c.id][0] == 2.0
+    lines = log.read_text().splitlines()
+    assert [re.sub(r"= 0x[0-9a-f]+|= \(nil\)", "= 0xNNNN", ln) for ln in lines[:3]] == [
+        "float *a &[1] = 0xNNNN", "float *b &[1] = 0xNNNN", "float *c &[1] = 0xNNNN"]
+    assert lines[3:] == ["COMMENT: c fwd", "# c[0] := (a[0] + b[0]);",
+                         "c[0]{=0e-3} = 2000e-3 = (a[0]{=1000e-3} + b[0]{=1000e-3})", "COMMENT: end"]
+    # ... and with full printf support, `%g` values (cc_backend.ml:164-165)
+    lib = cc_oracle.CompiledOracle([r], debug_log=True)
+    lib.run("c_fwd", bufs, log_file=str(log))
+    assert log.read_text().splitlines()[5] == "c[0]{=2} = 2 = (a[0]{=1} + b[0]{=1})"
+
+
 def _sections(text):
     parts = re.split(r"^=== .* ===\n", text, flags=re.M)
     return [p for p in parts[1:]]

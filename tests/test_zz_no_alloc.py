@@ -63,9 +63,16 @@ def test_static_scratch_run_equals_the_allocating_run_twice_in_a_row():
     sym = w.statics["batch_n"].sym
     for opts in (None, "serial=0"):
         runs = [B.HipRun(w.routine, w.init, opts) for _ in range(2)]
+        dev = runs[1].ctx.dev
         for step in range(4):
             runs[0].step({sym: step})
+            B.await_(dev)
+            # the successful path allocates nothing: pool bytes, scratch bytes, live events and
+            # routines of the device read the same before and after
+            used, info = B.get_used_memory(dev), B.get_debug_info(dev)
             runs[1].step({sym: step}, static_scratch=True)
+            B.await_(dev)
+            assert B.get_used_memory(dev) == used and B.get_debug_info(dev) == info
         for name in ("loss", "w1", "w2", "w3", "b1"):
             assert np.array_equal(runs[0].get(w.nodes[name]), runs[1].get(w.nodes[name])), name
         for h in runs:
