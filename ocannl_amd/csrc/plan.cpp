@@ -423,6 +423,36 @@ void choose_scope_coop(const Routine& r, Phase& ph) {
   if (lanes > 1) { ph.coop_lanes = lanes; ph.coop_scope = found[0]; ph.coop_accum = accum; }
 }
 
+// Does the innermost sequential symbol walk one of the phase's big operands with unit stride?  Only
+// the operands that every other one is small against count: a per-row scalar inlined into the
+// addend (the mean and deviation of a layer norm) is contiguous along the rows and says nothing
+// about how the tensors that carry the traffic lie.
+static bool reduction_walks_unit_stride(const Routine& r, const Phase& ph, const Stmt& set) {
+  std::map<int, int64_t> ext;
+  for (size_t i = 0; i < ph.par_syms.size(); ++i) ext[ph.par_syms[i]] = ph.par_ext[i];
+  for (size_t i = 0; i < ph.seq_syms.size(); ++i) ext[ph.seq_syms[i]] = ph.seq_to[i] - ph.seq_from[i] + 1;
+  std::vector<Access> acc; bool f = false; std::set<ScopeId> d;
+  scalar_accesses(*set.value, acc, f, d);
+  std::vector<int64_t> foot(acc.size(), 0);
+  int64_t biggest = 0;
+  for (size_t i = 0; i < acc.size(); ++i) {
+    if (acc[i].node == set.node) continue;
+    int64_t n = 1;
+    for (auto& kv : ext) {
+      bool m = false;
+      for (auto& ix : *acc[i].idcs) m = m || ix.mentions(kv.first);
+      if (m) n *= kv.second;
+    }
+    foot[i] = n;
+    biggest = std::max(biggest, n);
+  }
+  for (size_t i = 0; i < acc.size(); ++i) {
+    if (acc[i].node == set.node || foot[i] * 16 < biggest) continue;
+    if (get_stride(strides_of(r, acc[i].node, *acc[i].idcs), ph.seq_syms.back()) == 1) return true;
+  }
+  return false;
+}
+
 void choose_coop(const Routine& r, Phase& ph, const PlanOptions& opt) {
   ph.coop_lanes = 1;
   if (!opt.enable_coop) return;
@@ -432,21 +462,11 @@ void choose_coop(const Routine& r, Phase& ph, const PlanOptions& opt) {
   const Stmt& set = *ph.inner[0];
   const Prec p = r.node(set.node).prec;
   if (!(p == Prec::Single || p == Prec::Double || p == Prec::Bfloat16 || p == Prec::Half)) return;
-  const int rc = ph.seq_syms.back();
   const int64_t rext = ph.seq_to.back() - ph.seq_from.back() + 1;
   int64_t P = 1, R = 1;
   for (auto e : ph.par_ext) P *= e;
   for (size_t i = 0; i < ph.seq_syms.size(); ++i) R *= ph.seq_to[i] - ph.seq_from[i] + 1;
-  // does the innermost sequential symbol walk some operand with unit stride?
-  std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
-  scalar_accesses(*set.value, acc, f, d);
-  bool unit = false;
-  for (auto& a : acc) {
-    if (a.node == set.node) continue;
-    Strides st = strides_of(r, a.node, *a.idcs);
-    if (get_stride(st, rc) == 1) unit = true;
-  }
-  (void)w;
+  const bool unit = reduction_walks_unit_stride(r, ph, set);
   auto pow2_floor = [](int64_t x) { int64_t p2 = 1; while (p2 * 2 <= x) p2 *= 2; return p2; };
   if (unit && rext >= 16) ph.coop_lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
   else if (P < 16384 && R >= 256 && rext >= 2) ph.coop_lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
@@ -753,10 +773,26 @@ static AxisIndex subst_index(const AxisIndex& a, int sym, int64_t from, int64_t 
   return o;
 }
 
+static ScalarP subst_scalar(const ScalarP& sp, int sym, int64_t from, int64_t len, int hi, int lo, bool* ok);
+
+// statements of a scope body with `sym` rewritten; a loop that rebinds `sym` cannot be handled
+static Block subst_block(const Block& b, int sym, int64_t from, int64_t len, int hi, int lo, bool* ok) {
+  Block out;
+  for (auto& s : b) {
+    auto o = std::make_shared<Stmt>(*s);
+    if (s->kind == Stmt::For && s->sym == sym) *ok = false;
+    for (auto& ix : o->idcs) ix = subst_index(ix, sym, from, len, hi, lo);
+    o->value = subst_scalar(s->value, sym, from, len, hi, lo, ok);
+    o->body = subst_block(s->body, sym, from, len, hi, lo, ok);
+    out.push_back(o);
+  }
+  return out;
+}
+
 static ScalarP subst_scalar(const ScalarP& sp, int sym, int64_t from, int64_t len, int hi, int lo, bool* ok) {
   if (!sp) return sp;
-  if (sp->kind == Scalar::LocalScope) { *ok = false; return sp; }
   auto o = std::make_shared<Scalar>(*sp);
+  if (sp->kind == Scalar::LocalScope) o->body = subst_block(sp->body, sym, from, len, hi, lo, ok);
   for (auto& ix : o->idcs) ix = subst_index(ix, sym, from, len, hi, lo);
   if (o->kind == Scalar::Index) o->index = subst_index(o->index, sym, from, len, hi, lo);
   o->a = subst_scalar(sp->a, sym, from, len, hi, lo, ok);
@@ -786,12 +822,7 @@ static bool split_reduction(Routine& r, Phase& ph, const PlanOptions& opt, Plan&
   if (P >= 32768 || R < 128 || P * R < (1 << 20)) return false;
   for (auto f : ph.par_from) if (f != 0) return false;
   // lanes sharing the innermost loop already read contiguously: leave those to the lane groups
-  std::vector<Access> acc; bool fl = false; std::set<ScopeId> d;
-  scalar_accesses(*set.value, acc, fl, d);
-  for (auto& a : acc) {
-    if (a.node == set.node) continue;
-    if (get_stride(strides_of(r, a.node, *a.idcs), ph.seq_syms.back()) == 1) return false;
-  }
+  if (reduction_walks_unit_stride(r, ph, set)) return false;
   const int64_t s_target = std::min<int64_t>(std::max<int64_t>((131072 + P - 1) / P, 2), R / 8);
   // whole outer loops first, then a divisor of the next one
   size_t whole = 0;
@@ -2130,6 +2161,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     opt.enable_mfma = opt.enable_coop = opt.enable_row_groups = opt.enable_serial_group = opt.enable_parallel_groups = false;
     opt.enable_bf16_copies = opt.fuse_row_contractions = opt.side_queue = opt.fuse_epilogues = false;
   }
+  if (opt.reuse_stored && !opt.debug_log && r.merge_node < 0) reuse_stored_values(r);
   struct SeqGuard { bool old; SeqGuard(bool v) : old(g_all_sequential) { g_all_sequential = v; } ~SeqGuard() { g_all_sequential = old; } } seq_guard(opt.debug_log);
   Plan plan;
   plan.debug_log = opt.debug_log;
@@ -2202,9 +2234,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     }
     if (sp->kind == Stmt::DeclareLocal || sp->kind == Stmt::SetLocal)
       throw InvalidArgument("hip backend: Set_local of an undeclared scalar at routine scope (routine " + r.name + ")");
-    const size_t before = plan.phases.size();
     devirtualise(r, sp, opt, plan, label);
-    const bool devirt = plan.phases.size() != before;
     if (!analyze_nest(r, sp, ph)) continue;
 
     // fold the preceding Zero_out of the accumulation target into this phase (the accumulation then
@@ -2212,7 +2242,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     // the nest overwrites all of it: every axis is a full-range parallel iterator or has extent 1.
     Binop accum;
     int fill_at = -1;
-    if (!devirt && !opt.debug_log && reduction_shape(r, ph, &accum) && accum == Binop::Add) {
+    if (!opt.debug_log && reduction_shape(r, ph, &accum) && accum == Binop::Add) {
       // the latest Zero_out of the target with nothing touching the target in between
       const int target = ph.inner[0]->node;
       for (int q = (int)plan.phases.size() - 1; q >= 0; --q) {
@@ -2238,7 +2268,7 @@ Plan make_plan(Routine& r, const PlanOptions& requested) {
     }
     // a dead fill: the nest stores to every element of a tensor without reading it, and nothing has
     // touched the tensor since its Zero_out
-    if (!devirt && !opt.debug_log && fill_at < 0 && ph.seq_syms.empty() && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set) {
+    if (!opt.debug_log && fill_at < 0 && ph.seq_syms.empty() && ph.inner.size() == 1 && ph.inner[0]->kind == Stmt::Set) {
       const int target = ph.inner[0]->node;
       std::vector<Access> acc; bool w = false, f = false; std::set<ScopeId> d;
       block_accesses(ph.inner, acc, w, f, d);

@@ -179,6 +179,10 @@ struct PlanOptions {
   int row_tile_waves = 0;            // waves per workgroup of those kernels (4, 8 or 16); 0: 16 for rows of at most 512, else 8
   bool fuse_row_projections = true;   // contraction epilogue of a row group with a prologue (see Phase::proj_y)
   bool fuse_stored_rows = false;     // ... also when its result has to be stored anyway (a context node): measured slower
+  // a sub-expression that recomputes what an earlier statement stored (the reference's optimiser inlines a
+  // tensor into every reader at the assigned position: the backward pass of a relu holds the whole
+  // contraction behind its argument again) reads the stored tensor instead (reuse.cpp)
+  bool reuse_stored = true;
   bool enable_bf16_copies = true;   // keep bf16 copies of fp32 operands of mixed contractions (written by the producing kernels)
 };
 
@@ -196,6 +200,10 @@ struct Plan {
 };
 
 Plan make_plan(Routine& r, const PlanOptions& opt);
+
+// Rewrites, in place, sub-expressions of later statements that recompute a value an earlier statement
+// stored (see reuse.cpp); returns how many it replaced.
+int reuse_stored_values(Routine& r);
 
 // Positions of ph.par_syms ordered by their stride in the first array the phase writes, slowest
 // first: adjacent threads take adjacent values of the last one (coalesced stores).

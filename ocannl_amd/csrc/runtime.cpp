@@ -164,6 +164,7 @@ PlanOptions parse_options(const char* options) {
     else if (k == "row_waves") o.row_tile_waves = std::atoi(v.c_str());
     else if (k == "fused") { o.fuse_row_contractions = v != "0"; o.fuse_stored_rows = v == "2"; }
     else if (k == "parallel") o.enable_parallel_groups = v != "0";
+    else if (k == "reuse") o.reuse_stored = v != "0";
     else if (k == "min_mfma_flops") o.min_mfma_flops = std::stoll(v);
     else throw InvalidArgument("compile options: unknown key '" + k + "'");
   }

@@ -318,3 +318,16 @@ def test_a_row_group_that_rewrites_an_operand_keeps_the_contraction_apart():
     body = apart.source().split('extern "C"', 1)[1]
     assert "ocn_rowtile_contract<" not in body
     assert sum(k["kind"] == "mfma" for k in apart.kernels()) == 1
+
+
+def test_a_recomputed_contraction_reads_the_stored_relu_output_instead():
+    # With the reference's visit rule the sum `product + bias` behind a relu is virtual
+    # (test/einsum/moons_demo_variant.expected:39-44), so the relu's backward statement
+    # `g1 =+ relu_gate(v1, g)` holds the whole product again; the planner reads the stored relu output
+    # there (v1 > 0 exactly when relu(v1) > 0) instead of a 128-long loop per element.
+    import re
+    kw = dict(batch=4, seq=64, d_model=128, heads=2, d_ff=256, layers=1, vocab=256, prec="bfloat16", grad_prec="single")
+    w = W.transformer(inline="visits", **kw)
+    loops = lambda code: len(re.findall(r"for \(uint32_t i\d+ = 0; i\d+ <= 127; \+\+i\d+\) \{\s*v\d+_ffn1", code.source()))
+    assert loops(B.compile(w.routine, "reuse=0")) >= 1
+    assert loops(B.compile(w.routine)) == 0

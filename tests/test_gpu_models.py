@@ -423,3 +423,38 @@ def test_routine_inlined_by_the_visit_rule_against_the_checker():
     for name in ("loss", "w_q_l0", "w_o_l1", "w_ffn1_l0", "w_ffn2_l1", "w_out", "w_embed", "pos_encoding", "gamma_ln1_l0", "beta_ln2_l1", "b_ffn1_l0"):
         assert rel_err(hip.get(w.nodes[name]), ora.get(w.nodes[name]), "single") <= 1e-4, name
     hip.close()
+
+
+@pytest.mark.parametrize("prec,tol", [("single", 1e-4), ("bfloat16", 2e-2)])
+def test_visit_rule_routines_of_the_other_workloads_against_the_checker(prec, tol):
+    # the same inlining rule on the attention and char-MLP routines, and on a bf16 transformer (values of
+    # another precision than the statement they are inlined into, and the relu whose backward statement
+    # holds the feed-forward product again -- which reads the stored relu output instead, reuse.cpp)
+    if prec == "single":
+        w = W.char_mlp(inline="visits")
+        sym = w.statics["batch_n"].sym
+        hip, ora = HipRun(w.routine, w.init), OracleRun(w.routine, w.init)
+        for step in range(5):
+            hip.step({sym: step}); ora.step({sym: step})
+        for name in ("loss", "c", "w1", "b1", "w2", "b2"):
+            assert rel_err(hip.get(w.nodes[name]), ora.get(w.nodes[name]), "single") <= 1e-4, name
+        hip.close()
+    shape = dict(b=2, h=4, q=64, k=96, d=32)
+    w = W.attention(prec=prec, grad_prec="single", inline="visits", **shape)
+    wr = W.attention(prec="single", grad_prec="single", inline="visits", **shape)
+    hip, ora = HipRun(w.routine, w.init, "min_mfma_flops=1"), OracleRun(wr.routine, _widened_init(w, wr))
+    hip.step(); ora.step()
+    for name, p in (("out", prec), ("dq", "single"), ("dk", "single"), ("dv", "single")):
+        assert _err(W.to_float(hip.get(w.nodes[name]), p), ora.get(wr.nodes[name]), prec, elementwise=True) <= tol, name
+    hip.close()
+    kw = dict(batch=2, seq=32, d_model=64, heads=2, d_ff=128, layers=2, vocab=128, grad_prec="single", lr=0.05)
+    w = W.transformer(prec=prec, inline="visits", **kw)
+    wr = W.transformer(prec="single", inline="visits", **kw)
+    for opts in ("min_mfma_flops=100000", "min_mfma_flops=100000;reuse=0"):
+        hip, ora = HipRun(w.routine, w.init, opts), OracleRun(wr.routine, _widened_init(w, wr))
+        for _ in range(2):
+            hip.step(); ora.step()
+        for name in ("loss", "w_q_l0", "w_ffn1_l0", "w_ffn2_l1", "b_ffn1_l1", "w_out", "gamma_ln1_l0"):
+            n = w.nodes[name]
+            assert _err(W.to_float(hip.get(n), n.prec), ora.get(wr.nodes[name]), prec if n.prec == "bfloat16" else "single") <= tol, (opts, name)
+        hip.close()
