@@ -121,6 +121,14 @@ const Scalar* unwrap(const Routine& r, const Scalar& s, Prec* prec) {
   }
 }
 
+// A value computed (and rounded) in precision `from` is the same number after a store to a tensor of
+// precision `to` and the read back: equal precisions, or a wider floating-point type.
+bool stores_exactly(Prec from, Prec to) {
+  auto rank = [](Prec p) { return p == Prec::Double ? 3 : p == Prec::Single ? 2 : (p == Prec::Bfloat16 || p == Prec::Half) ? 1 : 0; };
+  if (rank(from) == 0 || rank(to) == 0) return false;   // integer-like and 8-bit types: not taken
+  return from == to || rank(to) > rank(from);
+}
+
 struct Stored {
   int node;                       // T
   std::vector<int> pos_of_free;   // free symbol q_k of E stands at this position of T's index tuple
@@ -180,6 +188,18 @@ int reuse_stored_values(Routine& r) {
     if (!set) continue;
 
     // ---- use: rewrite sub-expressions that recompute a stored value
+    // (ranges of the loop symbols around the sub-expression being looked at: the stored tensor is only
+    // known over its own extents, whatever the extents of the operands are)
+    std::map<int, std::pair<int64_t, int64_t>> range;
+    for (const Stmt* l : chain) range[l->sym] = {l->from, l->to};
+    auto inside = [&](const Stored& st, const Canon& c) {
+      const Node& t = r.node(st.node);
+      for (size_t k = 0; k < c.free_order.size(); ++k) {
+        auto it = range.find(c.free_order[k]);
+        if (it == range.end() || it->second.first < 0 || it->second.second > t.dims[st.pos_of_free[k]] - 1) return false;
+      }
+      return true;
+    };
     std::function<void(ScalarP&, Prec, bool)> visit = [&](ScalarP& sp, Prec prec, bool gate_arg) {
       Prec eval = prec;
       const Scalar* e = unwrap(r, *sp, &eval);
@@ -194,7 +214,7 @@ int reuse_stored_values(Routine& r) {
           it = through_relu.find(key);
           if (it != through_relu.end() && still_valid(it->second, i)) hit = &it->second;
         }
-        if (hit && hit->pos_of_free.size() == c.free_order.size()) {
+        if (hit && hit->pos_of_free.size() == c.free_order.size() && inside(*hit, c)) {
           auto g = std::make_shared<Scalar>();
           g->kind = Scalar::Get; g->node = hit->node;
           g->idcs.resize(r.node(hit->node).dims.size());
@@ -224,7 +244,7 @@ int reuse_stored_values(Routine& r) {
           const Prec sp_prec = r.node(s.scope.node).prec;
           std::function<void(Block&)> blk = [&](Block& b) {
             for (auto& st : b) {
-              if (st->kind == Stmt::For) blk(st->body);
+              if (st->kind == Stmt::For) { range[st->sym] = {st->from, st->to}; blk(st->body); range.erase(st->sym); }
               else if (st->kind == Stmt::SetLocal && st->value) visit(st->value, sp_prec, false);
             }
           };
@@ -250,12 +270,15 @@ int reuse_stored_values(Routine& r) {
       pos_of_sym[a.sym] = (int)p;
     }
     if (!whole) continue;
-    auto record = [&](const Scalar& value, Prec prec, std::map<std::string, Stored>& table) {
+    // `keeps`: only the sign of the value is asked for later (the relu form), which a store in bf16, with
+    // the exponent range of fp32, keeps as well
+    auto record = [&](const Scalar& value, Prec prec, std::map<std::string, Stored>& table, bool keeps) {
       Prec eval = prec;
       const Scalar* e = unwrap(r, value, &eval);
       Canon c;
       c.scalar(*e);
       if (!c.ok || !c.has_reduction || c.reads.count(set->node)) return;
+      if (!stores_exactly(eval, tn.prec) && !(keeps && eval == Prec::Single && tn.prec == Prec::Bfloat16)) return;
       Stored st;
       st.node = set->node; st.reads = c.reads; st.at = i;
       for (int s : c.free_order) {
@@ -266,8 +289,9 @@ int reuse_stored_values(Routine& r) {
       if (st.pos_of_free.size() != tn.dims.size()) return;   // every axis of T has to be addressed
       table[std::to_string((int)eval) + "|" + c.out.str()] = st;
     };
-    record(*set->value, tn.prec, plain);
-    if (set->value->kind == Scalar::Un && set->value->un == Unop::Relu) record(*set->value->a, tn.prec, through_relu);
+    record(*set->value, tn.prec, plain, false);
+    if (set->value->kind == Scalar::Un && set->value->un == Unop::Relu && stores_exactly(tn.prec, tn.prec))
+      record(*set->value->a, tn.prec, through_relu, true);
   }
   return replaced;
 }

@@ -13,7 +13,7 @@ from ocannl_amd import workloads as W
 
 
 class Gen:
-    def __init__(self, seed: int, precs=("single",)):
+    def __init__(self, seed: int, precs=("single",), recompute: bool = False):
         self.rng = np.random.default_rng(seed)
         self.seed = seed
         L.reset_symbols(0)
@@ -22,6 +22,8 @@ class Gen:
         self.C = int(rng.choice([5, 64, 130, 256, 1024, 2048]))
         if self.R * self.C > 300000:
             self.R = 64
+        if recompute and self.C > 256:     # (inlined reductions are drawn for rows of at most 256)
+            self.C = 130
         self._id = 0
         pick = lambda: str(rng.choice(precs))
         self.mats = [self.node(f"m{k}", pick(), (self.R, self.C)) for k in range(4)]
@@ -42,6 +44,11 @@ class Gen:
         self.tmp.mode = "local"
         self.used_static = False
         self.extended = False
+        # `recompute`: statements that spell out again, symbol for symbol, an inlined reduction that an
+        # earlier statement stored -- what the reference's inlining of a tensor into every reader at
+        # the assigned position leaves in a routine -- with whatever the draw puts in between
+        self.recompute = recompute
+        self.inlined = []      # builders of the stored expressions so far: (node stored to, f(i, j) -> scalar)
         self.nodes = self.mats + self.rows + self.cols + [self.wide, self.tr, self.scal] + ([self.sq] if self.sq else [])
 
     def wide_acc(self, nodes):
@@ -173,6 +180,20 @@ class Gen:
         i, j = L.fresh_symbol(), L.fresh_symbol()
         kind = int(rng.integers(0, 11))
         pick = lambda xs: xs[int(rng.integers(len(xs)))]
+        if self.recompute and self.inlined and rng.random() < 0.35:      # an earlier stored expression again
+            _, build = pick(self.inlined)
+            d = pick(self.mats)
+            form = int(rng.integers(0, 3))
+            if form == 0:
+                value = L.Binop("add", L.Binop("mul", L.Const(0.5), build(i, j)), L.Binop("mul", L.Const(0.25), L.Get(pick(self.mats), (L.It(i), L.It(j)))))
+            elif form == 1:
+                value = L.Binop("relu_gate", L.Binop("sub", build(i, j), L.Const(0.1)), L.Get(pick(self.mats), (L.It(i), L.It(j))))
+            else:                                                        # over part of the rows only
+                hi = max(0, R // 2 - 1)
+                return [L.For(i, 0, hi, [L.For(j, 0, C - 1, [L.Set(d, (L.It(i), L.It(j)), L.Binop("mul", L.Const(0.5), build(i, j)))])])]
+            return self.nest([(i, R), (j, C)], [L.Set(d, (L.It(i), L.It(j)), value)])
+        if self.recompute and C <= 256 and rng.random() < 0.3:
+            kind = 9
         if kind <= 2:                                                    # map over a matrix
             d = pick(self.mats)
             order = [(i, R), (j, C)] if rng.random() < 0.8 else [(j, C), (i, R)]
@@ -211,15 +232,30 @@ class Gen:
                 "fma", L.Get(r, (L.It(i),)), L.Get(c, (L.It(j),)), L.Get(m, (L.It(i), L.It(j)))))])
         if kind == 9 and C <= 256:                                       # inlined scalar reduction
             d, a = pick(self.mats), pick(self.mats)
-            k = L.fresh_symbol()
+            sids = [int(rng.integers(100, 10000))]
+            c = pick(self.cols)
+            if self.recompute and d is a and rng.random() < 0.8:         # (in place, nothing can be read back)
+                d = pick([m for m in self.mats if m is not a])
             t = self.node(f"t{self._id}", "single", (1,))
             t.mode = "virtual"
-            sc = L.Scope(t, int(rng.integers(100, 10000)))
-            scope = L.LocalScope(sc, [L.SetLocal(sc, L.Const(0.0)), L.For(k, 0, C - 1, [L.SetLocal(sc, L.Binop(
-                "add", L.GetLocal(sc), L.Binop("mul", L.Get(a, (L.It(i), L.It(k))), L.Get(pick(self.cols), (L.It(k),)))))])])
-            # (an average of bounded values: applied in place, along a row, it cannot grow)
-            return self.nest([(i, R), (j, C)], [L.Set(d, (L.It(i), L.It(j)), L.Binop("mul", L.Const(0.5), L.Binop(
-                "add", L.Get(a, (L.It(i), L.It(j))), L.Binop("mul", L.Const(1.0 / C), scope))))])
+
+            def build(i, j, a=a, c=c, t=t, sids=sids):
+                k = L.fresh_symbol()
+                sc = L.Scope(t, sids.pop() if sids else int(rng.integers(100, 10000)))
+                scope = L.LocalScope(sc, [L.SetLocal(sc, L.Const(0.0)), L.For(k, 0, C - 1, [L.SetLocal(sc, L.Binop(
+                    "add", L.GetLocal(sc), L.Binop("mul", L.Get(a, (L.It(i), L.It(k))), L.Get(c, (L.It(k),)))))])])
+                # (an average of bounded values: applied in place, along a row, it cannot grow)
+                return L.Binop("mul", L.Const(0.5), L.Binop("add", L.Get(a, (L.It(i), L.It(j))), L.Binop("mul", L.Const(1.0 / C), scope)))
+
+            self.inlined.append((d, build))
+            if self.recompute and rng.random() < 0.3:                    # the value through a relu, as a layer stores it
+                return self.nest([(i, R), (j, C)], [L.Set(d, (L.It(i), L.It(j)), L.Unop("relu", L.Binop("sub", build(i, j), L.Const(0.1))))])
+            first = self.nest([(i, R), (j, C)], [L.Set(d, (L.It(i), L.It(j)), build(i, j))])
+            if self.recompute and rng.random() < 0.4:                    # read again right away, into another matrix
+                i2, j2 = L.fresh_symbol(), L.fresh_symbol()
+                d2 = pick([m for m in self.mats if m is not d and m is not a] or self.mats)
+                first += self.nest([(i2, R), (j2, C)], [L.Set(d2, (L.It(i2), L.It(j2)), L.Binop("sub", build(i2, j2), L.Get(d, (L.It(i2), L.It(j2)))))])
+            return first
         if self.sq is not None:                                          # matrix product m[i, j] = sum_k a[i, k] sq[k, j]
             d, a = self.wide_acc(self.mats)[0], self.mats[1]
             k = L.fresh_symbol()

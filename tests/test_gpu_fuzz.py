@@ -43,6 +43,25 @@ def test_random_single_precision_routines(seed):
         hip.close()
 
 
+@pytest.mark.parametrize("seed", range(5000, 5000 + int(__import__("os").environ.get("FUZZ_SEEDS", 24))))
+def test_random_routines_that_spell_stored_expressions_out_again(seed):
+    # inlined reductions stored by one statement and written out again, symbol for symbol, by later ones
+    # (as a value, behind a relu gate, over part of the rows), with random statements in between that may
+    # or may not write the stored tensor or what the expression reads: the planner reads the stored value
+    # where that is the same number and nowhere else; `reuse=0` is the routine taken literally
+    gen = Gen(seed, precs=("single", "single", "bfloat16") if seed % 3 == 0 else ("single",), recompute=True)
+    r = gen.routine(int(gen.rng.integers(6, 14)))
+    init = gen.init()
+    ora = OracleRun(r, init)
+    ora.step(); ora.step()
+    mixed = seed % 3 == 0
+    for options, tol in (("reuse=0;mfma=0;coop=0", 5e-4), ("mfma=0;coop=0", 5e-4), (None, 2e-2 if mixed else 5e-4)):
+        hip = HipRun(r, init, options)
+        hip.step(); hip.step()
+        _compare(hip, ora, gen, tol, options)
+        hip.close()
+
+
 @pytest.mark.parametrize("seed", range(1000, 1000 + int(__import__("os").environ.get("FUZZ_SEEDS", 24)) // 2))
 def test_random_mixed_precision_routines(seed):
     # bf16 / fp32 / fp64 nodes mixed: every operation is computed in the precision of its destination
