@@ -150,6 +150,28 @@ def test_full_size_transformer_step_properties():
         h.close()
 
 
+def test_full_size_visit_rule_step_agrees_with_the_single_reader_form():
+    # benchmark configuration 4 at its real size in the two routine forms the bench line reports: the one
+    # that inlines single-reader tensors only and the one inlined by the reference's visit rule
+    # (low_level.ml:496-552).  They are the same mathematics with fewer tensors in memory, so losses and
+    # updated parameters agree to the bf16 bar (lr 1 so that the bf16 weights move within three steps);
+    # the visit-rule form must also keep every inlined contraction a read of what is stored (no generated
+    # kernel is left with a loop as long as a contraction's K)
+    a, b = W.transformer(lr=1.0), W.transformer(lr=1.0, inline="visits")
+    ha, hb = HipRun(a.routine, a.init), HipRun(b.routine, b.init)
+    assert abs(len(hb.code.kernels()) - len(ha.code.kernels())) <= 8
+    gen_bytes = lambda h: sum(k["bytes"] for k in h.code.kernels() if k["kind"] != "mfma")
+    assert gen_bytes(hb) < gen_bytes(ha)
+    for step in range(3):
+        ha.step(); hb.step()
+        la, lb = (float(W.to_float(h.get(w.nodes["loss"]), w.nodes["loss"].prec)[0]) for h, w in ((ha, a), (hb, b)))
+        assert abs(la - lb) <= 2e-2 * max(1.0, abs(la)), (step, la, lb)
+    for name in ("w_embed", "w_q_l0", "w_ffn1_l2", "b_ffn1_l1", "w_ffn2_l3", "w_out", "gamma_ln1_l0", "beta_ln2_l3"):
+        na, nb = a.nodes[name], b.nodes[name]
+        assert _err(W.to_float(hb.get(nb), nb.prec), W.to_float(ha.get(na), na.prec).astype(np.float64), nb.prec) <= 2e-2, name
+    ha.close(); hb.close()
+
+
 def test_full_size_transformer_learns_a_token_mapping():
     # benchmark configuration 4 at its real size and precision (bf16 values, fp32 gradients) on targets
     # that can be learnt: the token to predict is a fixed function of the input token, (7 t + 3) mod
