@@ -54,8 +54,10 @@ def test_random_routines_that_spell_stored_expressions_out_again(seed):
     init = gen.init()
     ora = OracleRun(r, init)
     ora.step(); ora.step()
-    mixed = seed % 3 == 0
-    for options, tol in (("reuse=0;mfma=0;coop=0", 5e-4), ("mfma=0;coop=0", 5e-4), (None, 2e-2 if mixed else 5e-4)):
+    # (with bf16 nodes in the draw a stored value minus its recomputation in bf16 is pure rounding noise,
+    # which a last-bit difference in exp or tanh upstream reshuffles: the bf16 bar for every node then)
+    tol = 2e-2 if seed % 3 == 0 else 5e-4
+    for options, tol in (("reuse=0;mfma=0;coop=0", tol), ("mfma=0;coop=0", tol), (None, tol)):
         hip = HipRun(r, init, options)
         hip.step(); hip.step()
         _compare(hip, ora, gen, tol, options)
