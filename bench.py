@@ -118,8 +118,8 @@ def cpu_baseline(name: str):
 def measure(workload: str, steps: int, warmup: int, options=None, kernel_table: bool = False, bracket_inside: bool = True):
     """Runs `steps` timed steps of one workload (after `warmup` untimed ones) and returns the
     measurements: whole-routine rate, the dominant kernel's roofline (its launches bracketed with HIP
-    events on the device stream inside the timed region), contraction TFLOP/s and generated-kernel GB/s
-    on algorithmic work.  `bracket_inside=False` (the launch-bound configurations, where the two event
+    events on the device stream inside the timed region, one launch per step in rotation), contraction
+    TFLOP/s and generated-kernel GB/s on algorithmic work.  `bracket_inside=False` (the launch-bound configurations, where the two event
     records per step are a visible part of a 20 us step): the timed region runs plain, and the
     dominant kernel is bracketed over a second pass of the same number of steps right after it."""
     from ocannl_amd import backend as B
@@ -173,25 +173,33 @@ def measure(workload: str, steps: int, warmup: int, options=None, kernel_table: 
                   f"mnk={k['m']}x{k['n']}x{k['k']}x{k['batch']} coop={k['coop_lanes']}", file=sys.stderr)
 
     # ---- timed region: exactly K steps, device idle on both sides; the dominant kernel's launches
-    #      are bracketed with HIP events on the stream they run on
+    #      are bracketed with HIP events on the stream they run on, ONE launch per step, in rotation (an
+    #      event record costs about 5 us of queue time on this platform: bracketing all eight launches of
+    #      the transformer step's dominant kernel would add 2.6 % to the step being measured)
     hip.rt.profile_kernel(-1)
-    if bracket_inside:
-        for i in dom_idx:
-            hip.rt.profile_kernel(i)
     hip.rt.profile_read()
+    sampled = []
+
+    def bracket_one(i):
+        hip.rt.profile_kernel(-1)
+        hip.rt.profile_kernel(dom_idx[i % len(dom_idx)])
+        sampled.append(dom_idx[i % len(dom_idx)])
+
     B.await_(hip.ctx.dev)
     t0 = time.perf_counter()
     for i in range(steps):
+        if bracket_inside:
+            bracket_one(i)
         step(i)
     B.await_(hip.ctx.dev)
     dt = time.perf_counter() - t0
     if not bracket_inside:
-        for i in dom_idx:
-            hip.rt.profile_kernel(i)
         for i in range(steps):
+            bracket_one(i)
             step(i)
     dom_ms, dom_launches = hip.rt.profile_read()
     hip.rt.profile_kernel(-1)
+    assert dom_launches == len(sampled), (dom_launches, len(sampled))
     loss = None
     if "loss" in w.nodes:
         from ocannl_amd import workloads as W
@@ -199,7 +207,7 @@ def measure(workload: str, steps: int, warmup: int, options=None, kernel_table: 
 
     avg_ms = dom_ms / max(dom_launches, 1)
     if bound == "mfma":
-        per_launch = sum(kernels[i]["flops"] for i in dom_idx) / len(dom_idx)
+        per_launch = sum(kernels[i]["flops"] for i in sampled) / len(sampled)   # (of the launches that were bracketed)
         achieved = per_launch / (avg_ms * 1e-3) / 1e12
         f32 = "gemm_f32" in dom_name
         peak = PEAKS["mfma_f32"] if f32 else PEAKS["mfma_bf16"]
