@@ -4,7 +4,16 @@
     micrograd_demo_logging-sync_cc-0-0.log.expected (forward code + reverse-mode derivatives);
   * the einsum tables of test/einsum/einsum_trivia.ml:378-481 (pointwise, batched matrix product,
     outer batch product, sums over batch axes; operand layout batch @ output @ input);
-  * test/operations/hello_world_op.ml:479-548 (matrix-vector product plus bias).
+  * test/operations/hello_world_op.ml:479-548 (matrix-vector product plus bias);
+  * test/operations/zero2hero_1of7_exec.ml: the polynomial 3x^2 - 4x + 5 with every node's value and
+    gradient at x = 5 and its two sweeps (:22-101, the second through a static index), the
+    four-parameter product-sum with an SGD step between two gradient passes (:103-136), the
+    two-input neuron (:169-178), as zero2hero_1of7_exec.expected prints them;
+  * test/operations/test_where_simple.ml (the `where` ternary and its two gradient statements,
+    tensor/operation.ml:457-467), test_fma_logic.ml (pointwise and compose-accumulate `fma`),
+    rope_test.ml Tests 1 and 2 (de-interleave / interleave through `2*i` and `2*i + 1` affine indices,
+    tensor/operation.ml:342-372, and the rotation of lib/nn_blocks.ml:195-207), written in the loop IR
+    directly.
 The expected numbers are in tests/golden/kat.json exactly as the reference prints them."""
 import json
 import os
@@ -85,6 +94,205 @@ def hello_world(n_out, n_in, hey_value, vec, bias):
     return r, init, {"y": y.value}
 
 
+def zero2hero_poly(sweep=None):
+    """f = 3 x^2 - 4 x + 5 (zero2hero_1of7_exec.ml:26,62): every intermediate a tensor of its own, as
+    `Train.every_non_literal_materialized` leaves them.  `sweep` (a list of values): x is element
+    `step` of a vector -- `x_flat @| step_sym`, the slice by a static symbol of :66-72, whose backward
+    statement adds x's gradient into that element of the vector's gradient."""
+    L.reset_symbols(0)
+    g = Graph("single", "single")
+    one = ("o",)
+    statics = []
+    if sweep is None:
+        x = g.param("x", one, (1,))
+        init_x = {x.value.id: np.array([5.0], np.float32)}
+        extra = {}
+    else:
+        from ocannl_amd.frontend import T
+        flat = g.param("x_flat", ("s", "o"), (len(sweep), 1))
+        step = L.StaticSymbol(L.fresh_symbol(), len(sweep))
+        statics = [step]
+        xv = g.node("x", (1,), mode="ctx"); xg = g.node("x_grad", (1,), mode="ctx")
+        x = T(xv, one, xg, (flat,), label="x")
+        x.fwd = [L.Set(xv, (L.Fixed(0),), L.Get(flat.value, (L.It(step.sym), L.Fixed(0))))]
+        at = (L.It(step.sym), L.Fixed(0))
+        x.bwd = lambda: [L.Set(flat.grad, at, L.Binop("add", L.Get(flat.grad, at), L.Get(xg, (L.Fixed(0),))))]
+        init_x = {flat.value.id: np.asarray(sweep, np.float32).reshape(-1, 1)}
+        extra = {"step": step}
+    pw = g.mul(x, x, one, "pow")
+    t3 = g.mul(ConstT(3.0), pw, one, "three_x2")
+    t4 = g.mul(ConstT(4.0), x, one, "four_x")
+    mi = g.sub(t3, t4, one, "minus")
+    f = g.add(mi, ConstT(5.0), one, "f")
+    body = g.grad_update(f)
+    nodes = {"pow": pw.value, "three_x2": t3.value, "four_x": t4.value, "minus": mi.value, "f": f.value, "x": x.value,
+             "grad_f": f.grad, "grad_minus": mi.grad, "grad_three_x2": t3.grad, "grad_four_x": t4.grad, "grad_pow": pw.grad,
+             "grad_x": x.grad}
+    for n in nodes.values():
+        n.mode = "ctx"
+    r = make_routine(g, "zero2hero_poly", body, statics=statics, outputs=list(nodes.values()))
+    return r, init_x, nodes, extra
+
+
+def zero2hero_simple_gradients():
+    """l = (a * b + c) * f with a gradient routine and a separate SGD routine (learning rate 0.1,
+    zero2hero_1of7_exec.ml:103-136)."""
+    L.reset_symbols(0)
+    g = Graph("single", "single")
+    one = ("o",)
+    a = g.param("a", one, (1,)); b = g.param("b", one, (1,)); c = g.param("c", one, (1,)); f = g.param("f", one, (1,))
+    e = g.mul(a, b, one, "e")
+    d = g.add(e, c, one, "d")
+    l = g.mul(d, f, one, "l")
+    grad_body = g.grad_update(l)
+    lr = g.input("learning_rate", one, (1,))
+    nodes = {"a": a.value, "b": b.value, "c": c.value, "f": f.value, "e": e.value, "d": d.value, "l": l.value,
+             "grad_a": a.grad, "grad_b": b.grad, "grad_c": c.grad, "grad_f": f.grad, "grad_e": e.grad, "grad_d": d.grad,
+             "grad_l": l.grad}
+    for n in nodes.values():
+        n.mode = "ctx"
+    sgd_body = g.sgd_update([a, b, c, f], lr)
+    grad = make_routine(g, "simple_grad", grad_body, outputs=list(nodes.values()))
+    sgd = make_routine(g, "simple_sgd", sgd_body, outputs=[a.value, b.value, c.value, f.value])
+    init = {a.value.id: np.array([2.0], np.float32), b.value.id: np.array([-3.0], np.float32),
+            c.value.id: np.array([10.0], np.float32), f.value.id: np.array([-2.0], np.float32),
+            lr.value.id: np.array([0.1], np.float32)}
+    return grad, sgd, init, nodes
+
+
+def zero2hero_neuron():
+    """v = w . x + b with w = [-3, 1], x = [2, 0], b = 6.7 (zero2hero_1of7_exec.ml:169-178)."""
+    L.reset_symbols(0)
+    g = Graph("single", "single")
+    w = g.param("w", ("o", "i"), (1, 2)); x = g.param("x", ("i",), (2,)); b = g.param("b", ("o",), (1,))
+    m = g.einsum(w, x, ("o",), ident="mul")
+    v = g.add(m, b, ("o",), "v")
+    body = g.grad_update(v)
+    nodes = {"v": v.value, "mul": m.value, "grad_w": w.grad, "grad_x": x.grad, "grad_b": b.grad}
+    for n in nodes.values():
+        n.mode = "ctx"
+    r = make_routine(g, "neuron_2d", body, outputs=list(nodes.values()))
+    init = {w.value.id: np.array([[-3.0, 1.0]], np.float32), x.value.id: np.array([2.0, 0.0], np.float32),
+            b.value.id: np.array([6.7], np.float32)}
+    return r, init, nodes
+
+
+def where_simple(cond_value):
+    """result =:+ where cond x y; x.grad =+ where cond g 0; y.grad =+ where cond 0 g
+    (tensor/operation.ml:462-466) around Train.grad_update."""
+    L.reset_symbols(0)
+    mk = lambda i, name: L.Node(i, name, "single", (1,))
+    cond, x, y, res, xg, yg, rg = (mk(i + 1, n) for i, n in enumerate(("cond", "x", "y", "result", "x_grad", "y_grad", "result_grad")))
+    at = (L.Fixed(0),)
+    G = lambda n: L.Get(n, at)
+    body = [L.ZeroOut(res), L.Set(res, at, L.Binop("add", G(res), L.Ternop("where", G(cond), G(x), G(y)))),
+            L.ZeroOut(xg), L.ZeroOut(yg), L.Set(rg, at, L.Const(1.0)),
+            L.Set(xg, at, L.Binop("add", G(xg), L.Ternop("where", G(cond), G(rg), L.Const(0.0)))),
+            L.Set(yg, at, L.Binop("add", G(yg), L.Ternop("where", G(cond), L.Const(0.0), G(rg))))]
+    init = {1: np.array([cond_value], np.float32), 2: np.array([2.0], np.float32), 3: np.array([3.0], np.float32)}
+    return L.Routine("where_simple", body), init, {"x": x, "y": y, "result": res, "x_grad": xg, "y_grad": yg}
+
+
+def fma_logic():
+    """out[i] = fma(a[i], x[i], b[i]) and out2 =:+ fma(p[o, k], q[k], r[o]) with p 1 x 1 (test_fma_logic.ml:36-57)."""
+    L.reset_symbols(0)
+    a, x, b, out = (L.Node(i + 1, n, "single", (4,)) for i, n in enumerate(("a", "x", "b", "out")))
+    p = L.Node(5, "p", "single", (1, 1)); q = L.Node(6, "q", "single", (1,)); r = L.Node(7, "r", "single", (1,))
+    out2 = L.Node(8, "out2", "single", (1,))
+    i, o, kk = L.fresh_symbol(), L.fresh_symbol(), L.fresh_symbol()
+    body = [L.For(i, 0, 3, [L.Set(out, (L.It(i),), L.Ternop("fma", L.Get(a, (L.It(i),)), L.Get(x, (L.It(i),)), L.Get(b, (L.It(i),))))]),
+            L.ZeroOut(out2),
+            L.For(o, 0, 0, [L.For(kk, 0, 0, [L.Set(out2, (L.It(o),), L.Binop("add", L.Get(out2, (L.It(o),)), L.Ternop(
+                "fma", L.Get(p, (L.It(o), L.It(kk))), L.Get(q, (L.It(kk),)), L.Get(r, (L.It(o),)))))])])]
+    f32 = lambda *v: np.array(v, np.float32)
+    init = {1: f32(1, 2, 3, 4), 2: f32(10, 20, 30, 40), 3: f32(0.5, 0.5, 0.5, 0.5), 5: f32(3).reshape(1, 1), 6: f32(2), 7: f32(10)}
+    return L.Routine("fma_logic", body), init, {"pointwise": out, "compose_accumulate": out2}
+
+
+def rope():
+    """rope_test.ml Test 1 (interleave (deinterleave_even x) (deinterleave_odd x) of 1..6) and Test 2
+    (d_k 4, three positions, x[pos, i] = 4 pos + i + 1, frequencies 10000^(-2k/4)): every `=:+` is a
+    Zero_out and an accumulation, the halves are addressed through affine indices."""
+    L.reset_symbols(0)
+    ids = iter(range(1, 40))
+    N = lambda name, dims: L.Node(next(ids), name, "single", dims)
+    body = []
+
+    def split(src, lead, half):      # deinterleave_even / _odd of the last axis
+        outs = []
+        for off, name in ((0, "even"), (1, "odd")):
+            t = N(f"{src.ident}_{name}", lead + (half,))
+            syms = [L.fresh_symbol() for _ in lead] + [L.fresh_symbol()]
+            lhs = tuple(L.It(s) for s in syms)
+            rhs = tuple(L.It(s) for s in syms[:-1]) + (L.Affine(((2, syms[-1]),), off),)
+            nest = [L.Set(t, lhs, L.Binop("add", L.Get(t, lhs), L.Get(src, rhs)))]
+            for s, d in reversed(list(zip(syms, lead + (half,)))):
+                nest = [L.For(s, 0, d - 1, nest)]
+            body.extend([L.ZeroOut(t)] + nest)
+            outs.append(t)
+        return outs
+
+    def join(even, odd, lead, half, name):
+        t = N(name, lead + (2 * half,))
+        body.append(L.ZeroOut(t))
+        for off, src in ((0, even), (1, odd)):
+            syms = [L.fresh_symbol() for _ in lead] + [L.fresh_symbol()]
+            rhs = tuple(L.It(s) for s in syms)
+            lhs = tuple(L.It(s) for s in syms[:-1]) + (L.Affine(((2, syms[-1]),), off),)
+            nest = [L.Set(t, lhs, L.Binop("add", L.Get(t, lhs), L.Get(src, rhs)))]
+            for s, d in reversed(list(zip(syms, lead + (half,)))):
+                nest = [L.For(s, 0, d - 1, nest)]
+            body.extend(nest)
+        return t
+
+    x6 = N("x_deint", (6,))
+    e6, o6 = split(x6, (), 3)
+    round_trip = join(e6, o6, (), 3, "roundtrip")
+    seq, dk = 3, 4
+    x = N("x", (seq, dk)); freqs = N("rope_freqs", (dk // 2,)); pos = N("pos_idx", (seq,))
+    xe, xo = split(x, (seq,), dk // 2)
+    cos_a, sin_a, oe, oo = (N(n, (seq, dk // 2)) for n in ("cos_a", "sin_a", "out_even", "out_odd"))
+    p, kf = L.fresh_symbol(), L.fresh_symbol()
+    at = (L.It(p), L.It(kf))
+    angle = lambda: L.Binop("mul", L.Get(pos, (L.It(p),)), L.Get(freqs, (L.It(kf),)))
+    G = lambda n: L.Get(n, at)
+    body.append(L.For(p, 0, seq - 1, [L.For(kf, 0, dk // 2 - 1, [
+        L.Set(cos_a, at, L.Unop("cos", angle())), L.Set(sin_a, at, L.Unop("sin", angle())),
+        L.Set(oe, at, L.Binop("sub", L.Binop("mul", G(xe), G(cos_a)), L.Binop("mul", G(xo), G(sin_a)))),
+        L.Set(oo, at, L.Binop("add", L.Binop("mul", G(xe), G(sin_a)), L.Binop("mul", G(xo), G(cos_a))))])]))
+    rotated = join(oe, oo, (seq,), dk // 2, "rotated")
+    init = {x6.id: np.arange(1, 7, dtype=np.float32),
+            x.id: (np.arange(seq * dk, dtype=np.float32) + 1).reshape(seq, dk),
+            freqs.id: np.array([10000.0 ** (-2.0 * k / dk) for k in range(dk // 2)], np.float32),
+            pos.id: np.arange(seq, dtype=np.float32)}
+    return L.Routine("rope_kat", body), init, {"roundtrip": round_trip, "rotated": rotated}
+
+
+def check_small_ops(run_cls, kat):
+    for key, cond in (("true", 1.0), ("false", 0.0)):
+        r, init, nodes = where_simple(cond)
+        run = run_cls(r, init)
+        run.step()
+        for name, want in kat["where_simple"][key].items():
+            assert float(run.get(nodes[name])[0]) == want, (key, name)
+        run.close()
+    r, init, nodes = fma_logic()
+    run = run_cls(r, init)
+    run.step()
+    for name, want in kat["fma_logic"].items():
+        if not name.startswith("_"):
+            assert list(run.get(nodes[name])) == want, name
+    run.close()
+    r, init, nodes = rope()
+    run = run_cls(r, init)
+    run.step()
+    assert list(run.get(nodes["roundtrip"])) == kat["rope"]["roundtrip"]
+    rot = run.get(nodes["rotated"])
+    assert [f"{v:.2f}" for v in rot[0]] == kat["rope"]["position0"]
+    assert [f"{v:.4f}" for v in rot[1]] == kat["rope"]["position1"]
+    run.close()
+
+
 def sig3(x):
     """The reference's table format: three significant digits, cut off rather than rounded (its
     tables print 2198 as 2.19e+3 and 1694 as 1.69e+3)."""
@@ -119,6 +327,126 @@ def check_hello(run_factory, kat):
     assert np.array_equal(y, 95.0 + np.arange(20, dtype=np.float32))
 
 
+def check_zero2hero(run_cls, kat):
+    """`run_cls(routine, init)` gives an object with step(static=None), get(node), and from_host-like
+    `set(node, array)`; the same driver for the checker and the HIP library."""
+    k = kat["zero2hero"]
+    # the polynomial at x = 5: every value and gradient of the printed tree
+    r, init, nodes, _ = zero2hero_poly()
+    run = run_cls(r, init)
+    run.step()
+    for name, want in k["poly_at_5"].items():
+        assert float(run.get(nodes[name])[0]) == want, name
+    # :38-52 sweeps x over -5 .. 4 by assigning it between runs
+    ys = []
+    for v in np.arange(10, dtype=np.float32) - 5.0:
+        run.set(nodes["x"], np.array([v], np.float32))
+        run.step()
+        ys.append(float(run.get(nodes["f"])[0]))
+    w = k["poly_sweep_int"]
+    assert (len(ys), min(ys), max(ys), ys[0]) == (w["count"], w["min"], w["max"], w["first"])
+    run.close()
+    # :60-101 sweeps through a static index over x_flat = i / 10 - 5 and reads f and x's gradient
+    xs = [i / 10.0 - 5.0 for i in range(100)]
+    r, init, nodes, extra = zero2hero_poly(xs)
+    run = run_cls(r, init)
+    ys, dys = [], []
+    for i in range(100):
+        run.step({extra["step"].sym: i})
+        ys.append(float(run.get(nodes["f"])[0])); dys.append(float(run.get(nodes["grad_x"])[0]))
+    w = k["poly_sweep_tenths"]
+    r2 = lambda v: float(f"{v:.2f}")     # print_summary prints %.2f
+    assert (len(ys), r2(min(ys)), r2(max(ys)), r2(ys[0])) == (w["count"], w["ys_min"], w["ys_max"], w["ys_first"])
+    assert (r2(min(dys)), r2(max(dys)), r2(dys[0])) == (w["dys_min"], w["dys_max"], w["dys_first"])
+    run.close()
+    # the product-sum: gradients, an SGD step, gradients again
+    grad, sgd, init, nodes = zero2hero_simple_gradients()
+    run = run_cls([grad, sgd], init)
+    run.step(index=0)
+    for name, want in k["simple_gradients"]["first"].items():
+        assert float(run.get(nodes[name])[0]) == want, name
+    run.step(index=1)
+    for name, want in k["simple_gradients"]["after_sgd"].items():
+        assert abs(float(run.get(nodes[name])[0]) - want) < 1e-6, name
+    run.step(index=0)
+    for name, want in k["simple_gradients"]["second"].items():
+        got = float(run.get(nodes[name])[0])
+        assert float(f"{got:.3g}") == want, (name, got)     # the tree prints three significant digits
+    run.close()
+    # the two-input neuron
+    r, init, nodes = zero2hero_neuron()
+    run = run_cls(r, init)
+    run.step()
+    w = k["neuron_2d"]
+    assert abs(float(run.get(nodes["v"])[0]) - w["v"]) < 1e-6 and float(run.get(nodes["mul"])[0]) == w["mul"]
+    assert list(run.get(nodes["grad_w"]).ravel()) == w["grad_w"] and list(run.get(nodes["grad_x"])) == w["grad_x"]
+    assert float(run.get(nodes["grad_b"])[0]) == w["grad_b"]
+    run.close()
+
+
+class _CheckerSession:
+    """One or several routines over shared host buffers, through the CPU checker."""
+
+    def __init__(self, routines, init):
+        from oracle import cc_oracle
+        from parity import oracle_buffers
+        self.routines = routines if isinstance(routines, list) else [routines]
+        self.lib = cc_oracle.CompiledOracle(self.routines)
+        self.bufs = {}
+        for r in self.routines:
+            for k, v in oracle_buffers(r, init).items():
+                self.bufs.setdefault(k, v)
+
+    def step(self, static=None, index=0):
+        r = self.routines[index]
+        self.lib.run(r.name, {n.id: self.bufs[n.id] for n in r.param_nodes()}, static or {})
+
+    def get(self, node):
+        return self.bufs[node.id]
+
+    def set(self, node, values):
+        self.bufs[node.id][...] = values
+
+    def close(self):
+        pass
+
+
+def _hip_session(options):
+    from ocannl_amd import backend as B
+
+    class Session:
+        """The same through the HIP library: one compiled batch, one context, one linked routine each."""
+
+        def __init__(self, routines, init):
+            self.routines = routines if isinstance(routines, list) else [routines]
+            self.code = B.compile_batch(self.routines, options)
+            self.ctx = B.Context()
+            for r in self.routines:
+                self.ctx.allocate(r.param_nodes())
+                for n in r.param_nodes():
+                    if n.id in init:
+                        self.ctx.set_values(n, init[n.id])
+            self.rts = [self.ctx.link(self.code, i) for i in range(len(self.routines))]
+
+        def step(self, static=None, index=0):
+            for sym, v in (static or {}).items():
+                self.rts[index].set_static(sym, v)
+            self.rts[index].run()
+
+        def get(self, node):
+            return self.ctx.get_values(node)
+
+        def set(self, node, values):
+            self.ctx.set_values(node, values)
+
+        def close(self):
+            B.await_(self.ctx.dev)
+            self.rts = []
+            self.ctx.free()
+
+    return Session
+
+
 def oracle_factory(r, init, nodes):
     o = OracleRun(r, init)
     o.step()
@@ -135,6 +463,14 @@ def test_einsum_tables_checker(kat):
 
 def test_hello_world_checker(kat):
     check_hello(oracle_factory, kat)
+
+
+def test_zero2hero_known_answers_checker(kat):
+    check_zero2hero(_CheckerSession, kat)
+
+
+def test_where_fma_rope_known_answers_checker(kat):
+    check_small_ops(_CheckerSession, kat)
 
 
 def hip_factory(options):
@@ -156,3 +492,5 @@ def test_known_answers_on_the_gpu(kat, options):
     check_micrograd(make(*micrograd()), kat)
     check_einsum(make(*einsum_trivia()), kat)
     check_hello(make, kat)
+    check_zero2hero(_hip_session(options), kat)
+    check_small_ops(_hip_session(options), kat)
