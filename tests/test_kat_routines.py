@@ -13,7 +13,11 @@
     tensor/operation.ml:457-467), test_fma_logic.ml (pointwise and compose-accumulate `fma`),
     rope_test.ml Tests 1 and 2 (de-interleave / interleave through `2*i` and `2*i + 1` affine indices,
     tensor/operation.ml:342-372, and the rotation of lib/nn_blocks.ml:195-207), written in the loop IR
-    directly.
+    directly;
+  * test/einsum/test_padding_reset.ml (one padded input read by a max over 3 x 3 windows, whose margin has
+    to hold -infinity, then by a sum over 3 x 3 windows, whose margin has to hold 0: the margin-only
+    reset loops of low_level.ml:2705-2802 run between the two), test_max_pool2d.ml (stride 2, window 2
+    over 0..15) and test_tropical_kernel.ml (max over the window of input + kernel).
 The expected numbers are in tests/golden/kat.json exactly as the reference prints them."""
 import json
 import os
@@ -293,6 +297,68 @@ def check_small_ops(run_cls, kat):
     run.close()
 
 
+def windows():
+    """The three window routines.  The padded input is uploaded with junk in its margin: only the reset
+    loops make the stated answers come out."""
+    L.reset_symbols(0)
+    f32 = "single"
+    xin = L.Node(1, "input", f32, (6, 6))          # 4 x 4 with a margin of one on every side
+    pooled = L.Node(2, "pooled", f32, (4, 4)); conv = L.Node(3, "conv_out", f32, (4, 4))
+    r = L.Node(4, "r4x4x1", f32, (4, 4, 1)); mp = L.Node(5, "max_pool2d", f32, (2, 2, 1))
+    kern = L.Node(6, "k", f32, (2, 2)); trop = L.Node(7, "tropical", f32, (2, 2, 1))
+    padding = ((1, 1), (1, 1))
+    body = []
+
+    def window_nest(out, out_idx, ext, stmt):
+        nest = [stmt]
+        for sym, e in reversed(ext):
+            nest = [L.For(sym, 0, e - 1, nest)]
+        return nest
+
+    # max over 3 x 3 windows of the padded input, margin = -infinity
+    body += L.loop_over_padding_region(xin.dims, padding, lambda ix: [L.Set(xin, ix, L.Const(float("-inf")))])
+    body += L.loop_over_dims(pooled.dims, lambda ix: [L.Set(pooled, ix, L.Const(float("-inf")))])
+    oh, ow, wh, ww = (L.fresh_symbol() for _ in range(4))
+    at = (L.It(oh), L.It(ow)); win = (L.Affine(((1, oh), (1, wh)), 0), L.Affine(((1, ow), (1, ww)), 0))
+    body += window_nest(pooled, at, [(oh, 4), (ow, 4), (wh, 3), (ww, 3)],
+                        L.Set(pooled, at, L.Binop("max", L.Get(pooled, at), L.Get(xin, win))))
+    # sum over 3 x 3 windows of the SAME input times 1, margin = 0
+    body += L.loop_over_padding_region(xin.dims, padding, lambda ix: [L.Set(xin, ix, L.Const(0.0))])
+    body.append(L.ZeroOut(conv))
+    oh, ow, kh, kw = (L.fresh_symbol() for _ in range(4))
+    at = (L.It(oh), L.It(ow)); win = (L.Affine(((1, oh), (1, kh)), 0), L.Affine(((1, ow), (1, kw)), 0))
+    body += window_nest(conv, at, [(oh, 4), (ow, 4), (kh, 3), (kw, 3)],
+                        L.Set(conv, at, L.Ternop("fma", L.Get(xin, win), L.Const(1.0), L.Get(conv, at))))
+    # max-pool stride 2 window 2, and the tropical kernel: max over the window of input + k
+    for out, with_kernel in ((mp, False), (trop, True)):
+        body += L.loop_over_dims(out.dims, lambda ix: [L.Set(out, ix, L.Const(float("-inf")))])
+        oh, ow, c, wh, ww = (L.fresh_symbol() for _ in range(5))
+        at = (L.It(oh), L.It(ow), L.It(c))
+        src = L.Get(r, (L.Affine(((2, oh), (1, wh)), 0), L.Affine(((2, ow), (1, ww)), 0), L.It(c)))
+        val = L.Binop("add", src, L.Get(kern, (L.It(wh), L.It(ww)))) if with_kernel else src
+        body += window_nest(out, at, [(oh, 2), (ow, 2), (c, 1), (wh, 2), (ww, 2)], L.Set(out, at, L.Binop("max", L.Get(out, at), val)))
+    padded = np.full((6, 6), 777.0, np.float32)
+    padded[1:5, 1:5] = np.arange(16, dtype=np.float32).reshape(4, 4) - 16.0
+    init = {1: padded, 4: np.arange(16, dtype=np.float32).reshape(4, 4, 1), 6: np.arange(4, dtype=np.float32).reshape(2, 2)}
+    return L.Routine("windows_kat", body), init, {"pooled": pooled, "conv": conv, "max_pool": mp, "tropical": trop}
+
+
+def check_windows(run_cls, kat):
+    k = kat["windows"]
+    r, init, nodes = windows()
+    run = run_cls(r, init)
+    for _ in range(2):                      # the reference runs the pair twice: the resets hold across runs
+        run.step()
+        pooled, conv = run.get(nodes["pooled"]), run.get(nodes["conv"])
+        w = k["padding_reset"]
+        assert (float(pooled[0, 0]), float(pooled[1, 1]), float(conv[0, 0]), float(conv[1, 1])) == \
+            (w["pooled_0_0"], w["pooled_1_1"], w["conv_0_0"], w["conv_1_1"])
+        assert np.isfinite(conv).all() and np.isfinite(pooled).all()
+    assert list(run.get(nodes["max_pool"]).ravel()) == k["max_pool_4x4_stride2_window2"]
+    assert list(run.get(nodes["tropical"]).ravel()) == k["tropical_4x4_kernel_0123"]
+    run.close()
+
+
 def sig3(x):
     """The reference's table format: three significant digits, cut off rather than rounded (its
     tables print 2198 as 2.19e+3 and 1694 as 1.69e+3)."""
@@ -473,6 +539,10 @@ def test_where_fma_rope_known_answers_checker(kat):
     check_small_ops(_CheckerSession, kat)
 
 
+def test_window_known_answers_checker(kat):
+    check_windows(_CheckerSession, kat)
+
+
 def hip_factory(options):
     from ocannl_amd.backend import HipRun
 
@@ -494,3 +564,4 @@ def test_known_answers_on_the_gpu(kat, options):
     check_hello(make, kat)
     check_zero2hero(_hip_session(options), kat)
     check_small_ops(_hip_session(options), kat)
+    check_windows(_hip_session(options), kat)
