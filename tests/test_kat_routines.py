@@ -17,7 +17,10 @@
   * test/einsum/test_padding_reset.ml (one padded input read by a max over 3 x 3 windows, whose margin has
     to hold -infinity, then by a sum over 3 x 3 windows, whose margin has to hold 0: the margin-only
     reset loops of low_level.ml:2705-2802 run between the two), test_max_pool2d.ml (stride 2, window 2
-    over 0..15) and test_tropical_kernel.ml (max over the window of input + kernel).
+    over 0..15) and test_tropical_kernel.ml (max over the window of input + kernel);
+  * test/einsum/test_accumulation_semantics.ml: a sum over the output axis, a diagonal (`i => ii`) and a
+    fixed-index projection (`i => i0`) whose untouched cells hold the zeros of the Zero_out in front of
+    them, a transpose.
 The expected numbers are in tests/golden/kat.json exactly as the reference prints them."""
 import json
 import os
@@ -359,6 +362,39 @@ def check_windows(run_cls, kat):
     run.close()
 
 
+def accumulation_semantics():
+    """The four assignments of test_accumulation_semantics.ml:20-101 as `=:+` lowers them: Zero_out,
+    then the accumulating Set over the product space.  Results are uploaded full of junk."""
+    L.reset_symbols(0)
+    f32 = "single"
+    r3 = L.Node(1, "r2x4x3", f32, (2, 4, 3)); red = L.Node(2, "result", f32, (2, 3))
+    v5 = L.Node(3, "v5", f32, (5,)); diag = L.Node(4, "diagonal", f32, (5, 5))
+    v4 = L.Node(5, "v4", f32, (4,)); sparse = L.Node(6, "sparse", f32, (4, 3))
+    m = L.Node(7, "r3x4", f32, (3, 4)); tr = L.Node(8, "transposed", f32, (4, 3))
+    b, i, o, d, p, q, t = (L.fresh_symbol() for _ in range(7))
+    acc = lambda node, lhs, rhs: L.Set(node, lhs, L.Binop("add", L.Get(node, lhs), rhs))
+    body = [L.ZeroOut(red), L.For(b, 0, 1, [L.For(i, 0, 2, [L.For(o, 0, 3, [
+                acc(red, (L.It(b), L.It(i)), L.Get(r3, (L.It(b), L.It(o), L.It(i))))])])]),
+            L.ZeroOut(diag), L.For(d, 0, 4, [acc(diag, (L.It(d), L.It(d)), L.Get(v5, (L.It(d),)))]),
+            L.ZeroOut(sparse), L.For(p, 0, 3, [acc(sparse, (L.It(p), L.Fixed(0)), L.Get(v4, (L.It(p),)))]),
+            L.For(q, 0, 3, [L.For(t, 0, 2, [L.Set(tr, (L.It(q), L.It(t)), L.Get(m, (L.It(t), L.It(q))))])])]
+    junk = lambda n: np.full(n.dims, 55.0, np.float32)
+    init = {1: np.arange(24, dtype=np.float32).reshape(2, 4, 3), 3: np.arange(5, dtype=np.float32),
+            5: np.arange(4, dtype=np.float32), 7: np.arange(12, dtype=np.float32).reshape(3, 4),
+            2: junk(red), 4: junk(diag), 6: junk(sparse), 8: junk(tr)}
+    return L.Routine("accumulation_semantics", body), init, {"reduction": red, "diagonal": diag, "sparse": sparse, "transposed": tr}
+
+
+def check_accumulation(run_cls, kat):
+    r, init, nodes = accumulation_semantics()
+    run = run_cls(r, init)
+    for _ in range(2):
+        run.step()
+        for name, node in nodes.items():
+            assert np.array_equal(run.get(node), np.asarray(kat["accumulation_semantics"][name], np.float32)), name
+    run.close()
+
+
 def sig3(x):
     """The reference's table format: three significant digits, cut off rather than rounded (its
     tables print 2198 as 2.19e+3 and 1694 as 1.69e+3)."""
@@ -543,6 +579,10 @@ def test_window_known_answers_checker(kat):
     check_windows(_CheckerSession, kat)
 
 
+def test_accumulation_semantics_checker(kat):
+    check_accumulation(_CheckerSession, kat)
+
+
 def hip_factory(options):
     from ocannl_amd.backend import HipRun
 
@@ -565,3 +605,4 @@ def test_known_answers_on_the_gpu(kat, options):
     check_zero2hero(_hip_session(options), kat)
     check_small_ops(_hip_session(options), kat)
     check_windows(_hip_session(options), kat)
+    check_accumulation(_hip_session(options), kat)
