@@ -54,19 +54,6 @@ OCN_DEV unsigned short single_to_bfloat16(float f) {
   const uint32_t w = __float_as_uint(f);
   return (unsigned short)((w + 0x7FFFu + ((w >> 16) & 1u)) >> 16);
 }
-// x / y of two bf16 values rounded to bf16, the bits `single_to_bfloat16(x / y)` gives.  With both
-// mantissas of 8 bits (integers a, b in [128, 255]) the exact quotient is never a bf16 rounding tie and
-// lies at least 2^-17 of its size from one: a tie (2m + 1) / 2^k would need a 2^k = b (2m + 1) with
-// 2m + 1 >= 257 dividing a <= 255 times a power of two.  A product with the hardware reciprocal (one
-// unit in the last place of fp32, 2^-23) therefore rounds to the same bf16 as the fp32 division,
-// which costs a dozen operations.  Taken when both operands and the quotient are normal numbers well
-// inside the exponent range (or the dividend is zero); anything else divides as written.
-OCN_DEV unsigned short ocn_bf16_div(unsigned short a, unsigned short b) {
-  const float x = bfloat16_to_single(a), y = bfloat16_to_single(b);
-  const uint32_t ea = (a >> 7) & 0xFFu, eb = (b >> 7) & 0xFFu;
-  if ((ea - 64u < 127u || (a & 0x7FFFu) == 0u) && eb - 64u < 127u) return single_to_bfloat16(x * __builtin_amdgcn_rcpf(y));
-  return single_to_bfloat16(x / y);
-}
 OCN_DEV float fp8_to_single(unsigned char v) {
   if (v == 0) return 0.0f;
   const uint32_t sgn = v >> 7, e = (v >> 2) & 31u, m = v & 3u;

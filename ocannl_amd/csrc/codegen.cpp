@@ -193,8 +193,6 @@ std::string emit_binop(Prec prec, Binop op, const std::string& a, const std::str
            a + ", " + b + ")";
   }
   std::string tf, ff;
-  // (both operands of a bf16 operation are bf16 values: the quotient has a short exact form)
-  if (prec == Prec::Bfloat16 && op == Binop::Div) return "ocn_bf16_div(" + a + ", " + b + ")";
   if (via_float(prec, &tf, &ff)) {
     Syn3 s = binop_syntax(Prec::Single, op);
     return ff + s.p + tf + a + ")" + s.i + " " + tf + b + ")" + s.s + ")";
