@@ -152,3 +152,31 @@ def test_conversions_between_precisions(dst):
     bad = [(o.ident, int((hip.get(o) != ora.get(o)).sum())) for o in outs if not np.array_equal(hip.get(o), ora.get(o))]
     hip.close()
     assert not bad, bad
+
+
+def test_bf16_quotients_bit_for_bit():
+    # bf16 division against the checker for every pair of 8-bit mantissas at several exponents and signs,
+    # and for zeros, infinities, NaN, subnormal operands and exponents near either end of the range
+    m = np.arange(128, 256, dtype=np.float64)
+    a, b = np.meshgrid(m, m, indexing="ij")
+    xs, ys = [], []
+    for ea, eb, sa, sb in ((0, 0, 1, 1), (-9, 3, -1, 1), (5, -4, 1, -1), (-60, 2, 1, 1), (40, -30, -1, -1), (-62, 63, 1, 1), (62, -63, 1, 1),
+                           (-100, 0, 1, 1), (0, -100, 1, 1), (100, 0, 1, 1), (0, 100, 1, 1), (-126, 0, 1, 1), (0, -126, 1, 1)):
+        xs.append(sa * a.ravel() * 2.0 ** (ea - 7)); ys.append(sb * b.ravel() * 2.0 ** (eb - 7))
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -3.0, 2.0 ** -130, -2.0 ** -133, 2.0 ** 127, 2.0 ** -126, 1e-40, 65280.0], np.float64)
+    sx, sy = np.meshgrid(special, special, indexing="ij")
+    xs.append(sx.ravel()); ys.append(sy.ravel())
+    x = W.as_prec(np.concatenate(xs).astype(np.float32), "bfloat16"); y = W.as_prec(np.concatenate(ys).astype(np.float32), "bfloat16")
+    n = x.size
+    L.reset_symbols(0)
+    xn, yn, zn = (L.Node(i + 1, name, "bfloat16", (n,)) for i, name in enumerate(("x", "y", "z")))
+    i = L.fresh_symbol()
+    r = L.Routine("bf16_div", [L.For(i, 0, n - 1, [L.Set(zn, (L.It(i),), L.Binop("div", L.Get(xn, (L.It(i),)), L.Get(yn, (L.It(i),))))])])
+    init = {1: x, 2: y}
+    hip, ora = HipRun(r, init), OracleRun(r, init)
+    hip.step(); ora.step()
+    got, want = hip.get(zn).view(np.uint16), ora.get(zn).view(np.uint16)
+    nan = lambda u: ((u & 0x7F80) == 0x7F80) & ((u & 0x7F) != 0)
+    same = (got == want) | (nan(got) & nan(want))
+    assert same.all(), (int((~same).sum()), x[~same][:4], y[~same][:4], got[~same][:4], want[~same][:4])
+    hip.close()
