@@ -139,7 +139,9 @@ int ocannl_hip_compile(const char* llir, size_t len, ocannl_hip_code** code);
    kernel produces -- attention weights times V -- runs as that kernel's epilogue on the 32 rows the
    workgroup holds in LDS), row_waves=4|8|16 (waves per workgroup of those kernels), row_vec=0|1 (a lane
    takes runs of four neighbouring row positions; off), group_window=<n> (how many phases apart
-   contractions may be and still share a launch), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
+   contractions may be and still share a launch), reuse=0|1 (a later sub-expression that spells out again what
+   an earlier statement stored -- the reference's optimiser inlines a tensor into every reader at the
+   assigned position, low_level.ml:496-552 -- reads the stored tensor instead; on), min_mfma_flops=<n>, large_models=0|1 (64-bit loop
    indices and offsets in generated kernels, the `large_models` setting of c_syntax.ml:111-112; a
    routine with a node of more than 2^31 - 1 elements gets them without asking). */
 int ocannl_hip_compile_opts(const char* llir, size_t len, const char* options, ocannl_hip_code** code);
