@@ -199,7 +199,7 @@ typedef unsigned int ocn_u32x4 __attribute__((ext_vector_type(4)));
 OCN_DEV void ocn_rowtile_put(unsigned short* p, float v) { *p = single_to_bfloat16(v); }
 OCN_DEV void ocn_rowtile_put(float* p, float v) { *p = v; }
 
-template <int T, int K, int NW, typename XT>
+template <int T, int K, int NW, typename XT, int XS = T>   // XS: elements from row to row of xs
 __device__ __forceinline__ void ocn_rowtile_contract(const unsigned short* __restrict__ a, long long a_row,
                                                      const unsigned short* __restrict__ b, long long b_row, XT* xs) {
   static_assert(T % 32 == 0 && K % 16 == 0 && K <= 128, "row tile: T in steps of 32, K in steps of 16 up to 128");
@@ -223,9 +223,9 @@ __device__ __forceinline__ void ocn_rowtile_contract(const unsigned short* __res
     for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk], bf[kk], acc, 0, 0, 0);
-    XT* out = xs + ((lane >> 5) * 4) * T + n0 + (lane & 31);
+    XT* out = xs + ((lane >> 5) * 4) * XS + n0 + (lane & 31);
 #pragma unroll
-    for (int e = 0; e < 16; ++e) ocn_rowtile_put(out + ((e >> 2) * 8 + (e & 3)) * T, acc[e]);
+    for (int e = 0; e < 16; ++e) ocn_rowtile_put(out + ((e >> 2) * 8 + (e & 3)) * XS, acc[e]);
   }
 }
 

@@ -993,7 +993,14 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           body.push_back(line);
         }
         const std::string xt = c_typ(xn.prec);
-        body.push_back(pind + "__shared__ __attribute__((aligned(16))) " + xt + " xs_[" + std::to_string(32 * q.row_len) + "];");
+        // rows of the tile lie 16 bytes more than a row apart where the static LDS budget allows: with a
+        // power-of-two row the 32 rows a matrix-core fragment read touches (one row per lane) would all
+        // start in the same banks
+        const int64_t xbytes = prec_in_bytes(xn.prec);
+        const int64_t ps_bytes = (q.proj_y >= 0 && q.proj_kp > 1) ? (int64_t)q.proj_kp * 32 * q.proj_n * 4 : 0;
+        const int64_t xpad = (32 * (q.row_len + 16 / xbytes) * xbytes + ps_bytes <= 65536) ? 16 / xbytes : 0;
+        const int64_t xld = q.row_len + xpad;
+        body.push_back(pind + "__shared__ __attribute__((aligned(16))) " + xt + " xs_[" + std::to_string(32 * xld) + "];");
         {
           pr.used_nodes.insert(q.fused_a.node); pr.used_nodes.insert(q.fused_b.node);
           std::string ao = std::to_string(q.fused_a.offset) + "ull", bo = std::to_string(q.fused_b.offset) + "ull";
@@ -1003,7 +1010,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
             if (q.fused_b_stride[k]) bo += " + " + tk + " * " + std::to_string(q.fused_b_stride[k]) + "ull";
           }
           body.push_back(pind + "ocn_rowtile_contract<" + std::to_string(q.row_len) + ", " + std::to_string(q.fused_k) + ", " +
-                         std::to_string(NW) + ", " + xt + ">(" +
+                         std::to_string(NW) + ", " + xt + ", " + std::to_string(xld) + ">(" +
                          r.node(q.fused_a.node).ident + " + (" + ao + "), " + std::to_string(q.fused_a_stride[ma]) + "ll, " +
                          r.node(q.fused_b.node).ident + " + (" + bo + "), " + std::to_string(q.fused_b_row) + "ll, xs_);");
         }
@@ -1034,7 +1041,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
         for (size_t k = 0; k < n; ++k)
           body.push_back(rind + "const " + pr.idx_t + " row" + std::to_string(k) + "_ = t" + std::to_string(k) + "_" +
                          (k == (size_t)ma ? " * 32u + wave_ * " + std::to_string(RPW) + "u + rl_;" : ";"));
-        pr.lds_node = q.fused_x; pr.lds_row = "(wave_ * " + std::to_string(RPW) + "u + rl_)"; pr.lds_ld = q.row_len;
+        pr.lds_node = q.fused_x; pr.lds_row = "(wave_ * " + std::to_string(RPW) + "u + rl_)"; pr.lds_ld = xld;
         if (q.fused_x_store) {
           // x is visible outside the kernel: its rows go to memory as well (adjacent lanes adjacent elements)
           pr.used_nodes.insert(q.fused_x);
@@ -1042,7 +1049,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           for (size_t k = 0; k < n; ++k) off = k == 0 ? "(uint64_t)row0_" : "(" + off + ") * " + std::to_string(q.row_outer_ext[k]) + "ull + row" + std::to_string(k) + "_";
           body.push_back(rind + "_Pragma(\"unroll\") for (uint32_t it_ = 0; it_ < " + std::to_string(pr.row_iters) + "; ++it_) " + xn.ident +
                          "[(" + off + ") * " + std::to_string(q.row_len) + "ull + lane_ + it_ * 64u] = xs_[" + pr.lds_row + " * " +
-                         std::to_string(q.row_len) + "u + lane_ + it_ * 64u];");
+                         std::to_string(xld) + "u + lane_ + it_ * 64u];");
         }
         for (size_t mi = 0; mi < q.members.size(); ++mi) {
           const Phase& m = q.members[mi];
@@ -1061,7 +1068,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
         }
         // contraction epilogue: the finished row of y replaces the row of x in LDS, as bf16 (the wave owns
         // both; a row of y takes at most the bytes of a row of x)
-        const int64_t ys = q.row_len * (int64_t)prec_in_bytes(xn.prec) / 2;   // row stride of y in LDS, in bf16 elements
+        const int64_t ys = xld * xbytes / 2;   // row stride of y in LDS, in bf16 elements
         if (q.proj_y >= 0) {
           auto yc = pr.cache_name.find(q.proj_y);
           if (yc == pr.cache_name.end() || yc->second.find("[it_]") == std::string::npos) throw InvalidArgument("planner: row-group epilogue over a tensor the group does not keep");
