@@ -253,11 +253,11 @@ def test_weight_gradients_go_to_the_side_queue_and_fused_prologues_show_up():
     assert all(k["queue"] == 0 for k in B.compile(w.routine).kernels())   # (off unless asked for)
     # Q K^T ahead of the soft-max chain runs inside the row-wise kernel (one launch less per block)
     fused, apart = B.compile(w.routine), B.compile(w.routine, "fused=0")
-    assert "ocn_rowtile_contract<256, 64, 16, unsigned short>" in fused.source().split("extern \"C\"", 1)[1]
+    assert "ocn_rowtile_contract<256, 64, 16, unsigned short, 264>" in fused.source().split("extern \"C\"", 1)[1]
     n = lambda c: sum(k["kind"] == "mfma" for k in c.kernels())
     assert n(B.compile(w.routine, "proj=0")) == n(apart) - 2
     # ... and attention weights times V runs in there as well
-    assert "ocn_rowtile_project<256, 64, 16, 4, 256>" in fused.source().split("extern \"C\"", 1)[1]
+    assert "ocn_rowtile_project<256, 64, 16, 4, 264>" in fused.source().split("extern \"C\"", 1)[1]
     assert n(fused) == n(apart) - 4
 
 
