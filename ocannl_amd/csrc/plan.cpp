@@ -466,8 +466,21 @@ void choose_coop(const Routine& r, Phase& ph, const PlanOptions& opt) {
   int64_t P = 1, R = 1;
   for (auto e : ph.par_ext) P *= e;
   for (size_t i = 0; i < ph.seq_syms.size(); ++i) R *= ph.seq_to[i] - ph.seq_from[i] + 1;
-  const bool unit = reduction_walks_unit_stride(r, ph, set);
   auto pow2_floor = [](int64_t x) { int64_t p2 = 1; while (p2 * 2 <= x) p2 *= 2; return p2; };
+  if (ph.sums_partials) {
+    // One thread per output would walk all the slices alone: a few thousand threads, each waiting on
+    // a long run of loads, and the launch lasts as long as that wait.  Adjacent outputs are adjacent
+    // in every slice, so with eight lanes to an output a wavefront still reads 32 contiguous bytes of
+    // each of eight slices; more lanes would cut the reads below the 32-byte sector, and are taken
+    // only where a lane would otherwise still walk more than 32 slices.
+    if (R >= 16 && rext >= 2) {
+      int64_t lanes = 8;
+      while (lanes < 64 && R / lanes > 32) lanes *= 2;
+      ph.coop_lanes = (int)std::min<int64_t>(lanes, pow2_floor(rext));
+    }
+    return;
+  }
+  const bool unit = reduction_walks_unit_stride(r, ph, set);
   if (unit && rext >= 16) ph.coop_lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
   else if (P < 16384 && R >= 256 && rext >= 2) ph.coop_lanes = (int)std::min<int64_t>(64, pow2_floor(rext));
   if (ph.coop_lanes == 64 && P <= 16 && rext >= 256 && R >= 2048) ph.coop_lanes = 256;
@@ -908,9 +921,16 @@ static bool split_reduction(Routine& r, Phase& ph, const PlanOptions& opt, Plan&
   v2->kind = Scalar::Bin; v2->bin = Binop::Add; v2->a = lhs; v2->b = get_t;
   auto set2 = std::make_shared<Stmt>();
   set2->kind = Stmt::Set; set2->node = set.node; set2->idcs = set.idcs; set2->value = v2;
+  // the slice axes in the order of their extents, the longest innermost: that is the loop lanes share
   StmtP nest2 = set2;
-  if (hi_ext > 1) nest2 = make_for(hi, 0, hi_ext - 1, nest2);
-  for (size_t i = whole; i-- > 0;) nest2 = make_for(ph.seq_syms[i], ph.seq_from[i], ph.seq_to[i], nest2);
+  {
+    struct SliceLoop { int sym; int64_t from, to; };
+    std::vector<SliceLoop> sl;
+    for (size_t i = 0; i < whole; ++i) sl.push_back({ph.seq_syms[i], ph.seq_from[i], ph.seq_to[i]});
+    if (hi_ext > 1) sl.push_back({hi, 0, hi_ext - 1});
+    std::stable_sort(sl.begin(), sl.end(), [](const SliceLoop& x, const SliceLoop& y) { return x.to - x.from < y.to - y.from; });
+    for (size_t i = sl.size(); i-- > 0;) nest2 = make_for(sl[i].sym, sl[i].from, sl[i].to, nest2);
+  }
   for (size_t k = order.size(); k-- > 0;)
     nest2 = make_for(ph.par_syms[order[k]], 0, ph.par_ext[order[k]] - 1, nest2);
 
@@ -923,6 +943,7 @@ static bool split_reduction(Routine& r, Phase& ph, const PlanOptions& opt, Plan&
   p2.label = ph.label;
   p2.stmt = nest2;
   p2.fused_zero_init = ph.fused_zero_init;
+  p2.sums_partials = true;
   Binop a1, a2;
   if (!analyze_nest(r, nest1, p1) || !analyze_nest(r, nest2, p2) || !reduction_shape(r, p1, &a1) ||
       !reduction_shape(r, p2, &a2) || p1.par_syms.size() != order.size() + whole + (hi_ext > 1 ? 1 : 0) ||
@@ -1474,6 +1495,10 @@ void group_independent(const Routine& r, Plan& plan) {
     for (int lv = 0; lv <= top; ++lv) {
       std::vector<size_t> same;
       for (size_t k = i; k < j; ++k) if (level[k - i] == lv) same.push_back(k);
+      // reductions first: few threads that each wait on a run of dependent loads; started at the head of
+      // the grid they wait while the streaming members run, at its tail the launch would wait for them
+      std::stable_sort(same.begin(), same.end(), [&](size_t x, size_t y) {
+        return !plan.phases[x].seq_syms.empty() && plan.phases[y].seq_syms.empty(); });
       for (size_t c = 0; c < same.size(); c += 32) {
         const size_t n = std::min<size_t>(32, same.size() - c);
         if (n == 1) { out.push_back(std::move(plan.phases[same[c]])); continue; }

@@ -79,6 +79,8 @@ struct Phase {
   const Scalar* coop_scope = nullptr;
   Binop coop_accum = Binop::Add;
   bool fused_zero_init = false;  // the preceding Zero_out of the target was folded in (beta = 0)
+  // second half of a split reduction: adds the slices' partial sums, which lie one output tensor apart
+  bool sums_partials = false;
   // Row group (kind Generic, `members` non-empty): consecutive phases that all work row by row
   // over the same rows -- pointwise over (rows x T), reductions of a row of T elements, per-row
   // scalars -- and whose mutual dependencies stay inside a row.  They run as ONE kernel in which a
