@@ -469,13 +469,13 @@ void choose_coop(const Routine& r, Phase& ph, const PlanOptions& opt) {
   auto pow2_floor = [](int64_t x) { int64_t p2 = 1; while (p2 * 2 <= x) p2 *= 2; return p2; };
   if (ph.sums_partials) {
     // One thread per output would walk all the slices alone: a few thousand threads, each waiting on
-    // a long run of loads, and the launch lasts as long as that wait.  Adjacent outputs are adjacent
-    // in every slice, so with eight lanes to an output a wavefront still reads 32 contiguous bytes of
-    // each of eight slices; more lanes would cut the reads below the 32-byte sector, and are taken
-    // only where a lane would otherwise still walk more than 32 slices.
-    if (R >= 16 && rext >= 2) {
+    // a long run of loads, and the launch lasts as long as that wait.  Lanes that share an output take
+    // slices next to one another, so one load of a wavefront stays inside lanes x (one slice) of
+    // memory and adjacent outputs fill the sectors it touches; 8 to 32 lanes, for at most about 16
+    // loads per lane where that is enough.
+    if (R >= 16) {
       int64_t lanes = 8;
-      while (lanes < 64 && R / lanes > 32) lanes *= 2;
+      while (lanes < 32 && R / lanes > 16) lanes *= 2;
       ph.coop_lanes = (int)std::min<int64_t>(lanes, pow2_floor(rext));
     }
     return;
@@ -863,7 +863,9 @@ static bool split_reduction(Routine& r, Phase& ph, const PlanOptions& opt, Plan&
     value = subst_scalar(value, ph.seq_syms[whole], ph.seq_from[whole], lo_ext, hi, lo, &ok);
     if (!ok) return false;
   }
-  // scratch tensor partial[slices.., p..]: output symbols ordered as the output stores them
+  // scratch tensor partial[slice, p..]: output symbols ordered as the output stores them.  The slice
+  // axes (the whole outer loops, then the upper part of the divided one) share ONE axis, as the
+  // digits of a mixed-radix number: the combine below walks it with a single loop.
   std::vector<size_t> order(ph.par_syms.size());
   for (size_t i = 0; i < order.size(); ++i) order[i] = i;
   Strides so = strides_of(r, set.node, set.idcs);
@@ -876,20 +878,26 @@ static bool split_reduction(Routine& r, Phase& ph, const PlanOptions& opt, Plan&
   t.ident = "part" + std::to_string(new_id) + "_" + out.ident;
   t.prec = out.prec == Prec::Double ? Prec::Double : Prec::Single;
   t.mode = Mode::Local;
-  Indices tix;
+  Indices tix, tix2;
   auto iter = [](int sym) { AxisIndex a; a.kind = AxisIndex::Iter; a.sym = sym; return a; };
-  auto shifted = [](int sym, int64_t from) {
+  const int64_t n_slices = S * hi_ext;
+  const int slice = fresh_symbol(r, next_sym);
+  {
     AxisIndex a;
-    if (from == 0) { a.kind = AxisIndex::Iter; a.sym = sym; }
-    else { a.kind = AxisIndex::Affine; a.terms = {{1, sym}}; a.offset = -from; }
-    return a;
-  };
-  for (size_t i = 0; i < whole; ++i) {
-    t.dims.push_back(ph.seq_to[i] - ph.seq_from[i] + 1);
-    tix.push_back(shifted(ph.seq_syms[i], ph.seq_from[i]));
+    a.kind = AxisIndex::Affine;
+    int64_t mult = n_slices;
+    for (size_t i = 0; i < whole; ++i) {
+      mult /= ph.seq_to[i] - ph.seq_from[i] + 1;
+      a.terms.push_back({mult, ph.seq_syms[i]});
+      a.offset -= mult * ph.seq_from[i];
+    }
+    if (hi_ext > 1) a.terms.push_back({1, hi});
+    if (a.terms.size() == 1 && a.terms[0].first == 1 && a.offset == 0) a = iter(a.terms[0].second);
+    t.dims.push_back(n_slices);
+    tix.push_back(a);
+    tix2.push_back(iter(slice));
   }
-  if (hi_ext > 1) { t.dims.push_back(hi_ext); tix.push_back(iter(hi)); }
-  for (size_t k : order) { t.dims.push_back(ph.par_ext[k]); tix.push_back(iter(ph.par_syms[k])); }
+  for (size_t k : order) { t.dims.push_back(ph.par_ext[k]); tix.push_back(iter(ph.par_syms[k])); tix2.push_back(iter(ph.par_syms[k])); }
 
   // the same accumulation with the scratch element in place of the output element
   auto self = std::make_shared<Scalar>();
@@ -912,25 +920,16 @@ static bool split_reduction(Routine& r, Phase& ph, const PlanOptions& opt, Plan&
   for (size_t k = order.size(); k-- > 0;)
     nest1 = make_for(ph.par_syms[order[k]], 0, ph.par_ext[order[k]] - 1, nest1);
 
-  // phase 2: out[p] := out[p] + partial[s.., p..] over the slices
+  // phase 2: out[p] := out[p] + partial[slice, p..] over the slices
   auto get_t = std::make_shared<Scalar>();
-  get_t->kind = Scalar::Get; get_t->node = t.id; get_t->idcs = tix;
+  get_t->kind = Scalar::Get; get_t->node = t.id; get_t->idcs = tix2;
   auto lhs = std::make_shared<Scalar>();
   lhs->kind = Scalar::Get; lhs->node = set.node; lhs->idcs = set.idcs;
   auto v2 = std::make_shared<Scalar>();
   v2->kind = Scalar::Bin; v2->bin = Binop::Add; v2->a = lhs; v2->b = get_t;
   auto set2 = std::make_shared<Stmt>();
   set2->kind = Stmt::Set; set2->node = set.node; set2->idcs = set.idcs; set2->value = v2;
-  // the slice axes in the order of their extents, the longest innermost: that is the loop lanes share
-  StmtP nest2 = set2;
-  {
-    struct SliceLoop { int sym; int64_t from, to; };
-    std::vector<SliceLoop> sl;
-    for (size_t i = 0; i < whole; ++i) sl.push_back({ph.seq_syms[i], ph.seq_from[i], ph.seq_to[i]});
-    if (hi_ext > 1) sl.push_back({hi, 0, hi_ext - 1});
-    std::stable_sort(sl.begin(), sl.end(), [](const SliceLoop& x, const SliceLoop& y) { return x.to - x.from < y.to - y.from; });
-    for (size_t i = sl.size(); i-- > 0;) nest2 = make_for(sl[i].sym, sl[i].from, sl[i].to, nest2);
-  }
+  StmtP nest2 = make_for(slice, 0, n_slices - 1, set2);
   for (size_t k = order.size(); k-- > 0;)
     nest2 = make_for(ph.par_syms[order[k]], 0, ph.par_ext[order[k]] - 1, nest2);
 

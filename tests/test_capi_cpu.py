@@ -109,10 +109,10 @@ def test_planner_rewrites_show_in_the_generated_source():
     r = L.Routine("colsum", [L.For(j, 0, 255, [L.For(i, 0, 4095, [
         L.Set(out, (L.It(j),), L.Binop("add", L.Get(out, (L.It(j),)), L.Get(x, (L.It(i), L.It(j)))))])])])
     assert len(B.compile(r).kernels()) == 2 and len(B.compile(r, "coop=0").kernels()) == 1
-    # the combine walks the 512 slices of an output with 16 lanes (32 slices each, 16 adjacent bytes
-    # of a slice per wavefront and output group), not with one thread
+    # the combine walks the 512 slices of an output with 32 lanes that take slices next to one another
+    # (16 each), not with one thread
     combine = B.compile(r).source().split("colsum_k1(")[1]
-    assert "gtid_ % 16u" in combine and "ocn_xshfl(part_, 8)" in combine
+    assert "gtid_ % 32u" in combine and "ocn_xshfl(part_, 16)" in combine and "+= 32)" in combine
 
 
 def test_padding_region_loops_visit_exactly_the_margin():
