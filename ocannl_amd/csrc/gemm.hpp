@@ -39,9 +39,11 @@ struct GemmArgs {
   void* c2_more[3];
   // Epilogue fusion (bf16 C, no accumulation, no K split): when `bias` is not null the stored value is
   // bf16(bf16(acc) + bias[n]) (bias: bf16, indexed by the column); when `relu_out` is not null, relu of
-  // the stored value also goes to that tensor at the same element offsets.
+  // the stored value also goes to that tensor at the same element offsets; with `relu_c` set the stored
+  // value itself is the relu (C is the only tensor written).
   const void* bias;
   void* relu_out;
+  int relu_c;
 };
 
 // Picks the kernel instance for the operand precisions / layouts and launches it on `stream`.

@@ -235,7 +235,8 @@ __device__ __forceinline__ float bf2f(unsigned b) { return __uint_as_float(b << 
 template <int TN, int OUT, bool ACC, bool CHECK>
 __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, long ld, int lane,
                                                long rows_left, long cols_left, void* origin2 = nullptr,
-                                               const unsigned short* bias = nullptr, unsigned short* relu_out = nullptr) {
+                                               const unsigned short* bias = nullptr, unsigned short* relu_out = nullptr,
+                                               bool relu_c = false) {
   using T = typename std::conditional<OUT == kOutBf16, unsigned short, float>::type;
   T* const base = static_cast<T*>(origin);
   unsigned short* const base2 = static_cast<unsigned short*>(origin2);
@@ -273,6 +274,7 @@ __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, 
         if (OUT == kOutBf16) {
           unsigned b = f2bf(v);
           if (!ACC && bias) b = f2bf(bf2f(b) + bf2f(bias[j * 32 + col]));   // (bias: at the tile row's first column)
+          if (!ACC && relu_c) b = ((b & 0x8000u) || (b & 0x7FFFu) > 0x7F80u) ? 0u : b;
           p[loff] = (unsigned short)b;
           if (!ACC && relu_out) (relu_out + (long)r * ld + j * 32)[loff] = (unsigned short)(((b & 0x8000u) || (b & 0x7FFFu) > 0x7F80u) ? 0u : b);   // fmaxf(0, y): negatives and NaN give +0
         }
@@ -293,7 +295,7 @@ __device__ __forceinline__ void store_tile_row(f32x16 (&acc)[TN], void* origin, 
 template <int TN, int OUT, bool ACC>
 __device__ __forceinline__ void store_tile_row_wide(f32x16 (&acc)[TN], float* stage, void* origin, long ld, int lane,
                                                     void* origin2 = nullptr, const unsigned short* bias = nullptr,
-                                                    unsigned short* relu_out = nullptr) {
+                                                    unsigned short* relu_out = nullptr, bool relu_c = false) {
   constexpr int CW = TN * 32, LS = CW + 4;
   static_assert(TN == 1 || TN == 2 || TN == 4, "tile rows of 1, 2 or 4 tiles");
   if constexpr (TN == 1) asm volatile("" : "+a"(acc[0]));
@@ -331,17 +333,16 @@ __device__ __forceinline__ void store_tile_row_wide(f32x16 (&acc)[TN], float* st
                                                                __uint_as_float(x & 0xFFFF0000u) + __uint_as_float(b & 0xFFFF0000u)); };
         out = u32x4{add2(out.x, bb.x), add2(out.y, bb.y), add2(out.z, bb.z), add2(out.w, bb.w)};
       }
+      // relu on bf16 bits, as fmaxf(0, y) gives it: negatives (and NaN) become +0
+      auto relu2 = [](unsigned x) {
+        const unsigned lo = x & 0xFFFFu, hi = x >> 16;
+        const unsigned rl = ((lo & 0x8000u) || (lo & 0x7FFFu) > 0x7F80u) ? 0u : lo;
+        const unsigned rh = ((hi & 0x8000u) || (hi & 0x7FFFu) > 0x7F80u) ? 0u : hi;
+        return rl | (rh << 16);
+      };
+      if (!ACC && relu_c) out = u32x4{relu2(out.x), relu2(out.y), relu2(out.z), relu2(out.w)};
       *dst = out;
-      if (!ACC && relu_out) {
-        // relu on bf16 bits, as fmaxf(0, y) gives it: negatives (and NaN) become +0
-        auto relu2 = [](unsigned x) {
-          const unsigned lo = x & 0xFFFFu, hi = x >> 16;
-          const unsigned rl = ((lo & 0x8000u) || (lo & 0x7FFFu) > 0x7F80u) ? 0u : lo;
-          const unsigned rh = ((hi & 0x8000u) || (hi & 0x7FFFu) > 0x7F80u) ? 0u : hi;
-          return rl | (rh << 16);
-        };
-        *reinterpret_cast<u32x4*>(relu_out + row_off + goff) = u32x4{relu2(out.x), relu2(out.y), relu2(out.z), relu2(out.w)};
-      }
+      if (!ACC && relu_out) *reinterpret_cast<u32x4*>(relu_out + row_off + goff) = u32x4{relu2(out.x), relu2(out.y), relu2(out.z), relu2(out.w)};
     } else {
       f32x4* const dst = reinterpret_cast<f32x4*>(static_cast<float*>(origin) + row_off + goff);
       if (ACC) v0 += *dst;
@@ -387,6 +388,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, void* c
   const bool epi = bf && !g.accumulate;
   const unsigned short* const bias = epi && g.bias ? static_cast<const unsigned short*>(g.bias) + n : nullptr;
   char* const origin3 = epi && g.relu_out ? static_cast<char*>(g.relu_out) + first * 2 : nullptr;
+  const bool relu_c = epi && g.relu_c;
   static_for<TM>([&](auto ic) OCN_LAMBDA_INLINE {
     constexpr int i = decltype(ic)::value;
     void* o = origin + (long)i * 32 * ld * (bf ? 2 : 4);
@@ -398,8 +400,8 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, void* cbase, void* c
       case 1: store_tile_row<TN, kOutF32, false, true>(acc[i], o, ld, lane, rl, cols_left); break;
       case 2: store_tile_row<TN, kOutF32, true, false>(acc[i], o, ld, lane, rl, cols_left); break;
       case 3: store_tile_row<TN, kOutF32, true, true>(acc[i], o, ld, lane, rl, cols_left); break;
-      case 4: store_tile_row_wide<TN, kOutBf16, false>(acc[i], stage, o, ld, lane, nullptr, bias, reinterpret_cast<unsigned short*>(o3)); break;
-      case 5: store_tile_row<TN, kOutBf16, false, true>(acc[i], o, ld, lane, rl, cols_left, nullptr, bias, reinterpret_cast<unsigned short*>(o3)); break;
+      case 4: store_tile_row_wide<TN, kOutBf16, false>(acc[i], stage, o, ld, lane, nullptr, bias, reinterpret_cast<unsigned short*>(o3), relu_c); break;
+      case 5: store_tile_row<TN, kOutBf16, false, true>(acc[i], o, ld, lane, rl, cols_left, nullptr, bias, reinterpret_cast<unsigned short*>(o3), relu_c); break;
       case 6: store_tile_row_wide<TN, kOutBf16, true>(acc[i], stage, o, ld, lane); break;
       case 7: store_tile_row<TN, kOutBf16, true, true>(acc[i], o, ld, lane, rl, cols_left); break;
       case 8: store_tile_row_wide<TN, kOutF32Copy, false>(acc[i], stage, o, ld, lane, o2); break;

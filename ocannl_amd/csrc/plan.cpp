@@ -2135,7 +2135,9 @@ void fold_epilogues(Routine& r, Plan& plan) {
     const Stmt* ys = identity_set(plan.phases[i + 1], (int64_t)xn.dims.size());
     if (!ys) continue;
     const Node& yn = r.node(ys->node);
-    const Scalar& v = *ys->value;
+    // (the visit rule inlines y as well when z is its only reader: one statement z := relu(x + bias))
+    const bool relu_of_sum = ys->value->kind == Scalar::Un && ys->value->un == Unop::Relu && ys->value->a->kind == Scalar::Bin;
+    const Scalar& v = relu_of_sum ? *ys->value->a : *ys->value;
     if (yn.prec != Prec::Bfloat16 || yn.dims != xn.dims || !(v.kind == Scalar::Bin && v.bin == Binop::Add)) continue;
     const Scalar* xg = nullptr; const Scalar* bg = nullptr;
     for (const Scalar* s : {v.a.get(), v.b.get()}) {
@@ -2146,8 +2148,8 @@ void fold_epilogues(Routine& r, Plan& plan) {
     const Node& bn = r.node(bg->node);
     if (bn.prec != Prec::Bfloat16 || bn.dims.size() != 1 || bn.dims[0] != g.N || bn.mode == Mode::Virtual) continue;
     // an optional relu of y right behind
-    int Z = -1;
-    if (i + 2 < plan.phases.size()) {
+    int Z = relu_of_sum ? ys->node : -1;   // C itself receives the relu
+    if (!relu_of_sum && i + 2 < plan.phases.size()) {
       const Stmt* zs = identity_set(plan.phases[i + 2], (int64_t)xn.dims.size());
       if (zs && zs->node != ys->node) {
         const Node& zn = r.node(zs->node);
@@ -2165,10 +2167,10 @@ void fold_epilogues(Routine& r, Plan& plan) {
     g.c.node = ys->node;
     g.epi_bias = bg->node;
     g.epi_relu = Z;
-    P.bytes += (double)bn.size_in_bytes() + (Z >= 0 ? tensor_bytes : 0.0);
+    P.bytes += (double)bn.size_in_bytes() + (Z >= 0 && !relu_of_sum ? tensor_bytes : 0.0);
     P.label += " + bias" + std::string(Z >= 0 ? " + relu" : "");
     r.nodes.at(X).mode = Mode::Virtual;   // never stored
-    plan.phases.erase(plan.phases.begin() + i + 1, plan.phases.begin() + i + (Z >= 0 ? 3 : 2));
+    plan.phases.erase(plan.phases.begin() + i + 1, plan.phases.begin() + i + (Z >= 0 && !relu_of_sum ? 3 : 2));
   }
 }
 

@@ -55,7 +55,7 @@ struct GemmDesc {
   // inlined scalar would be, adds the bias, rounds again and stores that as C (= y), and stores relu of
   // it to `epi_relu`.  -1: absent.
   int epi_bias = -1;     // vector indexed by n, bf16
-  int epi_relu = -1;     // tensor of C's shape and precision that receives relu(C)
+  int epi_relu = -1;     // tensor of C's shape and precision that receives relu(C); C itself: the stored value is the relu
   double flops() const {
     double f = 2.0 * (double)M * (double)N * (double)K * (double)(1 + group.size()) * (double)(1 + more.size());
     for (int i = 0; i < nbatch; ++i) f *= (double)batch_ext[i];

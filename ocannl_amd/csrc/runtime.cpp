@@ -438,7 +438,8 @@ void enqueue(ocannl_hip_routine& rt, float* kernel_ms, int cap, int v = 0, bool 
       a.c_is_bf16 = g.c.prec == Prec::Bfloat16;
       a.c2 = g.c_copy >= 0 ? rt.node_ptr[v].at(g.c_copy) : nullptr;
       a.bias = g.epi_bias >= 0 ? rt.node_ptr[v].at(g.epi_bias) : nullptr;
-      a.relu_out = g.epi_relu >= 0 ? rt.node_ptr[v].at(g.epi_relu) : nullptr;
+      a.relu_out = g.epi_relu >= 0 && g.epi_relu != g.c.node ? rt.node_ptr[v].at(g.epi_relu) : nullptr;
+      a.relu_c = g.epi_relu >= 0 && g.epi_relu == g.c.node ? 1 : 0;
       a.npairs = 1 + (int)g.more.size();
       for (size_t p = 0; p < g.more.size(); ++p) { a.a_more[p] = base(g.more[p].first); a.b_more[p] = base(g.more[p].second); }
       a.ngroups = 1 + (int)g.group.size();

@@ -382,3 +382,46 @@ def test_bias_and_relu_consumers_folded_into_the_epilogue(shape):
     assert np.array_equal(W.to_float(zf, "bfloat16"), np.maximum(W.to_float(yf, "bfloat16"), 0.0))
     assert np.any(W.to_float(zf, "bfloat16") > 0) and np.any(W.to_float(yf, "bfloat16") < 0)
     folded.close(); apart.close()
+
+
+@pytest.mark.parametrize("shape", [(256, 384, 128), (136, 72, 200), (1024, 2048, 512)])
+def test_relu_of_the_biased_product_in_one_statement_is_folded_too(shape):
+    # the same layer as the reference's visit rule hands it over when z is the only reader of y:
+    # z := relu(the inlined product + bias[o]) in ONE statement (low_level.ml:496-552).  The epilogue then
+    # stores relu of the biased, rounded result as C and nothing else: bit for bit what the statement
+    # computes from the product kept in scratch, and what the two-statement form stores as z.
+    from ocannl_amd.frontend import Graph, make_routine
+    Bn, O, I = shape
+    def build(inline):
+        L.reset_symbols(0)
+        g = Graph("bfloat16", "single")
+        x = g.input("x", ("b", "i"), (Bn, I)); w = g.param("w", ("o", "i"), (O, I)); bias = g.param("bias", ("o",), (O,))
+        y = g.add(g.einsum(w, x, ("b", "o"), ident="wx"), bias, ("b", "o"), ident="y")
+        z = g.unary("relu", y, ident="z")
+        outs = [z.value] if inline else [y.value, z.value]
+        r = make_routine(g, "mlp_layer", g.forward(z), outputs=outs, **({"inline": "visits"} if inline else {}))
+        return r, x, w, bias, y, z
+    r, x, w, bias, y, z = build(True)
+    assert all(n.id != y.value.id or n.mode == "virtual" for n in r.nodes()), "the harness did not inline y: the test would not reach the fold"
+    rng = np.random.default_rng(Bn)
+    init = {x.value.id: W.as_prec(rng.standard_normal((Bn, I)).astype(np.float32), "bfloat16"),
+            w.value.id: W.as_prec((rng.standard_normal((O, I)) / np.sqrt(I)).astype(np.float32), "bfloat16"),
+            bias.value.id: W.as_prec(rng.standard_normal(O).astype(np.float32), "bfloat16")}
+    folded, apart = HipRun(r, init, "min_mfma_flops=1"), HipRun(r, init, "min_mfma_flops=1;epilogues=0;fused=0")
+    kf, ka = folded.code.kernels(), apart.code.kernels()
+    assert [k["kind"] for k in kf] == ["mfma"] and len(ka) > 1, (kf, ka)
+    folded.step(); apart.step()
+    zf = folded.get(z.value)
+    assert np.array_equal(zf, apart.get(z.value))
+    from parity import OracleRun
+    ora = OracleRun(r, init); ora.step()
+    # (the checker adds the products one by one in bf16, the matrix cores in fp32: the bar is the relative
+    # Frobenius error, as for the other bf16 contractions)
+    want, got = W.to_float(ora.get(z.value), "bfloat16").astype(np.float64), W.to_float(zf, "bfloat16").astype(np.float64)
+    assert np.linalg.norm(got - want) <= 2e-2 * np.linalg.norm(want)
+    r2, x2, w2, bias2, y2, z2 = build(False)
+    two = HipRun(r2, {x2.value.id: init[x.value.id], w2.value.id: init[w.value.id], bias2.value.id: init[bias.value.id]}, "min_mfma_flops=1")
+    two.step()
+    assert np.array_equal(zf, two.get(z2.value))
+    assert np.any(W.to_float(zf, "bfloat16") > 0) and np.any(W.to_float(zf, "bfloat16") == 0)
+    folded.close(); apart.close(); two.close()
