@@ -310,6 +310,9 @@ struct Printer {
   int row_iters = 0;                        // > 0: loops over the row position run `it_` = 0..row_iters-1, unrolled
   std::map<int, std::string> cache_name;    // node -> register expression
   std::set<int> cache_defined;              // nodes whose cache holds the current value
+  // nodes whose store the member being printed leaves to a later member of the group that writes the
+  // same elements again (the registers are kept in step all the same)
+  std::set<int> skip_store;
   // `lhs = value;` with the cache kept in step
   const std::map<int, int>* mirrors = nullptr;   // fp32 node -> bf16 copy stored alongside (Plan::mirrors)
   std::string store_line(int node, const std::string& lhs, const std::string& value, const std::string& guard) {
@@ -343,6 +346,7 @@ struct Printer {
              "; " + mirror_lhs + " = single_to_bfloat16(" + t + "); } }";
     }
     cache_defined.insert(node);
+    if (skip_store.count(node)) return it->second + " = " + value + ";";
     std::string line = it->second + " = " + value + "; " + guard + "{ " + lhs + " = " + it->second + ";";
     if (!mirror_lhs.empty()) line += " " + mirror_lhs + " = single_to_bfloat16(" + it->second + ");";
     return line + " }";
@@ -812,6 +816,37 @@ struct Printer {
   }
 };
 
+// In a row group whose rows stay in registers: does a later member store the very elements member
+// `mi` stores (the same tensor through the same row indices)?  Readers in between take the value
+// from the registers, so the earlier store never reaches anyone.
+bool row_store_is_overwritten(const Phase& q, size_t mi) {
+  const Phase& m = q.members[mi];
+  if (m.row_role != Phase::RowPointwise || m.inner.size() != 1 || m.inner[0]->kind != Stmt::Set) return false;
+  const Stmt& st = *m.inner[0];
+  // -3: constant, -1: position in the row, k >= 0: outer axis k of the group, -2: anything else
+  auto role = [](const Phase& ph, const AxisIndex& ix, long long* fixed) -> int {
+    if (ix.kind == AxisIndex::Fixed) { *fixed = ix.fixed; return -3; }
+    if (ix.kind != AxisIndex::Iter) return -2;
+    if (ix.sym == ph.row_sym) return -1;
+    for (size_t k = 0; k < ph.row_outer_syms.size(); ++k) if (ph.row_outer_syms[k] == ix.sym) return (int)k;
+    return -2;
+  };
+  for (size_t mj = mi + 1; mj < q.members.size(); ++mj) {
+    const Phase& o = q.members[mj];
+    if (o.row_role != Phase::RowPointwise || o.inner.size() != 1 || o.inner[0]->kind != Stmt::Set) continue;
+    const Stmt& ot = *o.inner[0];
+    if (ot.node != st.node || ot.idcs.size() != st.idcs.size()) continue;
+    bool same = true;
+    for (size_t p = 0; p < st.idcs.size() && same; ++p) {
+      long long fa = 0, fb = 0;
+      const int ra = role(m, st.idcs[p], &fa), rb = role(o, ot.idcs[p], &fb);
+      same = ra != -2 && ra == rb && fa == fb;
+    }
+    if (same) return true;
+  }
+  return false;
+}
+
 std::string neutral_literal(Binop accum, bool dbl) {
   switch (accum) {
     case Binop::Max: return dbl ? "(-__builtin_huge_val())" : "(-INFINITY)";
@@ -1057,6 +1092,8 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           const std::string mi_ind = rind + "  ";
           for (size_t k = 0; k < m.row_outer_syms.size(); ++k)
             body.push_back(mi_ind + "const " + pr.idx_t + " " + sym_ident(m.row_outer_syms[k]) + " = row" + std::to_string(k) + "_;");
+          pr.skip_store.clear();
+          if (row_store_is_overwritten(q, mi) && pr.cache_name.count(m.inner[0]->node)) pr.skip_store.insert(m.inner[0]->node);
           if (m.row_role == Phase::RowPointwise) {
             body.push_back(pr.row_loop(sym_ident(m.row_sym), 0, q.row_len - 1, QG, mi_ind));
             emit_phase_statements(r, pr, m, 1, false, mi_ind + "  ", body);
@@ -1064,6 +1101,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           } else {
             emit_phase_statements(r, pr, m, QG, true, mi_ind, body);
           }
+          pr.skip_store.clear();
           body.push_back(rind + "}");
         }
         // contraction epilogue: the finished row of y replaces the row of x in LDS, as bf16 (the wave owns
@@ -1143,6 +1181,8 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           const std::string mi_ind = pind + "  ";
           for (size_t k = 0; k < m.row_outer_syms.size(); ++k)
             body.push_back(mi_ind + "const " + pr.idx_t + " " + sym_ident(m.row_outer_syms[k]) + " = row" + std::to_string(k) + "_;");
+          pr.skip_store.clear();
+          if (cached && row_store_is_overwritten(q, mi) && pr.cache_name.count(m.inner[0]->node)) pr.skip_store.insert(m.inner[0]->node);
           if (m.row_role == Phase::RowPointwise) {
             body.push_back(pr.row_loop(sym_ident(m.row_sym), 0, q.row_len - 1, QG, mi_ind));
             emit_phase_statements(r, pr, m, 1, false, mi_ind + "  ", body);
@@ -1150,6 +1190,7 @@ GeneratedModule generate_module(const Routine& r, const Plan& plan) {
           } else {
             emit_phase_statements(r, pr, m, QG, true, mi_ind, body);
           }
+          pr.skip_store.clear();
           body.push_back(pind + "}");
         }
         pr.row_iters = 0; pr.cache_name.clear(); pr.cache_defined.clear();
