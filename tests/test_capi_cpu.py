@@ -102,6 +102,11 @@ def test_planner_rewrites_show_in_the_generated_source():
     plain = B.compile(w.routine, "rows=0;bf16_copies=0")
     assert "row0_" not in plain.source() and len(plain.kernels()) > len(full.kernels())
     assert all(k["name"].startswith(("gemm_bf16_kernel", "gemm_bf16_dtl_kernel")) for k in full.kernels() if k["kind"] == "mfma")
+    # a gradient that several statements of one row group accumulate into is stored once, by the last of
+    # them (the earlier values live in the group's registers); apart, every statement stores it
+    stores = lambda text, name: len(re.findall(name + r"_\d+\[[^\]]*\] = ", text))
+    assert stores(src, "counts_grad") == 1 and stores(plain.source(), "counts_grad") == 2
+    assert stores(src, "centered_ln1_l0_grad") == 1 and stores(plain.source(), "centered_ln1_l0_grad") == 3
     # a column sum over many rows is split into partial sums + a combine
     L.reset_symbols(0)
     x = L.Node(1, "x", "single", (4096, 256)); out = L.Node(2, "out", "single", (256,))
