@@ -83,6 +83,34 @@ def test_split_column_reduction(accumulate):
     hip.close(); seq.close()
 
 
+def test_split_reduction_over_several_loops_one_of_them_not_from_zero():
+    # out[p, q] += sum_{a = 1..6, b < 12, c < 64} x[a, b, c, p, q]: the two outer loops become whole
+    # slices, the third is divided, and all three are the digits of ONE slice axis of the partial
+    # tensor (6 x 12 x 2 = 144 slices, the first loop shifted to start at zero), which the second half
+    # walks with one loop shared by a group of lanes
+    A, Bq, C, P, Q = 7, 12, 64, 8, 64
+    L.reset_symbols(0)
+    x = L.Node(1, "x", "single", (A, Bq, C, P, Q)); out = L.Node(2, "out", "single", (P, Q))
+    p_, q_, a_, b_, c_ = (L.fresh_symbol() for _ in range(5))
+    body = [L.For(p_, 0, P - 1, [L.For(q_, 0, Q - 1, [L.For(a_, 1, A - 1, [L.For(b_, 0, Bq - 1, [L.For(c_, 0, C - 1, [
+        L.Set(out, (L.It(p_), L.It(q_)), L.Binop("add", L.Get(out, (L.It(p_), L.It(q_))),
+                                                 L.Get(x, (L.It(a_), L.It(b_), L.It(c_), L.It(p_), L.It(q_)))))])])])])])]
+    r = L.Routine("sum3", body)
+    rng = np.random.default_rng(11)
+    init = {1: rng.standard_normal((A, Bq, C, P, Q)).astype(np.float32), 2: rng.standard_normal((P, Q)).astype(np.float32)}
+    hip, ora = HipRun(r, init), OracleRun(r, init)
+    src = hip.code.source()
+    m = re.search(r"float \* __restrict__ (part\d+_out)", src)
+    assert m and len(hip.code.kernels()) == 2, "the reduction was not split"
+    assert re.search(re.escape(m.group(1)) + r"\[\(\(24\*i\d+\+2\*i\d+\+i\d+\+-24\) \* 8", src), "slices not on one axis"
+    assert re.search(r"for \(uint32_t i\d+ = 0 \+ lane_; i\d+ <= 143; i\d+ \+= 16\)", src), "second half: sixteen lanes over the slices"
+    hip.step(); ora.step()
+    assert rel_err(hip.get(out), ora.get(out), "single") <= 1e-4
+    want = init[2].astype(np.float64) + init[1][1:].astype(np.float64).sum(axis=(0, 1, 2))
+    assert np.max(np.abs(hip.get(out) - want)) <= 1e-4 * np.max(np.abs(want))
+    hip.close()
+
+
 def test_scalar_reduction_shared_by_lanes():
     # loss = (sum_i -log p[i]) / n written as an inlined scalar reduction inside one statement
     n = 8192
