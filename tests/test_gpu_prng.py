@@ -41,6 +41,24 @@ def test_uniform_vec_single_known_answers():
     hip.close()
 
 
+def test_uniform_vec_of_a_tensor_id_known_answer():
+    # test/operations/test_vec_simple.ml: the key is the tensor's own id (a Constant_bits,
+    # arrayjit/lib/assignments.ml:793-796; 1 in that program), the counter the constant 42; the four
+    # single-precision numbers of test_vec_simple.expected:4-7
+    with open(os.path.join(GOLDEN, "kat.json")) as f:
+        want = json.load(f)["threefry_light_selfid1_key42_single_uniform_vec4"]
+    L.reset_symbols(0)
+    out = L.Node(1, "uniform_floats", "single", (4,))
+    bits = L.Binop("threefry4x32_light", L.ConstBits(1), L.ConstBits(42))
+    r = L.Routine("vec_simple", [L.SetFromVec(out, (L.Fixed(0),), 4, "uint4x32_to_prec_uniform", bits, "uint4x32")])
+    hip, ora = HipRun(r, {}), OracleRun(r, {})
+    hip.step(); ora.step()
+    got = hip.get(out)
+    assert np.array_equal(got.view(np.uint32), ora.get(out).view(np.uint32))
+    assert [float("%.4g" % v) for v in got] == want
+    hip.close()
+
+
 @pytest.mark.parametrize("prec,length", [("half", 8), ("bfloat16", 8), ("double", 2), ("uint32", 4), ("byte", 16)])
 def test_uniform_vec_other_precisions_bit_exact(prec, length):
     r, out = _uniform_vec_routine(64, prec, length)

@@ -84,6 +84,27 @@ def test_threefry_light_single_uniform_kat(lib, kat):
     assert all(0.0 <= g < 1.0 for g in got)
 
 
+def test_threefry_of_a_tensor_id_single_uniform_kat(lib, kat):
+    # test/operations/test_vec_simple.ml: threefry4x32 (embed_self_id ()) 42L, the light variant by
+    # default (arrayjit/lib/utils.ml:40), through the vectorised converter in single precision.  The
+    # id is a Constant_bits (arrayjit/lib/assignments.ml:793-796; the tensor's id in that program is 1),
+    # spread as an int64 like the 42: the four numbers of test_vec_simple.expected:4-7.
+    key, ctr, out = _u4([0] * 4), _u4([0] * 4), _u4([0] * 4)
+    lib.ocn_x_int64_to_uint4x32(1, key)
+    lib.ocn_x_int64_to_uint4x32(42, ctr)
+    lib.ocn_x_threefry_light(key, ctr, out)
+    f4 = (ctypes.c_float * 4)()
+    lib.ocn_x_u4_to_single_vec(out, f4)
+    assert [float("%.4g" % v) for v in f4] == kat["threefry_light_selfid1_key42_single_uniform_vec4"]
+    # a neighbouring id or the 32-bit spreading gives other numbers: the answer pins both
+    lib.ocn_x_int64_to_uint4x32(2, key)
+    lib.ocn_x_threefry_light(key, ctr, out); lib.ocn_x_u4_to_single_vec(out, f4)
+    assert [float("%.4g" % v) for v in f4] != kat["threefry_light_selfid1_key42_single_uniform_vec4"]
+    lib.ocn_x_uint32_to_uint4x32(1, key)
+    lib.ocn_x_threefry_light(key, ctr, out); lib.ocn_x_u4_to_single_vec(out, f4)
+    assert [float("%.4g" % v) for v in f4] != kat["threefry_light_selfid1_key42_single_uniform_vec4"]
+
+
 def test_threefry_light_half_uniform_vec_kat(lib, kat):
     # test/operations/threefry4x32_demo.ml:31-73: 5 counters x 8 half values, tolerance 0.01
     got = []
