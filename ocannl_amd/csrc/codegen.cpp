@@ -569,7 +569,11 @@ struct Printer {
         const Node& n = r.node(s.node);
         note(s.node, s.idcs);
         Pair c = convert_precision(n.prec, prec);
-        std::string dyn = std::string("((") + idx_t + ")(" + scalar(s.arg_prec, *s.a, ind, defs) + "))";
+        // (c_syntax.ml:753-768 prints the index value in its own precision and casts that.  For bf16 and
+        // fp8 that is the storage integer, 16512 for an id of 4.0, and the load leaves the table --
+        // here it would fault the GPU: those two are read as the numbers they stand for.)
+        const Prec ip = s.arg_prec == Prec::Bfloat16 || s.arg_prec == Prec::Fp8 ? Prec::Single : s.arg_prec;
+        std::string dyn = std::string("((") + idx_t + ")(" + scalar(ip, *s.a, ind, defs) + "))";
         return c.first + n.ident + "[" + offset_str(s.idcs, n.dims, s.dyn_axis, dyn) + "]" + c.second;
       }
       case Scalar::Const: {

@@ -180,3 +180,46 @@ def test_bf16_quotients_bit_for_bit():
     same = (got == want) | (nan(got) & nan(want))
     assert same.all(), (int((~same).sum()), x[~same][:4], y[~same][:4], got[~same][:4], want[~same][:4])
     hip.close()
+
+
+@pytest.mark.parametrize("prec", ["single", "bfloat16"])
+def test_embedding_lookup_outside_the_table_gives_zero_rows(prec):
+    # test/operations/test_one_hot_embedding_lookup.expected:8-11: an id outside [0, classes) or a
+    # fractional one gives a zero row, the rows of the other positions of the same batch are right.
+    # The table read is the guarded Get_dynamic of arrayjit/lib/c_syntax.ml:753-768: the load sits in
+    # the taken arm of the conditional only (ids far outside the table would otherwise read far outside
+    # the buffer), also inside a larger fused statement.
+    # bf16 ids: the reference's C casts the STORAGE bits of the id to the index (16512 for 4.0) and
+    # reads outside the table -- undefined there, so that case is held against the lookup's meaning
+    # only and the checker, which restates that C, is not run on it.
+    from ocannl_amd.frontend import Graph, make_routine, gather_rows
+    classes, width = 5, 192
+    L.reset_symbols(0)
+    g = Graph(prec, "single")
+    table = g.param("table", ("v", "e"), (classes, width)); ids = g.input("ids", ("b",), (8,))
+    emb = gather_rows(g, table, ids, "v")
+    act = g.unary("relu", emb, ident="act")
+    r = make_routine(g, "lookup", g.forward(act), outputs=[emb.value, act.value])
+    rng = np.random.default_rng(2)
+    tv = rng.standard_normal((classes, width)).astype(np.float32)
+    iv = np.array([0, 4, 5, -1, 2.5, 3, 3e9, -7e8], dtype=np.float32)
+    init = {table.value.id: W.as_prec(tv, prec), ids.value.id: W.as_prec(iv, prec)}
+    src = HipRun(r, init)
+    if prec == "bfloat16":
+        assert "(uint32_t)(bfloat16_to_single(ids_" in src.code.source()
+    hip = src
+    hip.step()
+    got = W.to_float(hip.get(emb.value), prec)
+    tq = W.to_float(init[table.value.id], prec)
+    idq = W.to_float(init[ids.value.id], prec)
+    for b in range(8):
+        inside = 0 <= idq[b] < classes and idq[b] == np.trunc(idq[b])
+        want = tq[int(idq[b])] if inside else np.zeros(width, np.float32)
+        assert np.array_equal(got[b], want), (b, idq[b])
+    assert [bool((got[b] == 0).all()) for b in range(8)] == [False, False, True, True, True, False, True, True]
+    assert np.array_equal(W.to_float(hip.get(act.value), prec), np.maximum(got, 0.0))
+    if prec == "single":
+        ora = OracleRun(r, init)
+        ora.step()
+        assert np.array_equal(hip.get(emb.value), ora.get(emb.value)) and np.array_equal(hip.get(act.value), ora.get(act.value))
+    hip.close()
