@@ -836,7 +836,28 @@ static bool split_reduction(Routine& r, Phase& ph, const PlanOptions& opt, Plan&
   for (auto f : ph.par_from) if (f != 0) return false;
   // lanes sharing the innermost loop already read contiguously: leave those to the lane groups
   if (reduction_walks_unit_stride(r, ph, set)) return false;
-  const int64_t s_target = std::min<int64_t>(std::max<int64_t>((131072 + P - 1) / P, 2), R / 8);
+  // threads wanted: enough to keep the loads of a streaming sum in flight; twice that where every term
+  // costs a division or a transcendental (the visit rule inlines a layer norm's normalisation into its
+  // gain gradient), whose threads are bound by their own arithmetic and gain from more of them
+  //   measured, the eight gain-gradient launches of the visit-rule transformer step: 14.6 -> 11.6 us each,
+  //   while the streaming sums of the other form do not change and their combine only grows
+  std::function<bool(const Scalar&)> costly = [&](const Scalar& x) -> bool {
+    if (x.kind == Scalar::Bin && (x.bin == Binop::Div || x.bin == Binop::Pow || x.bin == Binop::Mod)) return true;
+    if (x.kind == Scalar::Un && (x.un == Unop::Exp || x.un == Unop::Log || x.un == Unop::Exp2 || x.un == Unop::Log2 || x.un == Unop::Sin ||
+                                 x.un == Unop::Cos || x.un == Unop::Sqrt || x.un == Unop::Recip || x.un == Unop::RecipSqrt || x.un == Unop::Tanh))
+      return true;
+    if (x.kind == Scalar::LocalScope) {
+      bool any = false;
+      std::function<void(const Block&)> walk = [&](const Block& b) {
+        for (auto& st : b) { if (st->value && costly(*st->value)) any = true; walk(st->body); }
+      };
+      walk(x.body);
+      if (any) return true;
+    }
+    return (x.a && costly(*x.a)) || (x.b && costly(*x.b)) || (x.c && costly(*x.c));
+  };
+  const int64_t threads_wanted = costly(*set.value) ? 262144 : 131072;
+  const int64_t s_target = std::min<int64_t>(std::max<int64_t>((threads_wanted + P - 1) / P, 2), R / 8);
   // whole outer loops first, then a divisor of the next one
   size_t whole = 0;
   int64_t S = 1;
